@@ -1,0 +1,124 @@
+// Work-group collectives of one PE: all-reduce, broadcast, alltoall, fcollect,
+// barrier_all / sync_all / team_sync.
+//
+// Calling convention (same as the reference, include/rocshmem/rocshmem_COLL.hpp:33):
+// every thread of exactly one work-group per team member calls with identical
+// arguments; a team serves one collective at a time.
+#ifndef ROCSHMEM_AMD_DETAIL_COLLECTIVES_HPP_
+#define ROCSHMEM_AMD_DETAIL_COLLECTIVES_HPP_
+
+#include "copy_engine.hpp"
+#include "reduce_engine.hpp"
+#include "state.hpp"
+#include "sync.hpp"
+
+namespace rocshmem {
+namespace detail {
+
+#if defined(__HIPCC__)
+
+__device__ __forceinline__ void team_pad_sync(const Context *c, Team *t, int kind) {
+  sync_pes(c, &t->sync[kind], t->wrt_world.pe_start, t->wrt_world.stride,
+           t->num_pes, t->my_pe);
+}
+
+// src/ipc/context_ipc_device_coll.cpp:101-123
+__device__ __forceinline__ void sync_all(Context *c) {
+  sync_pes(c, c->world_sync, 0, 1, c->num_pes, c->my_pe);
+}
+__device__ __forceinline__ void barrier_all(Context *c) {
+  // quiet() of the calling PE is the release half of the barrier's first step.
+  sync_all(c);
+}
+
+// All-reduce over the team.  Replaces the reference's direct / ring selector
+// and its two algorithms (src/ipc/context_ipc_tmpl_device.hpp:166-418) by a
+// direct reduce-scatter + all-gather in one pass: after every member has
+// arrived, member k folds the k-th chunk of all P sources in ascending member
+// order and stores the result into the k-th chunk of all P destinations; a
+// second barrier ends the operation.  Each element is computed once, so all
+// members hold bit-identical results.  Keeps the reference's refusal of teams
+// with 2*P > ROCSHMEM_REDUCE_SYNC_SIZE (:412-415).
+template <typename E, ROCSHMEM_OP Op>
+__device__ __forceinline__ int wg_reduce(Context *c, Team *t,
+                                         typename ElemTraits<E>::storage *dest,
+                                         const typename ElemTraits<E>::storage *source,
+                                         int nreduce) {
+  using S = typename ElemTraits<E>::storage;
+  const int P = t->num_pes;
+  if (static_cast<size_t>(2 * P) > ROCSHMEM_REDUCE_SYNC_SIZE) return ROCSHMEM_ERROR;
+
+  team_pad_sync(c, t, SYNC_REDUCE);
+
+  const size_t n = static_cast<size_t>(nreduce);
+  constexpr size_t per = 16 / sizeof(S);
+  size_t chunk = (n + P - 1) / P;
+  chunk = (chunk + per - 1) / per * per;
+  size_t lo = static_cast<size_t>(t->my_pe) * chunk;
+  if (lo > n) lo = n;
+  size_t hi = lo + chunk;
+  if (hi > n) hi = n;
+
+  const int64_t to_first = static_cast<int64_t>(t->wrt_world.pe_start - c->my_pe) *
+                           static_cast<int64_t>(c->pe_stride);
+  const int64_t hop = static_cast<int64_t>(t->wrt_world.stride) *
+                      static_cast<int64_t>(c->pe_stride);
+  S *dst0 = reinterpret_cast<S *>(reinterpret_cast<char *>(dest) + to_first);
+  const S *src0 = reinterpret_cast<const S *>(reinterpret_cast<const char *>(source) + to_first);
+  if (hi > lo)
+    fold_span_any<E, Op, false>(dst0, src0, hop, P, lo, hi, flat_thread_id(), flat_block_size());
+
+  team_pad_sync(c, t, SYNC_REDUCE);
+  return ROCSHMEM_SUCCESS;
+}
+
+// dest on every member except the root becomes the root's source; the root's
+// dest is left alone (src/ipc/context_ipc_tmpl_device.hpp:420-472).  Members
+// pull after an entry barrier, so P-1 work-groups copy in parallel and the
+// root's source is known to be final; the exit barrier tells the root when
+// its source may change.
+__device__ __forceinline__ void wg_broadcast(Context *c, Team *t, void *dest,
+                                             const void *source, size_t bytes,
+                                             int pe_root) {
+  team_pad_sync(c, t, SYNC_BCAST);
+  if (t->my_pe != pe_root) {
+    const int root_world = t->wrt_world.pe_start + t->wrt_world.stride * pe_root;
+    copy_lanes(dest, remote_addr(c, static_cast<const char *>(source), root_world),
+               bytes, flat_thread_id(), flat_block_size(), g_state.nt_bytes);
+  }
+  team_pad_sync(c, t, SYNC_BCAST);
+}
+
+// dst_j[me*n + k] = src_me[j*n + k] for every member j, self included
+// (src/ipc/context_ipc_tmpl_device.hpp:480-501).
+__device__ __forceinline__ void wg_alltoall(Context *c, Team *t, void *dest,
+                                            const void *source, size_t block_bytes) {
+  char *d = static_cast<char *>(dest) + static_cast<size_t>(t->my_pe) * block_bytes;
+  const char *s = static_cast<const char *>(source);
+  const unsigned tid = flat_thread_id(), bs = flat_block_size();
+  for (int j = 0; j < t->num_pes; ++j) {
+    const int pe = t->wrt_world.pe_start + t->wrt_world.stride * j;
+    copy_lanes(remote_addr(c, d, pe), s + static_cast<size_t>(j) * block_bytes,
+               block_bytes, tid, bs, g_state.nt_bytes);
+  }
+  team_pad_sync(c, t, SYNC_ALLTOALL);
+}
+
+// dst_j[me*n + k] = src_me[k] (src/ipc/context_ipc_tmpl_device.hpp:509-531).
+__device__ __forceinline__ void wg_fcollect(Context *c, Team *t, void *dest,
+                                            const void *source, size_t block_bytes) {
+  char *d = static_cast<char *>(dest) + static_cast<size_t>(t->my_pe) * block_bytes;
+  const unsigned tid = flat_thread_id(), bs = flat_block_size();
+  for (int j = 0; j < t->num_pes; ++j) {
+    const int pe = t->wrt_world.pe_start + t->wrt_world.stride * j;
+    copy_lanes(remote_addr(c, d, pe), source, block_bytes, tid, bs, g_state.nt_bytes);
+  }
+  team_pad_sync(c, t, SYNC_ALLTOALL);
+}
+
+#endif  // __HIPCC__
+
+}  // namespace detail
+}  // namespace rocshmem
+
+#endif  // ROCSHMEM_AMD_DETAIL_COLLECTIVES_HPP_

@@ -1,0 +1,152 @@
+// Byte-copy engine behind putmem/getmem at thread, wavefront, work-group and
+// grid granularity.
+//
+// Replaces the reference's memcpy / memcpy_wg / memcpy_wave
+// (src/util.hpp:170-262), which move 8 bytes per lane per iteration through
+// cache-bypassing flat stores and make three strided passes (8/4/2 bytes) plus
+// a one-byte tail.  Here a cooperating group of lanes peels the destination to
+// 16-byte alignment, streams 16 bytes per lane per step with several loads in
+// flight (the source may sit at any byte offset — gfx950 global loads need no
+// alignment), and finishes the sub-16-byte tail with byte moves.  Bulk copies
+// use non-temporal stores so a message larger than L2 does not evict what the
+// caller still needs.
+//
+// The result is a byte-exact copy of [src, src+n) to [dst, dst+n) for every n
+// and every pair of alignments.  The reference's work-group and wavefront
+// loops leave the last byte of an odd-sized message (n >= 3) uncopied because
+// the tail move reuses a stale pointer (src/util.hpp:203-223); that defect is
+// not reproduced.
+#ifndef ROCSHMEM_AMD_DETAIL_COPY_ENGINE_HPP_
+#define ROCSHMEM_AMD_DETAIL_COPY_ENGINE_HPP_
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+
+namespace rocshmem {
+namespace detail {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef u32x4 u32x4_any __attribute__((aligned(1)));
+typedef uint64_t u64_any __attribute__((aligned(1)));
+typedef uint32_t u32_any __attribute__((aligned(1)));
+typedef uint16_t u16_any __attribute__((aligned(1)));
+
+// Messages at least this large are stored with the non-temporal hint.
+constexpr size_t kNonTemporalBytes = size_t{1} << 20;
+
+template <bool kNonTemporal>
+__device__ __forceinline__ void store16(char *p, u32x4 v) {
+  if constexpr (kNonTemporal) {
+    __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(p));
+  } else {
+    *reinterpret_cast<u32x4 *>(p) = v;
+  }
+}
+
+template <bool kNonTemporal>
+__device__ __forceinline__ u32x4 load16(const char *p) {
+  if constexpr (kNonTemporal) {
+    return __builtin_nontemporal_load(reinterpret_cast<const u32x4_any *>(p));
+  } else {
+    return *reinterpret_cast<const u32x4_any *>(p);
+  }
+}
+
+// Copy n bytes with `nlanes` cooperating lanes; this lane is number `lane`
+// (0-based, dense).  Lanes need not belong to one wavefront or work-group:
+// a whole grid can call this with global thread ids.
+template <int kUnroll, bool kNonTemporal>
+__device__ __forceinline__ void copy_lanes_impl(char *dst, const char *src,
+                                                size_t n, size_t lane,
+                                                size_t nlanes) {
+  size_t head = (16u - (reinterpret_cast<uintptr_t>(dst) & 15u)) & 15u;
+  if (head > n) head = n;
+  for (size_t k = lane; k < head; k += nlanes) dst[k] = src[k];
+  dst += head;
+  src += head;
+  n -= head;
+
+  const size_t nvec = n >> 4;
+  size_t i = lane;
+  if constexpr (kUnroll > 1) {
+    const size_t span = static_cast<size_t>(kUnroll) * nlanes;
+    for (; i + span - nlanes < nvec; i += span) {
+      u32x4 v[kUnroll];
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u)
+        v[u] = load16<kNonTemporal>(src + ((i + u * nlanes) << 4));
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u)
+        store16<kNonTemporal>(dst + ((i + u * nlanes) << 4), v[u]);
+    }
+  }
+  for (; i < nvec; i += nlanes)
+    store16<kNonTemporal>(dst + (i << 4), load16<kNonTemporal>(src + (i << 4)));
+
+  const size_t done = nvec << 4;
+  const size_t tail = n - done;
+  for (size_t k = lane; k < tail; k += nlanes) dst[done + k] = src[done + k];
+}
+
+__device__ __forceinline__ void copy_lanes(void *dst, const void *src, size_t n,
+                                           size_t lane, size_t nlanes,
+                                           size_t nt_bytes = kNonTemporalBytes) {
+  char *d = static_cast<char *>(dst);
+  const char *s = static_cast<const char *>(src);
+  if (n >= nt_bytes) {
+    copy_lanes_impl<4, true>(d, s, n, lane, nlanes);
+  } else {
+    copy_lanes_impl<4, false>(d, s, n, lane, nlanes);
+  }
+}
+
+// One lane copies n bytes on its own: 16-byte moves, then 8/4/2/1.
+__device__ __forceinline__ void copy_thread(void *dst, const void *src,
+                                            size_t n) {
+  char *d = static_cast<char *>(dst);
+  const char *s = static_cast<const char *>(src);
+  while (n >= 16) {
+    *reinterpret_cast<u32x4_any *>(d) = *reinterpret_cast<const u32x4_any *>(s);
+    d += 16; s += 16; n -= 16;
+  }
+  if (n & 8) {
+    *reinterpret_cast<u64_any *>(d) = *reinterpret_cast<const u64_any *>(s);
+    d += 8; s += 8;
+  }
+  if (n & 4) {
+    *reinterpret_cast<u32_any *>(d) = *reinterpret_cast<const u32_any *>(s);
+    d += 4; s += 4;
+  }
+  if (n & 2) {
+    *reinterpret_cast<u16_any *>(d) = *reinterpret_cast<const u16_any *>(s);
+    d += 2; s += 2;
+  }
+  if (n & 1) *d = *s;
+}
+
+// Rank of this lane among the currently active lanes of its wavefront, and
+// the number of active lanes.  The reference strides by the active-lane count
+// but indexes by the raw lane id (src/util.hpp:226-262), which skips data when
+// the active lanes are not the lowest ones; ranking the active lanes is
+// correct for any mask.
+__device__ __forceinline__ unsigned active_lane_rank(unsigned *count) {
+  const unsigned long long mask = __ballot(1);
+  const unsigned lo = static_cast<unsigned>(mask);
+  const unsigned hi = static_cast<unsigned>(mask >> 32);
+  *count = __popcll(mask);
+  return __builtin_amdgcn_mbcnt_hi(hi, __builtin_amdgcn_mbcnt_lo(lo, 0u));
+}
+
+__device__ __forceinline__ void copy_wave(void *dst, const void *src, size_t n,
+                                          size_t nt_bytes = kNonTemporalBytes) {
+  unsigned count;
+  const unsigned rank = active_lane_rank(&count);
+  copy_lanes(dst, src, n, rank, count, nt_bytes);
+}
+
+}  // namespace detail
+}  // namespace rocshmem
+
+#endif  // ROCSHMEM_AMD_DETAIL_COPY_ENGINE_HPP_

@@ -1,0 +1,222 @@
+// Element-wise combine behind the all-reduce ("to_all" / wg_reduce) path.
+//
+// The reference combines with OpWrap<Op>::Calc, dst[i] = dst[i] op src[i]
+// (src/rocshmem_calc.hpp:43-97), applied chunk by chunk as data travels round
+// a ring through a 1024-element work buffer
+// (src/ipc/context_ipc_tmpl_device.hpp:282-359).  Here every output element is
+// produced in one pass: the P source values are loaded (16 bytes per lane per
+// source, all P loads in flight), folded in registers in ASCENDING team-PE
+// order  (((x0 op x1) op x2) ...), and the result is stored to all P
+// destinations.  For integers, bitwise ops and min/max this equals the
+// reference for any order; for floating-point sums it differs from the
+// reference's cyclic order by rounding only.
+//
+// bf16 (no counterpart in the reference): operands are widened to fp32
+// exactly, folded in fp32, and rounded to nearest-even once at the end.
+#ifndef ROCSHMEM_AMD_DETAIL_REDUCE_ENGINE_HPP_
+#define ROCSHMEM_AMD_DETAIL_REDUCE_ENGINE_HPP_
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+#include <type_traits>
+
+#include "../rocshmem_common.hpp"
+
+namespace rocshmem {
+
+// Storage type of a bfloat16 element (1 sign, 8 exponent, 7 mantissa bits).
+struct rocshmem_bf16 {
+  uint16_t bits;
+};
+
+namespace detail {
+
+__host__ __device__ inline float bf16_to_f32(uint16_t b) {
+  union { uint32_t u; float f; } c;
+  c.u = static_cast<uint32_t>(b) << 16;
+  return c.f;
+}
+
+// Round-to-nearest-even; NaNs keep their sign and become quiet.
+__host__ __device__ inline uint16_t f32_to_bf16(float f) {
+  union { uint32_t u; float f; } c;
+  c.f = f;
+  uint32_t u = c.u;
+  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<uint16_t>((u >> 16) | 0x0040u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return static_cast<uint16_t>(u >> 16);
+}
+
+// acc op x for one element.  Integer sums and products wrap (computed in the
+// unsigned type), as the reference's += / *= do on the device.
+template <typename T, ROCSHMEM_OP Op>
+__host__ __device__ inline T combine(T acc, T x) {
+  if constexpr (Op == ROCSHMEM_SUM) {
+    if constexpr (std::is_integral<T>::value) {
+      using U = typename std::make_unsigned<T>::type;
+      return static_cast<T>(static_cast<U>(static_cast<U>(acc) + static_cast<U>(x)));
+    } else {
+      return acc + x;
+    }
+  } else if constexpr (Op == ROCSHMEM_PROD) {
+    if constexpr (std::is_integral<T>::value) {
+      using U = typename std::make_unsigned<T>::type;
+      return static_cast<T>(static_cast<U>(static_cast<U>(acc) * static_cast<U>(x)));
+    } else {
+      return acc * x;
+    }
+  } else if constexpr (Op == ROCSHMEM_MAX) {
+    if constexpr (std::is_same<T, float>::value) return fmaxf(acc, x);
+    else if constexpr (std::is_same<T, double>::value) return fmax(acc, x);
+    else return acc < x ? x : acc;
+  } else if constexpr (Op == ROCSHMEM_MIN) {
+    if constexpr (std::is_same<T, float>::value) return fminf(acc, x);
+    else if constexpr (std::is_same<T, double>::value) return fmin(acc, x);
+    else return x < acc ? x : acc;
+  } else if constexpr (Op == ROCSHMEM_AND) {
+    return static_cast<T>(acc & x);
+  } else if constexpr (Op == ROCSHMEM_OR) {
+    return static_cast<T>(acc | x);
+  } else {
+    static_assert(Op == ROCSHMEM_XOR, "unsupported reduction op");
+    return static_cast<T>(acc ^ x);
+  }
+}
+
+#if defined(__HIPCC__)
+
+typedef uint32_t r_u32x4 __attribute__((ext_vector_type(4)));
+typedef r_u32x4 r_u32x4_any __attribute__((aligned(1)));
+
+// 16 bytes of elements viewed as T[16/sizeof(T)].
+template <typename T>
+union Pack {
+  r_u32x4 raw;
+  T e[16 / sizeof(T)];
+};
+
+// Element type tag for bf16 storage with fp32 accumulation.
+struct Bf16Tag {};
+
+template <typename T>
+struct ElemTraits {
+  using storage = T;
+  using accum = T;
+  static constexpr int kPerVec = 16 / sizeof(T);
+  __device__ static accum widen(storage s) { return s; }
+  __device__ static storage narrow(accum a) { return a; }
+};
+template <>
+struct ElemTraits<Bf16Tag> {
+  using storage = uint16_t;
+  using accum = float;
+  static constexpr int kPerVec = 8;
+  __device__ static float widen(uint16_t s) { return bf16_to_f32(s); }
+  __device__ static uint16_t narrow(float a) { return f32_to_bf16(a); }
+};
+
+// Fold elements [lo, hi) across P team members and store the result on all P.
+//   src0 / dst0 : the buffers on team member 0
+//   hop         : bytes from one team member's buffer to the next member's
+//   kP          : P when known at compile time (loads fully unrolled), 0 when
+//                 only `np` is known
+// `lane` of `nlanes` dense cooperating lanes (a work-group or a whole grid).
+template <typename E, ROCSHMEM_OP Op, int kP, bool kNonTemporal>
+__device__ __forceinline__ void fold_span(
+    typename ElemTraits<E>::storage *dst0,
+    const typename ElemTraits<E>::storage *src0, int64_t hop, int np,
+    size_t lo, size_t hi, size_t lane, size_t nlanes) {
+  using Tr = ElemTraits<E>;
+  using S = typename Tr::storage;
+  using A = typename Tr::accum;
+  constexpr int V = Tr::kPerVec;
+  const int P = kP ? kP : np;
+
+  auto src_at = [&](int p, size_t i) -> const S * {
+    return reinterpret_cast<const S *>(reinterpret_cast<const char *>(src0 + i) + p * hop);
+  };
+  auto dst_at = [&](int p, size_t i) -> S * {
+    return reinterpret_cast<S *>(reinterpret_cast<char *>(dst0 + i) + p * hop);
+  };
+  auto scalar_one = [&](size_t i) {
+    A acc = Tr::widen(*src_at(0, i));
+    for (int p = 1; p < P; ++p) acc = combine<A, Op>(acc, Tr::widen(*src_at(p, i)));
+    const S out = Tr::narrow(acc);
+    for (int p = 0; p < P; ++p) *dst_at(p, i) = out;
+  };
+
+  // Elements before the first 16-byte boundary of the destination.
+  const uintptr_t mis = reinterpret_cast<uintptr_t>(dst0 + lo) & 15u;
+  size_t head = mis ? (16u - mis) / sizeof(S) : 0;
+  if (head > hi - lo) head = hi - lo;
+  for (size_t k = lane; k < head; k += nlanes) scalar_one(lo + k);
+  const size_t vlo = lo + head;
+  const size_t nvec = (hi - vlo) / V;
+
+  for (size_t v = lane; v < nvec; v += nlanes) {
+    const size_t i = vlo + v * V;
+    Pack<S> out;
+    if constexpr (kP != 0) {
+      Pack<S> in[kP ? kP : 1];
+#pragma unroll
+      for (int p = 0; p < kP; ++p) {
+        if constexpr (kNonTemporal)
+          in[p].raw = __builtin_nontemporal_load(reinterpret_cast<const r_u32x4_any *>(src_at(p, i)));
+        else
+          in[p].raw = *reinterpret_cast<const r_u32x4_any *>(src_at(p, i));
+      }
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        A acc = Tr::widen(in[0].e[e]);
+#pragma unroll
+        for (int p = 1; p < kP; ++p) acc = combine<A, Op>(acc, Tr::widen(in[p].e[e]));
+        out.e[e] = Tr::narrow(acc);
+      }
+    } else {
+      A acc[V];
+      Pack<S> in;
+      in.raw = *reinterpret_cast<const r_u32x4_any *>(src_at(0, i));
+#pragma unroll
+      for (int e = 0; e < V; ++e) acc[e] = Tr::widen(in.e[e]);
+      for (int p = 1; p < P; ++p) {
+        in.raw = *reinterpret_cast<const r_u32x4_any *>(src_at(p, i));
+#pragma unroll
+        for (int e = 0; e < V; ++e) acc[e] = combine<A, Op>(acc[e], Tr::widen(in.e[e]));
+      }
+#pragma unroll
+      for (int e = 0; e < V; ++e) out.e[e] = Tr::narrow(acc[e]);
+    }
+    for (int p = 0; p < P; ++p) {
+      if constexpr (kNonTemporal)
+        __builtin_nontemporal_store(out.raw, reinterpret_cast<r_u32x4 *>(dst_at(p, i)));
+      else
+        *reinterpret_cast<r_u32x4 *>(dst_at(p, i)) = out.raw;
+    }
+  }
+
+  const size_t tlo = vlo + nvec * V;
+  for (size_t k = tlo + lane; k < hi; k += nlanes) scalar_one(k);
+}
+
+// Dispatch on the team size so the common sizes get fully unrolled loads.
+template <typename E, ROCSHMEM_OP Op, bool kNonTemporal>
+__device__ __forceinline__ void fold_span_any(
+    typename ElemTraits<E>::storage *dst0,
+    const typename ElemTraits<E>::storage *src0, int64_t hop, int np,
+    size_t lo, size_t hi, size_t lane, size_t nlanes) {
+  switch (np) {
+    case 2: fold_span<E, Op, 2, kNonTemporal>(dst0, src0, hop, np, lo, hi, lane, nlanes); break;
+    case 4: fold_span<E, Op, 4, kNonTemporal>(dst0, src0, hop, np, lo, hi, lane, nlanes); break;
+    case 8: fold_span<E, Op, 8, kNonTemporal>(dst0, src0, hop, np, lo, hi, lane, nlanes); break;
+    default: fold_span<E, Op, 0, kNonTemporal>(dst0, src0, hop, np, lo, hi, lane, nlanes); break;
+  }
+}
+
+#endif  // __HIPCC__
+
+}  // namespace detail
+}  // namespace rocshmem
+
+#endif  // ROCSHMEM_AMD_DETAIL_REDUCE_ENGINE_HPP_

@@ -1,0 +1,178 @@
+// Remote memory access, put-with-signal and context lifecycle of one PE.
+#ifndef ROCSHMEM_AMD_DETAIL_RMA_HPP_
+#define ROCSHMEM_AMD_DETAIL_RMA_HPP_
+
+#include "copy_engine.hpp"
+#include "state.hpp"
+#include "sync.hpp"
+
+namespace rocshmem {
+namespace detail {
+
+#if defined(__HIPCC__)
+
+// Team-relative PE -> world PE for the calls that translate
+// (src/rocshmem_gpu.cpp:267-274: a null team_opaque passes pe through).
+__device__ __forceinline__ int translate_pe(rocshmem_ctx_t ctx, int pe) {
+  const TeamInfo *ti = reinterpret_cast<const TeamInfo *>(ctx.team_opaque);
+  return ti ? ti->pe_start + ti->stride * pe : pe;
+}
+
+// ---- thread granularity: copy, then order (context_ipc_device.cpp:62-88) ---
+__device__ __forceinline__ void putmem(Context *c, void *dest, const void *source,
+                                       size_t n, int pe) {
+  copy_thread(remote_addr(c, static_cast<char *>(dest), pe), source, n);
+  fence_full();
+}
+__device__ __forceinline__ void getmem(Context *c, void *dest, const void *source,
+                                       size_t n, int pe) {
+  copy_thread(dest, remote_addr(c, static_cast<const char *>(source), pe), n);
+  fence_full();
+}
+
+// ---- wavefront granularity (context_ipc_device.cpp:137-164) ---------------
+__device__ __forceinline__ void putmem_wave(Context *c, void *dest, const void *source,
+                                            size_t n, int pe) {
+  copy_wave(remote_addr(c, static_cast<char *>(dest), pe), source, n, g_state.nt_bytes);
+  fence_full();
+}
+__device__ __forceinline__ void getmem_wave(Context *c, void *dest, const void *source,
+                                            size_t n, int pe) {
+  copy_wave(dest, remote_addr(c, static_cast<const char *>(source), pe), n, g_state.nt_bytes);
+  fence_full();
+}
+
+// ---- work-group granularity: copy, then __syncthreads (:109-125) ----------
+__device__ __forceinline__ void putmem_wg(Context *c, void *dest, const void *source,
+                                          size_t n, int pe) {
+  copy_lanes(remote_addr(c, static_cast<char *>(dest), pe), source, n,
+             flat_thread_id(), flat_block_size(), g_state.nt_bytes);
+  __syncthreads();
+}
+__device__ __forceinline__ void getmem_wg(Context *c, void *dest, const void *source,
+                                          size_t n, int pe) {
+  copy_lanes(dest, remote_addr(c, static_cast<const char *>(source), pe), n,
+             flat_thread_id(), flat_block_size(), g_state.nt_bytes);
+  __syncthreads();
+}
+
+// ---- signal update by the one lane that leads the call (:221-298) ---------
+// The store / add is a release at agent scope, which orders it after the
+// payload the caller's group wrote before it.
+__device__ __forceinline__ void signal_update(Context *c, uint64_t *sig_addr,
+                                              uint64_t signal, int sig_op, int pe) {
+  unsigned long long *target =
+      reinterpret_cast<unsigned long long *>(remote_addr(c, sig_addr, pe));
+  switch (sig_op) {
+    case ROCSHMEM_SIGNAL_SET:
+      amo_set<unsigned long long>(target, signal);
+      break;
+    case ROCSHMEM_SIGNAL_ADD:
+      amo_add<unsigned long long>(target, signal);
+      break;
+    default:
+      break;  // unknown op: payload delivered, signal untouched
+  }
+}
+
+__device__ __forceinline__ void putmem_signal(Context *c, void *dest, const void *source,
+                                              size_t n, uint64_t *sig_addr,
+                                              uint64_t signal, int sig_op, int pe) {
+  putmem(c, dest, source, n, pe);
+  signal_update(c, sig_addr, signal, sig_op, pe);
+}
+__device__ __forceinline__ void putmem_signal_wave(Context *c, void *dest,
+                                                   const void *source, size_t n,
+                                                   uint64_t *sig_addr, uint64_t signal,
+                                                   int sig_op, int pe) {
+  putmem_wave(c, dest, source, n, pe);
+  // The leader is the lowest active lane, which exists for any active mask.
+  const unsigned long long mask = __ballot(1);
+  const unsigned lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+  if (lane == static_cast<unsigned>(__ffsll(static_cast<long long>(mask)) - 1))
+    signal_update(c, sig_addr, signal, sig_op, pe);
+}
+__device__ __forceinline__ void putmem_signal_wg(Context *c, void *dest,
+                                                 const void *source, size_t n,
+                                                 uint64_t *sig_addr, uint64_t signal,
+                                                 int sig_op, int pe) {
+  putmem_wg(c, dest, source, n, pe);
+  if (is_block_leader()) signal_update(c, sig_addr, signal, sig_op, pe);
+}
+
+// signal_fetch: atomic read of the caller's own word (:300-324).
+__device__ __forceinline__ uint64_t signal_fetch(const uint64_t *sig_addr) {
+  return amo_fetch(const_cast<unsigned long long *>(
+      reinterpret_cast<const unsigned long long *>(sig_addr)));
+}
+__device__ __forceinline__ uint64_t signal_fetch_wave(const uint64_t *sig_addr) {
+  const unsigned long long mask = __ballot(1);
+  const int leader = __ffsll(static_cast<long long>(mask)) - 1;
+  const unsigned lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+  unsigned long long v = 0;
+  if (static_cast<int>(lane) == leader) v = signal_fetch(sig_addr);
+  const unsigned lo = __builtin_amdgcn_readlane(static_cast<unsigned>(v), leader);
+  const unsigned hi = __builtin_amdgcn_readlane(static_cast<unsigned>(v >> 32), leader);
+  return (static_cast<uint64_t>(hi) << 32) | lo;
+}
+__device__ __forceinline__ uint64_t signal_fetch_wg(const uint64_t *sig_addr) {
+  __shared__ unsigned long long wg_value;
+  __syncthreads();
+  if (is_block_leader()) wg_value = signal_fetch(sig_addr);
+  __syncthreads();
+  return wg_value;
+}
+
+// ---- context lifecycle (src/rocshmem_gpu.cpp:286-325) ----------------------
+__device__ __forceinline__ Context *pool_claim(CtxPool *pool) {
+  const int words = (pool->capacity + 63) / 64;
+  for (int w = 0; w < words; ++w) {
+    unsigned long long m = __hip_atomic_load(&pool->free_mask[w], __ATOMIC_RELAXED,
+                                             __HIP_MEMORY_SCOPE_AGENT);
+    while (m) {
+      const int b = __ffsll(static_cast<long long>(m)) - 1;
+      const unsigned long long bit = 1ull << b;
+      const unsigned long long old = __hip_atomic_fetch_and(
+          &pool->free_mask[w], ~bit, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+      if (old & bit) return pool->slots + (w * 64 + b);
+      m = old & ~bit;
+    }
+  }
+  return nullptr;
+}
+__device__ __forceinline__ void pool_release(CtxPool *pool, Context *c) {
+  const int s = c->pool_slot;
+  __hip_atomic_fetch_or(&pool->free_mask[s >> 6], 1ull << (s & 63), __ATOMIC_RELEASE,
+                        __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Thread 0 claims a context of PE `pe` bound to `tinfo`; every thread learns
+// the outcome through *ctx (which lives in the caller's shared memory).
+__device__ __forceinline__ int wg_ctx_create_for(int pe, TeamInfo *tinfo, long options,
+                                                 rocshmem_ctx_t *ctx) {
+  if (is_block_leader()) {
+    Context *c = pool_claim(g_state.ctx_pool + pe);
+    if (c) {
+      c->tinfo = tinfo;
+      c->options = static_cast<unsigned>(options);
+    }
+    ctx->ctx_opaque = c;
+    ctx->team_opaque = tinfo;
+  }
+  __syncthreads();
+  return ctx->ctx_opaque ? 0 : -1;
+}
+
+__device__ __forceinline__ void wg_ctx_destroy(rocshmem_ctx_t *ctx) {
+  if (is_block_leader()) {
+    Context *c = reinterpret_cast<Context *>(ctx->ctx_opaque);
+    if (c && c->pool_slot >= 0) pool_release(g_state.ctx_pool + c->my_pe, c);
+  }
+}
+
+#endif  // __HIPCC__
+
+}  // namespace detail
+}  // namespace rocshmem
+
+#endif  // ROCSHMEM_AMD_DETAIL_RMA_HPP_

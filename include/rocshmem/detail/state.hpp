@@ -1,0 +1,202 @@
+// Device-visible runtime state: the symmetric-heap geometry, the per-PE
+// contexts and teams, and the work/sync area collectives use.
+//
+// One process hosts all P processing elements: PE p's share of the symmetric
+// heap is the slice [heap_base + p*pe_stride, +heap_size).  A symmetric
+// address handed to the API is always "my slice" address, and the matching
+// address on PE q is   addr + (q - my_pe) * pe_stride   — the closed form of
+// the reference's  ipc_bases[pe] + (dest - ipc_bases[my_pe])  translation
+// (src/ipc/context_ipc_device.cpp:62-69,109-125) for slices at a fixed stride.
+//
+// Every translation unit that includes the public header owns a private
+// __constant__ copy of DeviceState; the host runtime refreshes all registered
+// copies whenever the state changes, so no relocatable device code is needed
+// to link user kernels against the library.
+#ifndef ROCSHMEM_AMD_DETAIL_STATE_HPP_
+#define ROCSHMEM_AMD_DETAIL_STATE_HPP_
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <type_traits>
+
+#include "../rocshmem_common.hpp"
+
+namespace rocshmem {
+namespace detail {
+
+// How a work-group that asks for "the" context (default context, or
+// rocshmem_wg_ctx_create with no team) learns which PE it is acting as.
+enum PeRule : int {
+  PE_RULE_FIXED = 0,    // DeviceState::fixed_pe
+  PE_RULE_BLOCK_X = 1,  // blockIdx.x % n_pes
+  PE_RULE_BLOCK_Y = 2,  // blockIdx.y % n_pes
+  PE_RULE_BLOCK_Z = 3   // blockIdx.z % n_pes
+};
+
+// (pe_start, stride, size) of a team with respect to the world team; the
+// object rocshmem_ctx_t::team_opaque points at.  Mirrors what the reference
+// keeps in TeamInfo (src/team.hpp, used by src/rocshmem_gpu.cpp:267-274).
+struct TeamInfo {
+  int pe_start;
+  int stride;
+  int size;
+  int log_stride;
+};
+
+// Epoch-based flag array one collective kind of one team synchronises on.
+// slots[j] holds the highest epoch team member j has announced to this PE;
+// epoch is this PE's own count of completed rounds.  Nothing is ever reset,
+// so a round costs one store per peer and one polling sweep.
+struct SyncPad {
+  static constexpr int kMaxPes = 256;
+  unsigned long long slots[kMaxPes];
+  unsigned long long epoch;
+  unsigned long long pad_[7];
+};
+
+enum SyncKind : int {
+  SYNC_BARRIER = 0,
+  SYNC_REDUCE = 1,
+  SYNC_BCAST = 2,
+  SYNC_ALLTOALL = 3,
+  SYNC_KINDS = 4
+};
+
+// Per-PE, per-team object a rocshmem_team_t points at.
+struct Team {
+  TeamInfo wrt_world;
+  TeamInfo wrt_parent;
+  int my_pe;           // my index inside this team
+  int my_pe_in_world;
+  int num_pes;
+  int world_size;
+  int pool_index;      // which slice of the work/sync area this team owns
+  int pad_;
+  SyncPad *sync;       // [SYNC_KINDS] pads of this PE for this team
+  void *pWrk;          // ROCSHMEM_REDUCE_MIN_WRKDATA_SIZE * 8 bytes
+};
+
+// Per-PE communication context (device memory, pooled).
+struct Context {
+  char *heap_base;      // base of PE 0's slice
+  uint64_t pe_stride;   // bytes between consecutive slices
+  uint64_t ws_stride;   // bytes between consecutive PEs' work/sync areas
+  int my_pe;
+  int num_pes;
+  TeamInfo *tinfo;      // team this context translates PE numbers with
+  SyncPad *world_sync;  // this PE's pad for barrier_all / sync_all
+  unsigned options;
+  int pool_slot;        // index in the context pool, -1 for default contexts
+};
+
+// Pool of pre-built contexts for one PE.  A set bit in free_mask marks a free
+// slot; claiming is a fetch-and that clears the bit, releasing a fetch-or, so
+// work-groups never hold a lock (the reference guards a free list with a
+// ticket mutex, src/containers/free_list_impl.hpp:76-137).
+struct CtxPool {
+  static constexpr int kMaxWords = 64;  // up to 4096 contexts per PE
+  unsigned long long free_mask[kMaxWords];
+  int capacity;
+  int pad_;
+  Context *slots;       // [capacity]
+};
+
+struct DeviceState {
+  char *heap_base;
+  uint64_t pe_stride;
+  uint64_t heap_size;
+  uint64_t ws_stride;
+  int n_pes;
+  int pe_rule;
+  int fixed_pe;
+  int max_teams;
+  Context *default_ctx;   // [n_pes]
+  Team *world_team;       // [n_pes]
+  CtxPool *ctx_pool;      // [n_pes] one pool per PE
+  char *ws_base;          // work/sync area of PE 0
+  uint64_t nt_bytes;      // copies at least this large use non-temporal accesses
+};
+
+#if defined(__HIPCC__)
+
+// This translation unit's copy of the runtime state.
+__attribute__((used)) static __constant__ DeviceState g_state;
+
+__device__ __forceinline__ int acting_pe() {
+  const int n = g_state.n_pes;
+  switch (g_state.pe_rule) {
+    case PE_RULE_BLOCK_X: return static_cast<int>(blockIdx.x % n);
+    case PE_RULE_BLOCK_Y: return static_cast<int>(blockIdx.y % n);
+    case PE_RULE_BLOCK_Z: return static_cast<int>(blockIdx.z % n);
+    default: return g_state.fixed_pe;
+  }
+}
+
+// A null ctx_opaque denotes the default context of the acting PE.
+__device__ __forceinline__ Context *ctx_of(rocshmem_ctx_t ctx) {
+  Context *c = reinterpret_cast<Context *>(ctx.ctx_opaque);
+  return c ? c : g_state.default_ctx + acting_pe();
+}
+
+__device__ __forceinline__ Team *team_of(rocshmem_team_t team) {
+  return reinterpret_cast<Team *>(team);
+}
+
+// Address of the same symmetric object on PE `pe`.
+template <typename T>
+__device__ __forceinline__ T *remote_addr(const Context *c, T *local, int pe) {
+  const int64_t hop = static_cast<int64_t>(pe - c->my_pe) *
+                      static_cast<int64_t>(c->pe_stride);
+  return reinterpret_cast<T *>(
+      reinterpret_cast<char *>(const_cast<typename std::remove_const<T>::type *>(local)) + hop);
+}
+
+// Address of the same work/sync object on PE `pe`.
+template <typename T>
+__device__ __forceinline__ T *remote_ws(const Context *c, T *local, int pe) {
+  const int64_t hop = static_cast<int64_t>(pe - c->my_pe) *
+                      static_cast<int64_t>(c->ws_stride);
+  return reinterpret_cast<T *>(reinterpret_cast<char *>(local) + hop);
+}
+
+__device__ __forceinline__ unsigned flat_thread_id() {
+  return threadIdx.x + threadIdx.y * blockDim.x +
+         threadIdx.z * blockDim.x * blockDim.y;
+}
+__device__ __forceinline__ unsigned flat_block_size() {
+  return blockDim.x * blockDim.y * blockDim.z;
+}
+__device__ __forceinline__ bool is_block_leader() { return flat_thread_id() == 0; }
+__device__ __forceinline__ bool is_wave_leader() {
+  return (flat_thread_id() & 63u) == 0;
+}
+
+#endif  // __HIPCC__
+
+// ---- host side: keeping every translation unit's g_state current ----------
+using StateUploader = void (*)(const DeviceState *);
+// Implemented by the runtime library.  Registers `fn` and, when the runtime is
+// already initialised, calls it immediately.
+void register_state_uploader(StateUploader fn);
+
+#if defined(__HIPCC__)
+static void upload_state_to_this_tu(const DeviceState *s) {
+  hipError_t e = hipMemcpyToSymbol(HIP_SYMBOL(g_state), s, sizeof(DeviceState),
+                                   0, hipMemcpyHostToDevice);
+  if (e != hipSuccess) {
+    fprintf(stderr, "rocshmem: state upload failed: %s\n", hipGetErrorString(e));
+    abort();
+  }
+}
+__attribute__((used)) static const int state_uploader_registered_ =
+    (register_state_uploader(&upload_state_to_this_tu), 0);
+#endif
+
+}  // namespace detail
+}  // namespace rocshmem
+
+#endif  // ROCSHMEM_AMD_DETAIL_STATE_HPP_

@@ -1,0 +1,253 @@
+// Ordering, atomic memory operations, point-to-point waits and the PE barrier.
+//
+// The reference issues every atomic and fence at system scope, sequentially
+// consistent (src/ipc_policy.hpp:56-99, src/atomic.hpp:59-139) and polls with
+// a cache-bypassing load followed by s_waitcnt (src/assembly.hpp:115-162).
+// All PEs of this build live on one GPU, so agent scope is the widest scope
+// that exists: release = write back this XCD's L2 (buffer_wbl2 sc1),
+// acquire = invalidate it (buffer_inv sc1), polls and flag stores go through
+// to memory (sc1) so work-groups on different XCDs see each other.
+#ifndef ROCSHMEM_AMD_DETAIL_SYNC_HPP_
+#define ROCSHMEM_AMD_DETAIL_SYNC_HPP_
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+#include <type_traits>
+
+#include "state.hpp"
+
+namespace rocshmem {
+namespace detail {
+
+#if defined(__HIPCC__)
+
+__device__ __forceinline__ void fence_release() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+}
+__device__ __forceinline__ void fence_acquire() {
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+}
+// fence()/quiet(): order everything issued before against everything after.
+__device__ __forceinline__ void fence_full() {
+  __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "agent");
+}
+
+// Integer type of the same width, used to move float/double through atomics.
+template <size_t N> struct BitsOf;
+template <> struct BitsOf<1> { using type = uint8_t; };
+template <> struct BitsOf<2> { using type = uint16_t; };
+template <> struct BitsOf<4> { using type = uint32_t; };
+template <> struct BitsOf<8> { using type = uint64_t; };
+
+template <typename T>
+__device__ __forceinline__ T load_through(const T *p) {
+  using B = typename BitsOf<sizeof(T)>::type;
+  B b = __hip_atomic_load(reinterpret_cast<const B *>(p), __ATOMIC_RELAXED,
+                          __HIP_MEMORY_SCOPE_AGENT);
+  T out;
+  __builtin_memcpy(&out, &b, sizeof(T));
+  return out;
+}
+
+template <typename T>
+__device__ __forceinline__ void store_through(T *p, T v) {
+  using B = typename BitsOf<sizeof(T)>::type;
+  B b;
+  __builtin_memcpy(&b, &v, sizeof(T));
+  __hip_atomic_store(reinterpret_cast<B *>(p), b, __ATOMIC_RELAXED,
+                     __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// ---- atomic memory operations on an already-translated address -----------
+// Each is one device-wide RMW; the memory order is acquire-release so an AMO
+// can publish or consume data the way the reference's seq_cst ones do.
+template <typename T>
+__device__ __forceinline__ T amo_fetch_add(T *p, T v) {
+  return __hip_atomic_fetch_add(p, v, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+}
+template <typename T>
+__device__ __forceinline__ void amo_add(T *p, T v) {
+  (void)__hip_atomic_fetch_add(p, v, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+}
+template <typename T>
+__device__ __forceinline__ T amo_fetch_cas(T *p, T cond, T v) {
+  using B = typename BitsOf<sizeof(T)>::type;
+  B expected, desired;
+  __builtin_memcpy(&expected, &cond, sizeof(T));
+  __builtin_memcpy(&desired, &v, sizeof(T));
+  __hip_atomic_compare_exchange_strong(reinterpret_cast<B *>(p), &expected, desired,
+                                       __ATOMIC_ACQ_REL, __ATOMIC_ACQUIRE,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+  T out;
+  __builtin_memcpy(&out, &expected, sizeof(T));
+  return out;
+}
+template <typename T>
+__device__ __forceinline__ void amo_set(T *p, T v) {
+  using B = typename BitsOf<sizeof(T)>::type;
+  B b;
+  __builtin_memcpy(&b, &v, sizeof(T));
+  __hip_atomic_store(reinterpret_cast<B *>(p), b, __ATOMIC_RELEASE,
+                     __HIP_MEMORY_SCOPE_AGENT);
+}
+template <typename T>
+__device__ __forceinline__ T amo_fetch(T *p) {
+  using B = typename BitsOf<sizeof(T)>::type;
+  B b = __hip_atomic_load(reinterpret_cast<const B *>(p), __ATOMIC_ACQUIRE,
+                          __HIP_MEMORY_SCOPE_AGENT);
+  T out;
+  __builtin_memcpy(&out, &b, sizeof(T));
+  return out;
+}
+template <typename T>
+__device__ __forceinline__ T amo_swap(T *p, T v) {
+  using B = typename BitsOf<sizeof(T)>::type;
+  B b;
+  __builtin_memcpy(&b, &v, sizeof(T));
+  B old = __hip_atomic_exchange(reinterpret_cast<B *>(p), b, __ATOMIC_ACQ_REL,
+                                __HIP_MEMORY_SCOPE_AGENT);
+  T out;
+  __builtin_memcpy(&out, &old, sizeof(T));
+  return out;
+}
+template <typename T>
+__device__ __forceinline__ T amo_fetch_and(T *p, T v) {
+  return __hip_atomic_fetch_and(p, v, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+}
+template <typename T>
+__device__ __forceinline__ T amo_fetch_or(T *p, T v) {
+  return __hip_atomic_fetch_or(p, v, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+}
+template <typename T>
+__device__ __forceinline__ T amo_fetch_xor(T *p, T v) {
+  return __hip_atomic_fetch_xor(p, v, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// ---- point-to-point synchronisation ---------------------------------------
+// Comparator table of the reference's Context::test
+// (src/context_tmpl_device.hpp:337-377); an unknown comparator never holds.
+template <typename T>
+__device__ __forceinline__ bool compare(T x, int cmp, T val) {
+  switch (cmp) {
+    case ROCSHMEM_CMP_EQ: return x == val;
+    case ROCSHMEM_CMP_NE: return x != val;
+    case ROCSHMEM_CMP_GT: return x > val;
+    case ROCSHMEM_CMP_GE: return x >= val;
+    case ROCSHMEM_CMP_LT: return x < val;
+    case ROCSHMEM_CMP_LE: return x <= val;
+    default: return false;
+  }
+}
+
+// One poll.  A successful poll acquires, so data published before the value
+// was written (put_signal payloads) is visible afterwards.
+template <typename T>
+__device__ __forceinline__ int test(T *ivar, int cmp, T val) {
+  if (compare(load_through(ivar), cmp, val)) {
+    fence_acquire();
+    return 1;
+  }
+  return 0;
+}
+
+template <typename T>
+__device__ __forceinline__ void wait_until(T *ivar, int cmp, T val) {
+  while (!compare(load_through(ivar), cmp, val)) __builtin_amdgcn_s_sleep(1);
+  fence_acquire();
+}
+
+__device__ __forceinline__ size_t first_unmasked(size_t nelems, const int *status) {
+  size_t i = 0;
+  if (status) {
+    while (i < nelems && status[i] != 0) ++i;
+  }
+  return i;
+}
+
+// src/context_tmpl_device.hpp:220-250
+template <typename T>
+__device__ __forceinline__ size_t wait_until_any(T *ivars, size_t nelems,
+                                                 const int *status, int cmp, T val) {
+  if (!nelems) return SIZE_MAX;
+  const size_t pos = first_unmasked(nelems, status);
+  if (pos == nelems) return SIZE_MAX;
+  for (;;) {
+    for (size_t i = pos; i < nelems; ++i) {
+      if (status && status[i]) continue;
+      if (test(ivars + i, cmp, val)) return i;
+    }
+    __builtin_amdgcn_s_sleep(1);
+  }
+}
+
+// src/context_tmpl_device.hpp:252-275
+template <typename T>
+__device__ __forceinline__ void wait_until_all(T *ivars, size_t nelems,
+                                               const int *status, int cmp, T val) {
+  if (!nelems) return;
+  const size_t pos = first_unmasked(nelems, status);
+  if (pos == nelems) return;
+  for (size_t i = pos; i < nelems; ++i) {
+    if (status && status[i]) continue;
+    wait_until(ivars + i, cmp, val);
+  }
+}
+
+// src/context_tmpl_device.hpp:277-310: sweeps until one sweep finds at least
+// one satisfied entry and reports every entry that sweep found.
+template <typename T>
+__device__ __forceinline__ size_t wait_until_some(T *ivars, size_t nelems,
+                                                  size_t *indices, const int *status,
+                                                  int cmp, T val) {
+  if (!nelems) return 0;
+  const size_t pos = first_unmasked(nelems, status);
+  if (pos == nelems) return 0;
+  size_t ncompleted = 0;
+  while (ncompleted == 0) {
+    for (size_t i = pos; i < nelems; ++i) {
+      if (status && status[i]) continue;
+      if (test(ivars + i, cmp, val)) indices[ncompleted++] = i;
+    }
+    if (ncompleted == 0) __builtin_amdgcn_s_sleep(1);
+  }
+  return ncompleted;
+}
+
+// ---- barrier between the work-groups that act for the PEs of a team --------
+// Called by every thread of exactly one work-group per team member.  The
+// first wavefront does the work with its lanes in parallel: lane j announces
+// this round's epoch in member j's pad and polls member j's announcement in
+// the local pad.  (The reference's thread 0 walks the flags one by one and
+// resets them: src/ipc/context_ipc_device_coll.cpp:31-99.)
+__device__ __forceinline__ void sync_pes(const Context *c, SyncPad *pad,
+                                         int pe_start, int stride, int size,
+                                         int my_index) {
+  __syncthreads();
+  const unsigned tid = flat_thread_id();
+  if (tid < 64u) {
+    unsigned nl = flat_block_size();
+    if (nl > 64u) nl = 64u;
+    const unsigned long long round = load_through(&pad->epoch) + 1ull;
+    fence_release();
+    for (unsigned j = tid; j < static_cast<unsigned>(size); j += nl) {
+      SyncPad *peer = remote_ws(c, pad, pe_start + static_cast<int>(j) * stride);
+      store_through(&peer->slots[my_index], round);
+    }
+    for (unsigned j = tid; j < static_cast<unsigned>(size); j += nl) {
+      while (load_through(&pad->slots[j]) < round) __builtin_amdgcn_s_sleep(1);
+    }
+    fence_acquire();
+    // All lanes of this wavefront have left their polling loops here.
+    if (tid == 0) store_through(&pad->epoch, round);
+  }
+  __syncthreads();
+}
+
+#endif  // __HIPCC__
+
+}  // namespace detail
+}  // namespace rocshmem
+
+#endif  // ROCSHMEM_AMD_DETAIL_SYNC_HPP_

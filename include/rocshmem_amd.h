@@ -1,0 +1,318 @@
+/* C entry points of the MI355X symmetric-heap data-movement library.
+ *
+ * The reference library has no C or FFI layer: its interface is the C++ API of
+ * include/rocshmem/rocshmem.hpp, with the data path living in __device__
+ * functions that user kernels call.  This header is that interface flattened
+ * for callers that cannot compile HIP C++ (ctypes, cgo, JNI ...):
+ *
+ *   - the host API (init / malloc / teams) one to one, and
+ *   - for every device-side operation a "driver": a kernel launch in which
+ *     work-groups call the public device function exactly as a user kernel
+ *     would, with the PE each work-group acts for given by the caller.
+ *
+ * Conventions
+ *   - All P processing elements live in this process on one GPU.  A symmetric
+ *     address is always passed as the address on PE `my_pe` (what
+ *     rocshmem_amd_malloc returned while that PE was acting, or
+ *     rocshmem_amd_pe_ptr of it).
+ *   - `stream` is a hipStream_t (NULL = the null stream).  Drivers only
+ *     enqueue; call rocshmem_amd_stream_sync to wait.
+ *   - Return value 0 = success, negative = argument error (nothing launched).
+ *     HIP failures are fatal (message on stderr, exit), as in the reference
+ *     (src/util.hpp:41-49).
+ */
+#ifndef ROCSHMEM_AMD_H_
+#define ROCSHMEM_AMD_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *rocshmem_amd_stream_t;
+typedef void *rocshmem_amd_team_t;
+
+/* Element types (reductions, atomics, waits). */
+enum rocshmem_amd_dtype {
+  ROCSHMEM_AMD_SHORT = 0,
+  ROCSHMEM_AMD_INT = 1,
+  ROCSHMEM_AMD_LONG = 2,
+  ROCSHMEM_AMD_LONGLONG = 3,
+  ROCSHMEM_AMD_FLOAT = 4,
+  ROCSHMEM_AMD_DOUBLE = 5,
+  ROCSHMEM_AMD_BF16 = 6,
+  ROCSHMEM_AMD_UINT = 7,
+  ROCSHMEM_AMD_ULONG = 8,
+  ROCSHMEM_AMD_ULONGLONG = 9
+};
+
+/* Reduction operators: values of ROCSHMEM_OP (rocshmem_common.hpp:40-49). */
+enum rocshmem_amd_op {
+  ROCSHMEM_AMD_SUM = 0,
+  ROCSHMEM_AMD_MAX = 1,
+  ROCSHMEM_AMD_MIN = 2,
+  ROCSHMEM_AMD_PROD = 3,
+  ROCSHMEM_AMD_AND = 4,
+  ROCSHMEM_AMD_OR = 5,
+  ROCSHMEM_AMD_XOR = 6
+};
+
+enum rocshmem_amd_granularity {
+  ROCSHMEM_AMD_THREAD = 0, /* rocshmem_putmem / getmem            */
+  ROCSHMEM_AMD_WAVE = 1,   /* rocshmem_putmem_wave / getmem_wave  */
+  ROCSHMEM_AMD_WG = 2      /* rocshmem_putmem_wg / getmem_wg      */
+};
+
+enum rocshmem_amd_rma_op { ROCSHMEM_AMD_PUT = 0, ROCSHMEM_AMD_GET = 1 };
+
+enum rocshmem_amd_amo_op {
+  ROCSHMEM_AMD_AMO_FETCH_ADD = 0,
+  ROCSHMEM_AMD_AMO_ADD = 1,
+  ROCSHMEM_AMD_AMO_FETCH_INC = 2,
+  ROCSHMEM_AMD_AMO_INC = 3,
+  ROCSHMEM_AMD_AMO_COMPARE_SWAP = 4,
+  ROCSHMEM_AMD_AMO_FETCH = 5,
+  ROCSHMEM_AMD_AMO_SET = 6,
+  ROCSHMEM_AMD_AMO_SWAP = 7,
+  ROCSHMEM_AMD_AMO_FETCH_AND = 8,
+  ROCSHMEM_AMD_AMO_FETCH_OR = 9,
+  ROCSHMEM_AMD_AMO_FETCH_XOR = 10
+};
+
+enum rocshmem_amd_wait_fn {
+  ROCSHMEM_AMD_TEST = 0,
+  ROCSHMEM_AMD_WAIT_UNTIL = 1,
+  ROCSHMEM_AMD_WAIT_UNTIL_ANY = 2,
+  ROCSHMEM_AMD_WAIT_UNTIL_ALL = 3,
+  ROCSHMEM_AMD_WAIT_UNTIL_SOME = 4
+};
+
+enum rocshmem_amd_sync_fn {
+  ROCSHMEM_AMD_BARRIER_ALL = 0, /* rocshmem_ctx_wg_barrier_all */
+  ROCSHMEM_AMD_SYNC_ALL = 1,    /* rocshmem_ctx_wg_sync_all    */
+  ROCSHMEM_AMD_TEAM_SYNC = 2    /* rocshmem_ctx_wg_team_sync   */
+};
+
+/* ===================== host API (runtime, heap, teams) ===================== */
+
+/* rocshmem_init (include/rocshmem/rocshmem.hpp:62, src/rocshmem.cpp:73-105).
+ * npes <= 0: take ROCSHMEM_EMU_NPES (default 1); heap_bytes_per_pe == 0: take
+ * ROCSHMEM_HEAP_SIZE (default 1 GiB, src/memory/heap_memory.hpp:114). */
+int rocshmem_amd_init(int npes, size_t heap_bytes_per_pe);
+/* rocshmem_finalize (rocshmem.hpp:103). */
+int rocshmem_amd_finalize(void);
+/* rocshmem_n_pes / rocshmem_my_pe (rocshmem.hpp:130-137). */
+int rocshmem_amd_n_pes(void);
+int rocshmem_amd_my_pe(void);
+/* Emulation controls (no reference counterpart): which PE the host acts as,
+ * and how default-context work-groups find their PE (0 fixed, 1/2/3 =
+ * blockIdx.x/y/z mod P). */
+int rocshmem_amd_set_pe(int pe);
+int rocshmem_amd_set_pe_rule(int rule);
+/* rocshmem_malloc / rocshmem_free (rocshmem.hpp:115-123): NULL on size 0 or
+ * exhaustion; the object exists at the same offset on every PE. */
+void *rocshmem_amd_malloc(size_t size);
+int rocshmem_amd_free(void *ptr);
+/* Address of a symmetric object on another PE; NULL if ptr is not in the heap. */
+void *rocshmem_amd_pe_ptr(const void *ptr, int pe);
+/* Allocator accounting: SingleHeap::get_size/get_used/get_avail
+ * (src/memory/single_heap.cpp:56-62), per PE. */
+size_t rocshmem_amd_heap_size(void);
+size_t rocshmem_amd_heap_used(void);
+size_t rocshmem_amd_heap_avail(void);
+size_t rocshmem_amd_pe_stride(void);
+
+/* Teams (rocshmem.hpp:165-236; src/rocshmem.cpp:193-319, src/team.cpp:51-111). */
+rocshmem_amd_team_t rocshmem_amd_team_world(void);
+int rocshmem_amd_team_split_strided(rocshmem_amd_team_t parent, int start, int stride,
+                                    int size, rocshmem_amd_team_t *new_team);
+void rocshmem_amd_team_destroy(rocshmem_amd_team_t team);
+int rocshmem_amd_team_n_pes(rocshmem_amd_team_t team);
+int rocshmem_amd_team_my_pe(rocshmem_amd_team_t team);
+int rocshmem_amd_team_translate_pe(rocshmem_amd_team_t src_team, int src_pe,
+                                   rocshmem_amd_team_t dest_team);
+/* The same team as seen by another PE (NULL if that PE is not a member). */
+rocshmem_amd_team_t rocshmem_amd_team_on(rocshmem_amd_team_t team, int pe);
+
+/* Plain device memory and staging for callers without a HIP binding. */
+void *rocshmem_amd_dev_alloc(size_t size);
+int rocshmem_amd_dev_free(void *ptr);
+int rocshmem_amd_copy_in(void *dst_dev, const void *src_host, size_t n);
+int rocshmem_amd_copy_out(void *dst_host, const void *src_dev, size_t n);
+int rocshmem_amd_fill(void *dst_dev, int byte, size_t n);
+int rocshmem_amd_stream_sync(rocshmem_amd_stream_t stream);
+/* hipEvent pair on `stream`; elapsed time in milliseconds. */
+void *rocshmem_amd_timer_create(void);
+int rocshmem_amd_timer_start(void *timer, rocshmem_amd_stream_t stream);
+int rocshmem_amd_timer_stop(void *timer, rocshmem_amd_stream_t stream);
+float rocshmem_amd_timer_elapsed_ms(void *timer);
+int rocshmem_amd_timer_destroy(void *timer);
+
+/* ============================ RMA drivers ================================== */
+
+/* rocshmem_ctx_putmem[_wave|_wg] / rocshmem_ctx_getmem[_wave|_wg]
+ * (rocshmem_RMA.hpp, rocshmem_RMA_X.hpp:243-274,744-775;
+ *  src/ipc/context_ipc_device.cpp:62-164).
+ * n_wgs work-groups of wg_size threads act for PE my_pe.  The message of
+ * nbytes is cut into tiles of tile_bytes (0 = one equal share per group,
+ * rounded up to 16 bytes); group g — a work-group, a wavefront or a thread,
+ * per `gran` — moves tiles g, g+G, g+2G ... with one API call each.  The whole
+ * transfer is repeated `iters` times inside the kernel. */
+int rocshmem_amd_rma(int rma_op, int gran, void *dest, const void *source, size_t nbytes,
+                     size_t tile_bytes, int my_pe, int pe, int n_wgs, int wg_size,
+                     int iters, rocshmem_amd_stream_t stream);
+
+/* Host-initiated bulk copy between PEs over the whole GPU: the host-side
+ * rocshmem_putmem / rocshmem_getmem (rocshmem_RMA.hpp; reference forwards them
+ * to MPI_Put / MPI_Get, src/host/host_helpers.hpp:52-88). */
+int rocshmem_amd_putmem(void *dest, const void *source, size_t nbytes, int my_pe, int pe,
+                        rocshmem_amd_stream_t stream);
+int rocshmem_amd_getmem(void *dest, const void *source, size_t nbytes, int my_pe, int pe,
+                        rocshmem_amd_stream_t stream);
+
+/* wf_coal_policy coalesce (src/wf_coal_policy.cpp:57-172) on one wavefront:
+ * lane i of the 64 is active iff bit i of active_mask; inputs are 64-entry
+ * host arrays; outputs say whether the lane must send and its message size. */
+int rocshmem_amd_wf_coalesce(const int *pe, const uint64_t *src, const uint64_t *dst,
+                             const uint64_t *size, uint64_t active_mask, int *sends_out,
+                             uint64_t *size_out);
+
+/* ========================= collective drivers ============================== */
+
+/* rocshmem_ctx_<T>_<op>_wg_reduce (rocshmem_COLL.hpp:348-598;
+ * src/ipc/context_ipc_tmpl_device.hpp:361-418): one work-group per team member.
+ * dest/source are the addresses on the member the host currently acts as
+ * (which must belong to the team).  Returns the device status
+ * (ROCSHMEM_SUCCESS 0 / ROCSHMEM_ERROR 1), after waiting for the kernel. */
+int rocshmem_amd_wg_reduce(int dtype, int op, rocshmem_amd_team_t team, void *dest,
+                           const void *source, int nreduce, int wg_size,
+                           rocshmem_amd_stream_t stream);
+/* rocshmem_ctx_<T>_wg_alltoall / _wg_broadcast / _wg_fcollect
+ * (rocshmem_COLL.hpp:44-258; context_ipc_tmpl_device.hpp:420-531).
+ * elem_size in {1,2,4,8} selects the typed entry point (char/short/int/long). */
+int rocshmem_amd_wg_alltoall(int elem_size, rocshmem_amd_team_t team, void *dest,
+                             const void *source, int nelems, int wg_size,
+                             rocshmem_amd_stream_t stream);
+int rocshmem_amd_wg_broadcast(int elem_size, rocshmem_amd_team_t team, void *dest,
+                              const void *source, int nelems, int pe_root, int wg_size,
+                              rocshmem_amd_stream_t stream);
+int rocshmem_amd_wg_fcollect(int elem_size, rocshmem_amd_team_t team, void *dest,
+                             const void *source, int nelems, int wg_size,
+                             rocshmem_amd_stream_t stream);
+/* rocshmem_ctx_wg_barrier_all / _wg_sync_all / _wg_team_sync
+ * (rocshmem.hpp:440-493; src/ipc/context_ipc_device_coll.cpp:31-123).
+ * One work-group per PE runs `rounds` rounds of: put the round number into
+ * the next member's `scratch` word, synchronise, check the word it received.
+ * scratch: symmetric uint64.  Returns the number of wrong observations. */
+int rocshmem_amd_wg_sync(int sync_fn, rocshmem_amd_team_t team, uint64_t *scratch,
+                         int rounds, int wg_size, rocshmem_amd_stream_t stream);
+
+/* Host-called all-reduce over an active set, all CUs:
+ * rocshmem_ctx_<T>_<op>_to_all(ctx, dest, source, nreduce, PE_start,
+ * logPE_stride, PE_size, pWrk, pSync) (src/rocshmem.cpp:724-735,974-980;
+ * src/host/host_templates.hpp:333-376, in place when dest == source).
+ * dest/source: addresses on PE PE_start. */
+int rocshmem_amd_to_all(int dtype, int op, void *dest, const void *source, int nreduce,
+                        int PE_start, int logPE_stride, int PE_size,
+                        rocshmem_amd_stream_t stream);
+/* Team form: host rocshmem_ctx_<T>_<op>_reduce (src/rocshmem.cpp:737-747). */
+int rocshmem_amd_reduce(int dtype, int op, rocshmem_amd_team_t team, void *dest,
+                        const void *source, int nreduce, rocshmem_amd_stream_t stream);
+/* Host-called alltoall / broadcast / fcollect over a team, all CUs (byte
+ * counts per team member).  broadcast: host rocshmem_ctx_<T>_broadcast
+ * (rocshmem_COLL.hpp; src/host/host_templates.hpp:160-200). */
+int rocshmem_amd_alltoallmem(rocshmem_amd_team_t team, void *dest, const void *source,
+                             size_t nbytes, rocshmem_amd_stream_t stream);
+int rocshmem_amd_broadcastmem(rocshmem_amd_team_t team, void *dest, const void *source,
+                              size_t nbytes, int pe_root, rocshmem_amd_stream_t stream);
+int rocshmem_amd_fcollectmem(rocshmem_amd_team_t team, void *dest, const void *source,
+                             size_t nbytes, rocshmem_amd_stream_t stream);
+
+/* ====================== atomics, signals, waits ============================ */
+
+/* rocshmem_<T>_atomic_<op> (rocshmem_AMO.hpp; src/ipc_policy.hpp:69-99).
+ * `counters` is a symmetric array of n_slots elements (address on my_pe).
+ * Operation i targets global counter ids[i] in [0, P*n_slots): PE
+ * ids[i] / n_slots, element ids[i] % n_slots, with operand values[i]
+ * (values == NULL: operand 1) and, for compare_swap, conds[i].  Fetching
+ * operations store their result in fetched[i] (may be NULL).  ids, values,
+ * conds, fetched are device arrays.  Thread t of the grid performs operations
+ * t, t+T, t+2T ... */
+int rocshmem_amd_amo(int amo_op, int dtype, void *counters, uint32_t n_slots,
+                     const uint32_t *ids, const void *values, const void *conds,
+                     void *fetched, size_t n_ops, int my_pe, int n_wgs, int wg_size,
+                     rocshmem_amd_stream_t stream);
+
+/* rocshmem_putmem_signal[_wave|_wg] (rocshmem_SIG_OP.hpp:27-228;
+ * src/ipc/context_ipc_device.cpp:221-298).  Every group (thread / wavefront /
+ * work-group per `gran`) of the grid acting for my_pe sends its tile of the
+ * message (tiling as in rocshmem_amd_rma, one tile per group) and updates the
+ * signal word on `pe`, `calls` times. */
+int rocshmem_amd_put_signal(int gran, void *dest, const void *source, size_t nbytes,
+                            uint64_t *sig_addr, uint64_t signal, int sig_op, int my_pe,
+                            int pe, int n_wgs, int wg_size, int calls,
+                            rocshmem_amd_stream_t stream);
+/* rocshmem_signal_fetch[_wave|_wg] (rocshmem_SIG_OP.hpp:616-618): value read
+ * by PE my_pe from its own word. */
+int rocshmem_amd_signal_fetch(int gran, const uint64_t *sig_addr, int my_pe,
+                              uint64_t *value_out);
+
+/* Ping-pong (tests/functional_tests/ping_pong_tester.cpp:43-61,
+ * examples/rocshmem_put_signal_test.cc:31-47): work-group 0 acts for pe_a,
+ * work-group 1 for pe_b; `iters` round trips of putmem_signal_wg (payload
+ * nbytes from `buf` to the peer's `buf`, signal word `sig` set to the round
+ * number) answered after rocshmem_ulong_wait_until.  buf/sig: addresses on
+ * pe_a.  ticks_out (host, optional) receives the wall_clock64 ticks pe_a
+ * spent; tick_hz_out the tick rate. */
+int rocshmem_amd_pingpong(void *buf, uint64_t *sig, size_t nbytes, int iters, int pe_a,
+                          int pe_b, int wg_size, uint64_t *ticks_out, double *tick_hz_out,
+                          rocshmem_amd_stream_t stream);
+
+/* MoE-style dispatch with put_signal.  For every ordered pair (s, d) of the P
+ * world PEs, `wgs_per_pair` work-groups acting for s send rows
+ * [send_row[s*P+d], +count[s*P+d]) of s's `send` buffer to rows starting at
+ * recv_row[s*P+d] of d's `recv` buffer with rocshmem_putmem_signal_wg, adding
+ * the number of rows they sent to d's sig[s]; one more work-group per PE d
+ * waits with rocshmem_ulong_wait_until(sig[s], GE, count[s*P+d]) for every s.
+ * count/send_row/recv_row: device arrays of P*P uint32.  send/recv/sig:
+ * addresses on PE 0. */
+int rocshmem_amd_dispatch_put_signal(void *recv, const void *send, uint64_t *sig,
+                                     const uint32_t *count, const uint32_t *send_row,
+                                     const uint32_t *recv_row, size_t row_bytes,
+                                     int wgs_per_pair, int wg_size,
+                                     rocshmem_amd_stream_t stream);
+
+/* rocshmem_<T>_test / _wait_until / _wait_until_any / _all / _some
+ * (rocshmem_P2P_SYNC.hpp:44-556; src/context_tmpl_device.hpp:201-377) called
+ * by one thread on the device array ivars (nelems elements of dtype); `value`
+ * points at one host element of dtype.  ret_out: the function's return value
+ * (test: 0/1; any: index or SIZE_MAX; some: count; others 0); indices_out
+ * (host, nelems entries, optional) receives wait_until_some's indices.
+ * Blocking forms return only once satisfied: use them on values that already
+ * hold, or with the waker below. */
+int rocshmem_amd_wait_test(int wait_fn, int dtype, void *ivars, size_t nelems,
+                           const int *status, int cmp, const void *value,
+                           size_t *ret_out, size_t *indices_out);
+/* Same call made by work-group 0 while work-group 1 stores `wake_value` into
+ * ivars[wake_index] after roughly delay_ticks wall-clock ticks. */
+int rocshmem_amd_wait_test_woken(int wait_fn, int dtype, void *ivars, size_t nelems,
+                                 const int *status, int cmp, const void *value,
+                                 size_t wake_index, const void *wake_value,
+                                 uint64_t delay_ticks, size_t *ret_out,
+                                 size_t *indices_out);
+
+/* Context lifecycle (rocshmem.hpp:334-370; src/rocshmem_gpu.cpp:286-325): each
+ * of n_wgs work-groups creates per_wg contexts (rocshmem_wg_ctx_create, or
+ * rocshmem_wg_team_create_ctx when team != NULL), records each return code in
+ * status_out[wg*per_wg + k] and the context's rocshmem_ctx_my_pe / n_pes in
+ * pe_out / npes_out (host arrays), then destroys them all. */
+int rocshmem_amd_ctx_cycle(rocshmem_amd_team_t team, int n_wgs, int wg_size, int per_wg,
+                           int *status_out, int *pe_out, int *npes_out);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* ROCSHMEM_AMD_H_ */

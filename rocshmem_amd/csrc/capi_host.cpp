@@ -1,0 +1,136 @@
+// C entry points that wrap the host runtime: bring-up, symmetric allocation,
+// teams, staging copies and timers.  No kernels are launched from this file.
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstdlib>
+
+#include "drv_common.hpp"
+#include "rocshmem_amd.h"
+
+using rocshmem::runtime::rt;
+
+extern "C" {
+
+int rocshmem_amd_init(int npes, size_t heap_bytes_per_pe) {
+  return rt().init(npes, heap_bytes_per_pe);
+}
+int rocshmem_amd_finalize(void) {
+  rt().finalize();
+  return 0;
+}
+int rocshmem_amd_n_pes(void) { return rocshmem::rocshmem_n_pes(); }
+int rocshmem_amd_my_pe(void) { return rocshmem::rocshmem_my_pe(); }
+int rocshmem_amd_set_pe(int pe) {
+  if (!rt().live || pe < 0 || pe >= rt().npes) return -1;
+  rt().set_pe(pe);
+  return 0;
+}
+int rocshmem_amd_set_pe_rule(int rule) {
+  if (!rt().live || rule < 0 || rule > 3) return -1;
+  rt().set_pe_rule(rule);
+  return 0;
+}
+void *rocshmem_amd_malloc(size_t size) { return rt().sym_malloc(size); }
+int rocshmem_amd_free(void *ptr) {
+  rt().sym_free(ptr);
+  return 0;
+}
+void *rocshmem_amd_pe_ptr(const void *ptr, int pe) {
+  return rt().live ? rt().pe_ptr(ptr, pe) : nullptr;
+}
+size_t rocshmem_amd_heap_size(void) { return rt().allocator.size(); }
+size_t rocshmem_amd_heap_used(void) { return rt().allocator.used(); }
+size_t rocshmem_amd_heap_avail(void) { return rt().allocator.avail(); }
+size_t rocshmem_amd_pe_stride(void) { return rt().pe_stride; }
+
+rocshmem_amd_team_t rocshmem_amd_team_world(void) { return rocshmem::ROCSHMEM_TEAM_WORLD; }
+int rocshmem_amd_team_split_strided(rocshmem_amd_team_t parent, int start, int stride,
+                                    int size, rocshmem_amd_team_t *new_team) {
+  rocshmem::rocshmem_team_t t = rocshmem::ROCSHMEM_TEAM_INVALID;
+  const int rc = rocshmem::rocshmem_team_split_strided(
+      static_cast<rocshmem::rocshmem_team_t>(parent), start, stride, size, nullptr, 0, &t);
+  *new_team = t;
+  return rc;
+}
+void rocshmem_amd_team_destroy(rocshmem_amd_team_t team) {
+  rocshmem::rocshmem_team_destroy(static_cast<rocshmem::rocshmem_team_t>(team));
+}
+int rocshmem_amd_team_n_pes(rocshmem_amd_team_t team) {
+  return rocshmem::rocshmem_team_n_pes(static_cast<rocshmem::rocshmem_team_t>(team));
+}
+int rocshmem_amd_team_my_pe(rocshmem_amd_team_t team) {
+  return rocshmem::rocshmem_team_my_pe(static_cast<rocshmem::rocshmem_team_t>(team));
+}
+int rocshmem_amd_team_translate_pe(rocshmem_amd_team_t src_team, int src_pe,
+                                   rocshmem_amd_team_t dest_team) {
+  return rocshmem::rocshmem_team_translate_pe(
+      static_cast<rocshmem::rocshmem_team_t>(src_team), src_pe,
+      static_cast<rocshmem::rocshmem_team_t>(dest_team));
+}
+rocshmem_amd_team_t rocshmem_amd_team_on(rocshmem_amd_team_t team, int pe) {
+  return rocshmem::rocshmem_emu_team_on(static_cast<rocshmem::rocshmem_team_t>(team), pe);
+}
+
+void *rocshmem_amd_dev_alloc(size_t size) {
+  void *p = nullptr;
+  if (size == 0) return nullptr;
+  DRV_CHECK_HIP(hipMalloc(&p, size));
+  return p;
+}
+int rocshmem_amd_dev_free(void *ptr) {
+  if (ptr) DRV_CHECK_HIP(hipFree(ptr));
+  return 0;
+}
+int rocshmem_amd_copy_in(void *dst_dev, const void *src_host, size_t n) {
+  if (n) DRV_CHECK_HIP(hipMemcpy(dst_dev, src_host, n, hipMemcpyHostToDevice));
+  return 0;
+}
+int rocshmem_amd_copy_out(void *dst_host, const void *src_dev, size_t n) {
+  if (n) DRV_CHECK_HIP(hipMemcpy(dst_host, src_dev, n, hipMemcpyDeviceToHost));
+  return 0;
+}
+int rocshmem_amd_fill(void *dst_dev, int byte, size_t n) {
+  if (n) DRV_CHECK_HIP(hipMemset(dst_dev, byte, n));
+  return 0;
+}
+int rocshmem_amd_stream_sync(rocshmem_amd_stream_t stream) {
+  DRV_CHECK_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+  return 0;
+}
+
+struct DrvTimer {
+  hipEvent_t start, stop;
+};
+void *rocshmem_amd_timer_create(void) {
+  DrvTimer *t = new DrvTimer;
+  DRV_CHECK_HIP(hipEventCreate(&t->start));
+  DRV_CHECK_HIP(hipEventCreate(&t->stop));
+  return t;
+}
+int rocshmem_amd_timer_start(void *timer, rocshmem_amd_stream_t stream) {
+  DRV_CHECK_HIP(hipEventRecord(static_cast<DrvTimer *>(timer)->start,
+                               static_cast<hipStream_t>(stream)));
+  return 0;
+}
+int rocshmem_amd_timer_stop(void *timer, rocshmem_amd_stream_t stream) {
+  DRV_CHECK_HIP(hipEventRecord(static_cast<DrvTimer *>(timer)->stop,
+                               static_cast<hipStream_t>(stream)));
+  return 0;
+}
+float rocshmem_amd_timer_elapsed_ms(void *timer) {
+  DrvTimer *t = static_cast<DrvTimer *>(timer);
+  DRV_CHECK_HIP(hipEventSynchronize(t->stop));
+  float ms = 0.f;
+  DRV_CHECK_HIP(hipEventElapsedTime(&ms, t->start, t->stop));
+  return ms;
+}
+int rocshmem_amd_timer_destroy(void *timer) {
+  DrvTimer *t = static_cast<DrvTimer *>(timer);
+  DRV_CHECK_HIP(hipEventDestroy(t->start));
+  DRV_CHECK_HIP(hipEventDestroy(t->stop));
+  delete t;
+  return 0;
+}
+
+}  // extern "C"

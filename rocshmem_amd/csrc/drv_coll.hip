@@ -1,0 +1,544 @@
+// Drivers for collectives: the per-work-group device API (one work-group per
+// team member) and the host-called whole-GPU forms.
+#include "drv_common.hpp"
+#include "rocshmem_amd.h"
+
+namespace rocshmem {
+namespace drv {
+
+// ---------------------------------------------------------------------------
+// Per-work-group device API.  Work-group j acts for team member j.
+// ---------------------------------------------------------------------------
+struct WgCollArgs {
+  detail::Team *team_row;    // team objects of this team, indexed by world PE
+  detail::Context *ctx_row;  // default contexts, indexed by world PE
+  char *dest0;               // addresses of the buffers on world PE 0
+  const char *src0;
+  uint64_t pe_stride;
+  int pe_start;
+  int stride;
+  int nelems;
+  int root;
+  int *status;
+};
+
+struct Member {
+  rocshmem_ctx_t ctx;
+  rocshmem_team_t team;
+  char *dest;
+  const char *source;
+};
+__device__ __forceinline__ Member member_of(const WgCollArgs &a) {
+  const int pe = a.pe_start + static_cast<int>(blockIdx.x) * a.stride;
+  Member m;
+  m.ctx = rocshmem_ctx_t{a.ctx_row + pe, &a.team_row[pe].wrt_world};
+  m.team = reinterpret_cast<rocshmem_team_t>(a.team_row + pe);
+  m.dest = a.dest0 + static_cast<uint64_t>(pe) * a.pe_stride;
+  m.source = a.src0 + static_cast<uint64_t>(pe) * a.pe_stride;
+  return m;
+}
+
+// Public reduce entry point for (T, Op).
+template <typename T, ROCSHMEM_OP Op>
+struct PublicReduce;
+#define DRV_PUBLIC_REDUCE(T, TN, OPN, OP)                                          \
+  template <>                                                                      \
+  struct PublicReduce<T, OP> {                                                     \
+    using storage = T;                                                             \
+    __device__ static int call(rocshmem_ctx_t c, rocshmem_team_t t, T *d, const T *s, \
+                               int n) {                                            \
+      return rocshmem_ctx_##TN##_##OPN##_wg_reduce(c, t, d, s, n);                 \
+    }                                                                              \
+  };
+#define DRV_PUBLIC_ARITH(T, TN)                \
+  DRV_PUBLIC_REDUCE(T, TN, sum, ROCSHMEM_SUM)  \
+  DRV_PUBLIC_REDUCE(T, TN, max, ROCSHMEM_MAX)  \
+  DRV_PUBLIC_REDUCE(T, TN, min, ROCSHMEM_MIN)  \
+  DRV_PUBLIC_REDUCE(T, TN, prod, ROCSHMEM_PROD)
+#define DRV_PUBLIC_INT(T, TN)                  \
+  DRV_PUBLIC_ARITH(T, TN)                      \
+  DRV_PUBLIC_REDUCE(T, TN, and, ROCSHMEM_AND)  \
+  DRV_PUBLIC_REDUCE(T, TN, or, ROCSHMEM_OR)    \
+  DRV_PUBLIC_REDUCE(T, TN, xor, ROCSHMEM_XOR)
+DRV_PUBLIC_INT(short, short)
+DRV_PUBLIC_INT(int, int)
+DRV_PUBLIC_INT(long, long)
+DRV_PUBLIC_INT(long long, longlong)
+DRV_PUBLIC_ARITH(float, float)
+DRV_PUBLIC_ARITH(double, double)
+template <>
+struct PublicReduce<rocshmem_bf16, ROCSHMEM_SUM> {
+  using storage = rocshmem_bf16;
+  __device__ static int call(rocshmem_ctx_t c, rocshmem_team_t t, rocshmem_bf16 *d,
+                             const rocshmem_bf16 *s, int n) {
+    return rocshmem_ctx_bf16_sum_wg_reduce(c, t, d, s, n);
+  }
+};
+
+template <typename T, ROCSHMEM_OP Op>
+__global__ void wg_reduce_kernel(WgCollArgs a) {
+  const Member m = member_of(a);
+  const int rc = PublicReduce<T, Op>::call(m.ctx, m.team, reinterpret_cast<T *>(m.dest),
+                                           reinterpret_cast<const T *>(m.source), a.nelems);
+  if (threadIdx.x == 0 && rc != ROCSHMEM_SUCCESS) atomicMax(a.status, rc);
+}
+
+enum WgMove { MOVE_ALLTOALL, MOVE_BROADCAST, MOVE_FCOLLECT };
+
+template <typename T, int kMove>
+__device__ __forceinline__ void wg_move_call(const Member &m, int n, int root);
+#define DRV_MOVE(T, TN)                                                            \
+  template <>                                                                      \
+  __device__ __forceinline__ void wg_move_call<T, MOVE_ALLTOALL>(const Member &m,  \
+                                                                 int n, int) {     \
+    rocshmem_ctx_##TN##_wg_alltoall(m.ctx, m.team, reinterpret_cast<T *>(m.dest),  \
+                                    reinterpret_cast<const T *>(m.source), n);     \
+  }                                                                                \
+  template <>                                                                      \
+  __device__ __forceinline__ void wg_move_call<T, MOVE_BROADCAST>(const Member &m, \
+                                                                  int n, int root) { \
+    rocshmem_ctx_##TN##_wg_broadcast(m.ctx, m.team, reinterpret_cast<T *>(m.dest), \
+                                     reinterpret_cast<const T *>(m.source), n, root); \
+  }                                                                                \
+  template <>                                                                      \
+  __device__ __forceinline__ void wg_move_call<T, MOVE_FCOLLECT>(const Member &m,  \
+                                                                 int n, int) {     \
+    rocshmem_ctx_##TN##_wg_fcollect(m.ctx, m.team, reinterpret_cast<T *>(m.dest),  \
+                                    reinterpret_cast<const T *>(m.source), n);     \
+  }
+DRV_MOVE(char, char)
+DRV_MOVE(short, short)
+DRV_MOVE(int, int)
+DRV_MOVE(long, long)
+
+template <typename T, int kMove>
+__global__ void wg_move_kernel(WgCollArgs a) {
+  wg_move_call<T, kMove>(member_of(a), a.nelems, a.root);
+}
+
+struct SyncArgs {
+  detail::Team *team_row;
+  detail::Context *ctx_row;
+  uint64_t *scratch0;  // address on world PE 0
+  uint64_t pe_stride;
+  int pe_start, stride, size;
+  int fn;
+  int rounds;
+  int *errors;
+};
+
+__global__ void wg_sync_kernel(SyncArgs a) {
+  const int j = blockIdx.x;
+  const int pe = a.pe_start + j * a.stride;
+  const int next = (j + 1) % a.size;  // team-relative: p() translates it
+  rocshmem_ctx_t ctx{a.ctx_row + pe, &a.team_row[pe].wrt_world};
+  rocshmem_team_t team = reinterpret_cast<rocshmem_team_t>(a.team_row + pe);
+  uint64_t *mine = reinterpret_cast<uint64_t *>(reinterpret_cast<char *>(a.scratch0) +
+                                                static_cast<uint64_t>(pe) * a.pe_stride);
+  for (int r = 1; r <= a.rounds; ++r) {
+    if (threadIdx.x == 0) rocshmem_ctx_uint64_p(ctx, mine, static_cast<uint64_t>(r), next);
+    if (a.fn == ROCSHMEM_AMD_BARRIER_ALL) rocshmem_ctx_wg_barrier_all(ctx);
+    else if (a.fn == ROCSHMEM_AMD_SYNC_ALL) rocshmem_ctx_wg_sync_all(ctx);
+    else rocshmem_ctx_wg_team_sync(ctx, team);
+    if (threadIdx.x == 0) {
+      const uint64_t seen = rocshmem_ctx_uint64_atomic_fetch(ctx, mine, pe);
+      if (seen != static_cast<uint64_t>(r)) atomicAdd(a.errors, 1);
+    }
+    // Nobody may overwrite the word of round r before everyone has read it.
+    if (a.fn == ROCSHMEM_AMD_BARRIER_ALL) rocshmem_ctx_wg_barrier_all(ctx);
+    else if (a.fn == ROCSHMEM_AMD_SYNC_ALL) rocshmem_ctx_wg_sync_all(ctx);
+    else rocshmem_ctx_wg_team_sync(ctx, team);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Host-called, whole-GPU forms.
+// ---------------------------------------------------------------------------
+template <typename E>
+struct GridReduceArgs {
+  typename detail::ElemTraits<E>::storage *dst0;        // buffers on the first member
+  const typename detail::ElemTraits<E>::storage *src0;
+  int64_t hop;                                          // bytes between members
+  int np;
+  size_t n;
+  size_t span;                                          // elements per work-group span
+};
+
+// Each work-group folds contiguous spans of the index space: it reads the span
+// from all P sources and writes it to all P destinations.
+template <typename E, ROCSHMEM_OP Op, bool kNonTemporal>
+__global__ void grid_reduce_kernel(GridReduceArgs<E> a) {
+  using S = typename detail::ElemTraits<E>::storage;
+  const uintptr_t mis = reinterpret_cast<uintptr_t>(a.dst0) & 15u;
+  size_t head = mis ? (16u - mis) / sizeof(S) : 0;
+  if (head > a.n) head = a.n;
+  if (blockIdx.x == 0 && head)
+    detail::fold_span_any<E, Op, false>(a.dst0, a.src0, a.hop, a.np, 0, head, threadIdx.x,
+                                        blockDim.x);
+  const size_t body = a.n - head;
+  const size_t nspans = (body + a.span - 1) / a.span;
+  for (size_t s = blockIdx.x; s < nspans; s += gridDim.x) {
+    const size_t lo = head + s * a.span;
+    const size_t hi = lo + a.span < a.n ? lo + a.span : a.n;
+    detail::fold_span_any<E, Op, kNonTemporal>(a.dst0, a.src0, a.hop, a.np, lo, hi,
+                                               threadIdx.x, blockDim.x);
+  }
+}
+
+template <typename E, ROCSHMEM_OP Op>
+void launch_grid_reduce(void *dst0, const void *src0, int64_t hop, int np, size_t n,
+                        hipStream_t stream) {
+  using S = typename detail::ElemTraits<E>::storage;
+  GridReduceArgs<E> a;
+  a.dst0 = static_cast<S *>(dst0);
+  a.src0 = static_cast<const S *>(src0);
+  a.hop = hop;
+  a.np = np;
+  a.n = n;
+  const int wg = 256;
+  // 4 vectors per lane per span: 16 KiB of every source per work-group visit.
+  a.span = static_cast<size_t>(wg) * 4 * (16 / sizeof(S));
+  const size_t nspans = (n + a.span - 1) / a.span;
+  const size_t max_wgs = 256 * 8;
+  const int grid = static_cast<int>(nspans < max_wgs ? (nspans ? nspans : 1) : max_wgs);
+  const bool nt = n * sizeof(S) >= runtime::rt().state.nt_bytes;
+  if (nt)
+    hipLaunchKernelGGL((grid_reduce_kernel<E, Op, true>), dim3(grid), dim3(wg), 0, stream, a);
+  else
+    hipLaunchKernelGGL((grid_reduce_kernel<E, Op, false>), dim3(grid), dim3(wg), 0, stream, a);
+  DRV_CHECK_HIP(hipGetLastError());
+}
+
+// Whole-GPU alltoall / broadcast / fcollect: the P*P (or P) blocks are cut
+// into spans, and work-groups walk the list of all spans.
+struct GridMoveArgs {
+  char *dest0;        // buffers on the first member
+  const char *src0;
+  int64_t hop;
+  int np;
+  int root;
+  size_t nbytes;      // per block
+  size_t span;
+};
+
+template <int kMove, bool kNonTemporal>
+__global__ void grid_move_kernel(GridMoveArgs a) {
+  const size_t spans_per_block = (a.nbytes + a.span - 1) / a.span;
+  const size_t nblocks = kMove == MOVE_BROADCAST ? static_cast<size_t>(a.np)
+                                                 : static_cast<size_t>(a.np) * a.np;
+  const size_t total = nblocks * spans_per_block;
+  for (size_t s = blockIdx.x; s < total; s += gridDim.x) {
+    const size_t blk = s / spans_per_block;
+    const size_t off = (s % spans_per_block) * a.span;
+    const size_t len = a.nbytes - off < a.span ? a.nbytes - off : a.span;
+    char *d;
+    const char *src;
+    if constexpr (kMove == MOVE_BROADCAST) {
+      const int j = static_cast<int>(blk);
+      if (j == a.root) continue;
+      d = a.dest0 + j * a.hop + off;
+      src = a.src0 + a.root * a.hop + off;
+    } else {
+      const int i = static_cast<int>(blk / a.np);  // sender
+      const int j = static_cast<int>(blk % a.np);  // receiver
+      d = a.dest0 + j * a.hop + static_cast<size_t>(i) * a.nbytes + off;
+      src = a.src0 + i * a.hop + (kMove == MOVE_ALLTOALL ? static_cast<size_t>(j) * a.nbytes : 0) + off;
+    }
+    detail::copy_lanes_impl<4, kNonTemporal>(d, src, len, threadIdx.x, blockDim.x);
+  }
+}
+
+template <int kMove>
+void launch_grid_move(char *dest0, const char *src0, int64_t hop, int np, int root,
+                      size_t nbytes, hipStream_t stream) {
+  if (!nbytes) return;
+  GridMoveArgs a{dest0, src0, hop, np, root, nbytes, 0};
+  a.span = nbytes <= (64u << 10) ? nbytes : (64u << 10);
+  const size_t spans_per_block = (nbytes + a.span - 1) / a.span;
+  const size_t nblocks = kMove == MOVE_BROADCAST ? np : static_cast<size_t>(np) * np;
+  const size_t total = nblocks * spans_per_block;
+  const size_t max_wgs = 256 * 16;
+  const int grid = static_cast<int>(total < max_wgs ? total : max_wgs);
+  if (nbytes >= runtime::rt().state.nt_bytes)
+    hipLaunchKernelGGL((grid_move_kernel<kMove, true>), dim3(grid), dim3(256), 0, stream, a);
+  else
+    hipLaunchKernelGGL((grid_move_kernel<kMove, false>), dim3(grid), dim3(256), 0, stream, a);
+  DRV_CHECK_HIP(hipGetLastError());
+}
+
+// Resolve a team handle (of the acting PE) to what the kernels need.
+struct TeamView {
+  const detail::Team *host;
+  detail::Team *row;
+};
+inline bool view_team(rocshmem_amd_team_t team, TeamView *v) {
+  auto &r = runtime::rt();
+  v->host = r.host_team(static_cast<rocshmem_team_t>(team));
+  if (!v->host || v->host->my_pe < 0) return false;
+  v->row = r.d_teams + static_cast<size_t>(v->host->pool_index) * r.npes;
+  return true;
+}
+// Address on world PE 0 of a symmetric address given for the acting PE.
+inline char *on_pe0(const void *p) {
+  auto &r = runtime::rt();
+  return const_cast<char *>(static_cast<const char *>(p)) -
+         static_cast<size_t>(r.acting_pe) * r.pe_stride;
+}
+inline bool in_heap(const void *p) {
+  return runtime::rt().offset_of(p) != runtime::Pow2Allocator::kNoBlock;
+}
+
+template <typename T, ROCSHMEM_OP Op>
+void launch_wg_reduce(const WgCollArgs &a, int size, int wg_size, hipStream_t s) {
+  hipLaunchKernelGGL((wg_reduce_kernel<T, Op>), dim3(size), dim3(wg_size), 0, s, a);
+}
+
+}  // namespace drv
+}  // namespace rocshmem
+
+using namespace rocshmem;
+using namespace rocshmem::drv;
+
+namespace {
+
+template <typename Fn>
+bool for_dtype_op(int dtype, int op, Fn &&fn) {
+  // fn is a generic lambda taking (type tag, op tag).
+  auto ops_int = [&](auto tag) -> bool {
+    switch (op) {
+      case ROCSHMEM_AMD_SUM: fn(tag, std::integral_constant<ROCSHMEM_OP, ROCSHMEM_SUM>{}); return true;
+      case ROCSHMEM_AMD_MAX: fn(tag, std::integral_constant<ROCSHMEM_OP, ROCSHMEM_MAX>{}); return true;
+      case ROCSHMEM_AMD_MIN: fn(tag, std::integral_constant<ROCSHMEM_OP, ROCSHMEM_MIN>{}); return true;
+      case ROCSHMEM_AMD_PROD: fn(tag, std::integral_constant<ROCSHMEM_OP, ROCSHMEM_PROD>{}); return true;
+      case ROCSHMEM_AMD_AND: fn(tag, std::integral_constant<ROCSHMEM_OP, ROCSHMEM_AND>{}); return true;
+      case ROCSHMEM_AMD_OR: fn(tag, std::integral_constant<ROCSHMEM_OP, ROCSHMEM_OR>{}); return true;
+      case ROCSHMEM_AMD_XOR: fn(tag, std::integral_constant<ROCSHMEM_OP, ROCSHMEM_XOR>{}); return true;
+      default: return false;
+    }
+  };
+  auto ops_float = [&](auto tag) -> bool {
+    switch (op) {
+      case ROCSHMEM_AMD_SUM: fn(tag, std::integral_constant<ROCSHMEM_OP, ROCSHMEM_SUM>{}); return true;
+      case ROCSHMEM_AMD_MAX: fn(tag, std::integral_constant<ROCSHMEM_OP, ROCSHMEM_MAX>{}); return true;
+      case ROCSHMEM_AMD_MIN: fn(tag, std::integral_constant<ROCSHMEM_OP, ROCSHMEM_MIN>{}); return true;
+      case ROCSHMEM_AMD_PROD: fn(tag, std::integral_constant<ROCSHMEM_OP, ROCSHMEM_PROD>{}); return true;
+      default: return false;
+    }
+  };
+  switch (dtype) {
+    case ROCSHMEM_AMD_SHORT: return ops_int(static_cast<short *>(nullptr));
+    case ROCSHMEM_AMD_INT: return ops_int(static_cast<int *>(nullptr));
+    case ROCSHMEM_AMD_LONG: return ops_int(static_cast<long *>(nullptr));
+    case ROCSHMEM_AMD_LONGLONG: return ops_int(static_cast<long long *>(nullptr));
+    case ROCSHMEM_AMD_FLOAT: return ops_float(static_cast<float *>(nullptr));
+    case ROCSHMEM_AMD_DOUBLE: return ops_float(static_cast<double *>(nullptr));
+    case ROCSHMEM_AMD_BF16:
+      if (op != ROCSHMEM_AMD_SUM) return false;
+      fn(static_cast<rocshmem_bf16 *>(nullptr), std::integral_constant<ROCSHMEM_OP, ROCSHMEM_SUM>{});
+      return true;
+    default: return false;
+  }
+}
+
+// Engine element tag for a public element type.
+template <typename T> struct EngineTag { using type = T; };
+template <> struct EngineTag<rocshmem_bf16> { using type = detail::Bf16Tag; };
+
+size_t dtype_size(int dtype) {
+  switch (dtype) {
+    case ROCSHMEM_AMD_SHORT: case ROCSHMEM_AMD_BF16: return 2;
+    case ROCSHMEM_AMD_INT: case ROCSHMEM_AMD_FLOAT: case ROCSHMEM_AMD_UINT: return 4;
+    default: return 8;
+  }
+}
+
+int grid_reduce_common(int dtype, int op, void *dst_first, const void *src_first, int64_t hop,
+                       int np, int nreduce, hipStream_t stream) {
+  if (nreduce < 0) return -1;
+  if (nreduce == 0) return 0;
+  const bool ok = for_dtype_op(dtype, op, [&](auto *tag, auto opc) {
+    using T = typename std::remove_pointer<decltype(tag)>::type;
+    using E = typename EngineTag<T>::type;
+    launch_grid_reduce<E, decltype(opc)::value>(dst_first, src_first, hop, np,
+                                                static_cast<size_t>(nreduce), stream);
+  });
+  return ok ? 0 : -1;
+}
+
+WgCollArgs make_wg_args(const TeamView &v, void *dest, const void *source, int nelems, int root,
+                        int *status) {
+  auto &r = runtime::rt();
+  WgCollArgs a;
+  a.team_row = v.row;
+  a.ctx_row = r.d_default_ctx;
+  a.dest0 = on_pe0(dest);
+  a.src0 = on_pe0(source);
+  a.pe_stride = r.pe_stride;
+  a.pe_start = v.host->wrt_world.pe_start;
+  a.stride = v.host->wrt_world.stride;
+  a.nelems = nelems;
+  a.root = root;
+  a.status = status;
+  return a;
+}
+
+template <int kMove>
+int wg_move_common(int elem_size, rocshmem_amd_team_t team, void *dest, const void *source,
+                   int nelems, int root, int wg_size, hipStream_t s) {
+  TeamView v;
+  if (!view_team(team, &v) || !valid_launch(1, wg_size) || nelems < 0) return -1;
+  if (!in_heap(dest) || !in_heap(source)) return -1;
+  if (kMove == MOVE_BROADCAST && (root < 0 || root >= v.host->num_pes)) return -1;
+  const WgCollArgs a = make_wg_args(v, dest, source, nelems, root, nullptr);
+  const dim3 g(v.host->num_pes), b(wg_size);
+  switch (elem_size) {
+    case 1: hipLaunchKernelGGL((wg_move_kernel<char, kMove>), g, b, 0, s, a); break;
+    case 2: hipLaunchKernelGGL((wg_move_kernel<short, kMove>), g, b, 0, s, a); break;
+    case 4: hipLaunchKernelGGL((wg_move_kernel<int, kMove>), g, b, 0, s, a); break;
+    case 8: hipLaunchKernelGGL((wg_move_kernel<long, kMove>), g, b, 0, s, a); break;
+    default: return -1;
+  }
+  DRV_CHECK_HIP(hipGetLastError());
+  return 0;
+}
+
+template <int kMove>
+int grid_move_common(rocshmem_amd_team_t team, void *dest, const void *source, size_t nbytes,
+                     int root, hipStream_t s) {
+  TeamView v;
+  if (!view_team(team, &v)) return -1;
+  if (!in_heap(dest) || !in_heap(source)) return -1;
+  if (kMove == MOVE_BROADCAST && (root < 0 || root >= v.host->num_pes)) return -1;
+  auto &r = runtime::rt();
+  const int64_t first = static_cast<int64_t>(v.host->wrt_world.pe_start) * r.pe_stride;
+  const int64_t hop = static_cast<int64_t>(v.host->wrt_world.stride) * r.pe_stride;
+  launch_grid_move<kMove>(on_pe0(dest) + first, on_pe0(source) + first, hop, v.host->num_pes,
+                          root, nbytes, s);
+  return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int rocshmem_amd_wg_reduce(int dtype, int op, rocshmem_amd_team_t team, void *dest,
+                           const void *source, int nreduce, int wg_size,
+                           rocshmem_amd_stream_t stream) {
+  TeamView v;
+  if (!view_team(team, &v) || !valid_launch(1, wg_size) || nreduce < 0) return -1;
+  if (!in_heap(dest) || !in_heap(source)) return -1;
+  int *d_status;
+  DRV_CHECK_HIP(hipMalloc(&d_status, sizeof(int)));
+  DRV_CHECK_HIP(hipMemset(d_status, 0, sizeof(int)));
+  const WgCollArgs a = make_wg_args(v, dest, source, nreduce, 0, d_status);
+  hipStream_t s = as_stream(stream);
+  const bool ok = for_dtype_op(dtype, op, [&](auto *tag, auto opc) {
+    using T = typename std::remove_pointer<decltype(tag)>::type;
+    launch_wg_reduce<T, decltype(opc)::value>(a, v.host->num_pes, wg_size, s);
+  });
+  int status = -1;
+  if (ok) {
+    DRV_CHECK_HIP(hipGetLastError());
+    DRV_CHECK_HIP(hipStreamSynchronize(s));
+    DRV_CHECK_HIP(hipMemcpy(&status, d_status, sizeof(int), hipMemcpyDeviceToHost));
+  }
+  DRV_CHECK_HIP(hipFree(d_status));
+  return status;
+}
+
+int rocshmem_amd_wg_alltoall(int elem_size, rocshmem_amd_team_t team, void *dest,
+                             const void *source, int nelems, int wg_size,
+                             rocshmem_amd_stream_t stream) {
+  return wg_move_common<MOVE_ALLTOALL>(elem_size, team, dest, source, nelems, 0, wg_size,
+                                       as_stream(stream));
+}
+int rocshmem_amd_wg_broadcast(int elem_size, rocshmem_amd_team_t team, void *dest,
+                              const void *source, int nelems, int pe_root, int wg_size,
+                              rocshmem_amd_stream_t stream) {
+  return wg_move_common<MOVE_BROADCAST>(elem_size, team, dest, source, nelems, pe_root,
+                                        wg_size, as_stream(stream));
+}
+int rocshmem_amd_wg_fcollect(int elem_size, rocshmem_amd_team_t team, void *dest,
+                             const void *source, int nelems, int wg_size,
+                             rocshmem_amd_stream_t stream) {
+  return wg_move_common<MOVE_FCOLLECT>(elem_size, team, dest, source, nelems, 0, wg_size,
+                                       as_stream(stream));
+}
+
+int rocshmem_amd_wg_sync(int sync_fn, rocshmem_amd_team_t team, uint64_t *scratch, int rounds,
+                         int wg_size, rocshmem_amd_stream_t stream) {
+  auto &r = runtime::rt();
+  if (!r.live || rounds < 0 || !valid_launch(1, wg_size) || !in_heap(scratch)) return -1;
+  if (sync_fn < ROCSHMEM_AMD_BARRIER_ALL || sync_fn > ROCSHMEM_AMD_TEAM_SYNC) return -1;
+  TeamView v;
+  if (sync_fn == ROCSHMEM_AMD_TEAM_SYNC) {
+    if (!view_team(team, &v)) return -1;
+  } else {
+    if (!view_team(r.team_handle(0, r.acting_pe), &v)) return -1;
+  }
+  int *d_err;
+  DRV_CHECK_HIP(hipMalloc(&d_err, sizeof(int)));
+  DRV_CHECK_HIP(hipMemset(d_err, 0, sizeof(int)));
+  SyncArgs a;
+  a.team_row = v.row;
+  a.ctx_row = r.d_default_ctx;
+  a.scratch0 = reinterpret_cast<uint64_t *>(on_pe0(scratch));
+  a.pe_stride = r.pe_stride;
+  a.pe_start = v.host->wrt_world.pe_start;
+  a.stride = v.host->wrt_world.stride;
+  a.size = v.host->num_pes;
+  a.fn = sync_fn;
+  a.rounds = rounds;
+  a.errors = d_err;
+  hipStream_t s = as_stream(stream);
+  hipLaunchKernelGGL(wg_sync_kernel, dim3(a.size), dim3(wg_size), 0, s, a);
+  DRV_CHECK_HIP(hipGetLastError());
+  DRV_CHECK_HIP(hipStreamSynchronize(s));
+  int err = 0;
+  DRV_CHECK_HIP(hipMemcpy(&err, d_err, sizeof(int), hipMemcpyDeviceToHost));
+  DRV_CHECK_HIP(hipFree(d_err));
+  return err;
+}
+
+int rocshmem_amd_to_all(int dtype, int op, void *dest, const void *source, int nreduce,
+                        int PE_start, int logPE_stride, int PE_size,
+                        rocshmem_amd_stream_t stream) {
+  auto &r = runtime::rt();
+  if (!r.live || PE_start < 0 || logPE_stride < 0 || logPE_stride > 30 || PE_size < 1) return -1;
+  const int stride = 1 << logPE_stride;
+  if (PE_start + static_cast<long>(stride) * (PE_size - 1) >= r.npes) return -1;
+  if (!in_heap(dest) || !in_heap(source)) return -1;
+  if (r.pe_of(dest) != PE_start || r.pe_of(source) != PE_start) return -1;
+  const size_t bytes = static_cast<size_t>(nreduce < 0 ? 0 : nreduce) * dtype_size(dtype);
+  if (r.offset_of(dest) + bytes > r.heap_size || r.offset_of(source) + bytes > r.heap_size) return -1;
+  return grid_reduce_common(dtype, op, dest, source, static_cast<int64_t>(stride) * r.pe_stride,
+                            PE_size, nreduce, as_stream(stream));
+}
+
+int rocshmem_amd_reduce(int dtype, int op, rocshmem_amd_team_t team, void *dest,
+                        const void *source, int nreduce, rocshmem_amd_stream_t stream) {
+  TeamView v;
+  if (!view_team(team, &v) || !in_heap(dest) || !in_heap(source)) return -1;
+  auto &r = runtime::rt();
+  const size_t bytes = static_cast<size_t>(nreduce < 0 ? 0 : nreduce) * dtype_size(dtype);
+  if (r.offset_of(dest) + bytes > r.heap_size || r.offset_of(source) + bytes > r.heap_size) return -1;
+  const int64_t first = static_cast<int64_t>(v.host->wrt_world.pe_start) * r.pe_stride;
+  const int64_t hop = static_cast<int64_t>(v.host->wrt_world.stride) * r.pe_stride;
+  return grid_reduce_common(dtype, op, on_pe0(dest) + first, on_pe0(source) + first, hop,
+                            v.host->num_pes, nreduce, as_stream(stream));
+}
+
+int rocshmem_amd_alltoallmem(rocshmem_amd_team_t team, void *dest, const void *source,
+                             size_t nbytes, rocshmem_amd_stream_t stream) {
+  return grid_move_common<MOVE_ALLTOALL>(team, dest, source, nbytes, 0, as_stream(stream));
+}
+int rocshmem_amd_broadcastmem(rocshmem_amd_team_t team, void *dest, const void *source,
+                              size_t nbytes, int pe_root, rocshmem_amd_stream_t stream) {
+  return grid_move_common<MOVE_BROADCAST>(team, dest, source, nbytes, pe_root, as_stream(stream));
+}
+int rocshmem_amd_fcollectmem(rocshmem_amd_team_t team, void *dest, const void *source,
+                             size_t nbytes, rocshmem_amd_stream_t stream) {
+  return grid_move_common<MOVE_FCOLLECT>(team, dest, source, nbytes, 0, as_stream(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,46 @@
+// Shared by the driver translation units: error check, context handles for a
+// given PE, and the tiling rule the RMA and signal drivers use.
+#ifndef ROCSHMEM_AMD_DRV_COMMON_HPP_
+#define ROCSHMEM_AMD_DRV_COMMON_HPP_
+
+#include <hip/hip_runtime.h>
+
+#include <cstdio>
+#include <cstdlib>
+
+#include "rocshmem/rocshmem.hpp"
+#include "runtime.hpp"
+
+#define DRV_CHECK_HIP(expr)                                                       \
+  do {                                                                            \
+    hipError_t drv_err_ = (expr);                                                 \
+    if (drv_err_ != hipSuccess) {                                                 \
+      fprintf(stderr, "rocshmem: HIP error %d (%s) at %s:%d\n", (int)drv_err_,    \
+              hipGetErrorString(drv_err_), __FILE__, __LINE__);                   \
+      exit(EXIT_FAILURE);                                                         \
+    }                                                                             \
+  } while (0)
+
+namespace rocshmem {
+namespace drv {
+
+inline bool valid_launch(int n_wgs, int wg_size) {
+  return n_wgs >= 1 && wg_size >= 1 && wg_size <= 1024;
+}
+inline bool valid_pe(int pe) {
+  return runtime::rt().live && pe >= 0 && pe < runtime::rt().npes;
+}
+inline hipStream_t as_stream(void *s) { return static_cast<hipStream_t>(s); }
+
+// Bytes per tile when the caller leaves the choice to the driver: an equal
+// share per group, rounded up to 16 bytes.
+inline size_t auto_tile(size_t nbytes, size_t groups) {
+  size_t t = (nbytes + groups - 1) / groups;
+  t = (t + 15) / 16 * 16;
+  return t ? t : 16;
+}
+
+}  // namespace drv
+}  // namespace rocshmem
+
+#endif  // ROCSHMEM_AMD_DRV_COMMON_HPP_

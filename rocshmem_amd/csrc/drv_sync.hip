@@ -1,0 +1,666 @@
+// Drivers for atomics, put-with-signal, point-to-point waits, the ping-pong
+// and MoE-dispatch patterns, and context lifecycle.
+#include "drv_common.hpp"
+#include "rocshmem_amd.h"
+
+namespace rocshmem {
+namespace drv {
+
+// ---------------------------------------------------------------------------
+// Atomic memory operations.
+// ---------------------------------------------------------------------------
+template <typename T>
+struct AmoArgs {
+  T *counters;  // address on my_pe
+  uint32_t n_slots;
+  const uint32_t *ids;
+  const T *values;
+  const T *conds;
+  T *fetched;
+  size_t n_ops;
+  rocshmem_ctx_t ctx;
+};
+
+template <typename T>
+__device__ __host__ inline T zero_of() {
+  return static_cast<T>(0);
+}
+
+// Public entry points for element type T.
+template <typename T>
+struct PublicAmo;
+#define DRV_AMO_STD(T, TN)                                                                 \
+  __device__ static T fetch_add(rocshmem_ctx_t c, T *d, T v, int pe) {                     \
+    return rocshmem_ctx_##TN##_atomic_fetch_add(c, d, v, pe);                              \
+  }                                                                                        \
+  __device__ static void add(rocshmem_ctx_t c, T *d, T v, int pe) {                        \
+    rocshmem_ctx_##TN##_atomic_add(c, d, v, pe);                                           \
+  }                                                                                        \
+  __device__ static T fetch_inc(rocshmem_ctx_t c, T *d, int pe) {                          \
+    return rocshmem_ctx_##TN##_atomic_fetch_inc(c, d, pe);                                 \
+  }                                                                                        \
+  __device__ static void inc(rocshmem_ctx_t c, T *d, int pe) {                             \
+    rocshmem_ctx_##TN##_atomic_inc(c, d, pe);                                              \
+  }                                                                                        \
+  __device__ static T compare_swap(rocshmem_ctx_t c, T *d, T cond, T v, int pe) {          \
+    return rocshmem_ctx_##TN##_atomic_compare_swap(c, d, cond, v, pe);                     \
+  }
+#define DRV_AMO_EXT(T, TN)                                                                 \
+  __device__ static T fetch(rocshmem_ctx_t c, T *d, int pe) {                              \
+    return rocshmem_ctx_##TN##_atomic_fetch(c, d, pe);                                     \
+  }                                                                                        \
+  __device__ static void set(rocshmem_ctx_t c, T *d, T v, int pe) {                        \
+    rocshmem_ctx_##TN##_atomic_set(c, d, v, pe);                                           \
+  }                                                                                        \
+  __device__ static T swap(rocshmem_ctx_t c, T *d, T v, int pe) {                          \
+    return rocshmem_ctx_##TN##_atomic_swap(c, d, v, pe);                                   \
+  }
+#define DRV_AMO_BIT(T, TN)                                                                 \
+  __device__ static T fetch_and(rocshmem_ctx_t c, T *d, T v, int pe) {                     \
+    return rocshmem_ctx_##TN##_atomic_fetch_and(c, d, v, pe);                              \
+  }                                                                                        \
+  __device__ static T fetch_or(rocshmem_ctx_t c, T *d, T v, int pe) {                      \
+    return rocshmem_ctx_##TN##_atomic_fetch_or(c, d, v, pe);                               \
+  }                                                                                        \
+  __device__ static T fetch_xor(rocshmem_ctx_t c, T *d, T v, int pe) {                     \
+    return rocshmem_ctx_##TN##_atomic_fetch_xor(c, d, v, pe);                              \
+  }
+#define DRV_NO_STD(T)                                                                      \
+  __device__ static T fetch_add(rocshmem_ctx_t, T *, T, int) { return zero_of<T>(); }               \
+  __device__ static void add(rocshmem_ctx_t, T *, T, int) {}                               \
+  __device__ static T fetch_inc(rocshmem_ctx_t, T *, int) { return zero_of<T>(); }                  \
+  __device__ static void inc(rocshmem_ctx_t, T *, int) {}                                  \
+  __device__ static T compare_swap(rocshmem_ctx_t, T *, T, T, int) { return zero_of<T>(); }
+#define DRV_NO_BIT(T)                                                                      \
+  __device__ static T fetch_and(rocshmem_ctx_t, T *, T, int) { return zero_of<T>(); }               \
+  __device__ static T fetch_or(rocshmem_ctx_t, T *, T, int) { return zero_of<T>(); }                \
+  __device__ static T fetch_xor(rocshmem_ctx_t, T *, T, int) { return zero_of<T>(); }
+
+template <> struct PublicAmo<int> {
+  static constexpr bool kStd = true, kBit = false;
+  DRV_AMO_STD(int, int) DRV_AMO_EXT(int, int) DRV_NO_BIT(int)
+};
+template <> struct PublicAmo<long> {
+  static constexpr bool kStd = true, kBit = false;
+  DRV_AMO_STD(long, long) DRV_AMO_EXT(long, long) DRV_NO_BIT(long)
+};
+template <> struct PublicAmo<long long> {
+  static constexpr bool kStd = true, kBit = false;
+  DRV_AMO_STD(long long, longlong) DRV_AMO_EXT(long long, longlong) DRV_NO_BIT(long long)
+};
+template <> struct PublicAmo<unsigned int> {
+  static constexpr bool kStd = true, kBit = true;
+  DRV_AMO_STD(unsigned int, uint) DRV_AMO_EXT(unsigned int, uint) DRV_AMO_BIT(unsigned int, uint)
+};
+template <> struct PublicAmo<unsigned long> {
+  static constexpr bool kStd = true, kBit = true;
+  DRV_AMO_STD(unsigned long, ulong) DRV_AMO_EXT(unsigned long, ulong) DRV_AMO_BIT(unsigned long, ulong)
+};
+template <> struct PublicAmo<unsigned long long> {
+  static constexpr bool kStd = true, kBit = true;
+  DRV_AMO_STD(unsigned long long, ulonglong) DRV_AMO_EXT(unsigned long long, ulonglong)
+  DRV_AMO_BIT(unsigned long long, ulonglong)
+};
+template <> struct PublicAmo<float> {
+  static constexpr bool kStd = false, kBit = false;
+  DRV_NO_STD(float) DRV_AMO_EXT(float, float) DRV_NO_BIT(float)
+};
+template <> struct PublicAmo<double> {
+  static constexpr bool kStd = false, kBit = false;
+  DRV_NO_STD(double) DRV_AMO_EXT(double, double) DRV_NO_BIT(double)
+};
+
+template <typename T, int kAmo>
+__global__ void amo_kernel(AmoArgs<T> a) {
+  using P = PublicAmo<T>;
+  const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < a.n_ops;
+       i += stride) {
+    const uint32_t id = a.ids[i];
+    const int pe = static_cast<int>(id / a.n_slots);
+    T *target = a.counters + (id % a.n_slots);
+    const T v = a.values ? a.values[i] : static_cast<T>(1);
+    T out = zero_of<T>();
+    if constexpr (kAmo == ROCSHMEM_AMD_AMO_FETCH_ADD) out = P::fetch_add(a.ctx, target, v, pe);
+    else if constexpr (kAmo == ROCSHMEM_AMD_AMO_ADD) P::add(a.ctx, target, v, pe);
+    else if constexpr (kAmo == ROCSHMEM_AMD_AMO_FETCH_INC) out = P::fetch_inc(a.ctx, target, pe);
+    else if constexpr (kAmo == ROCSHMEM_AMD_AMO_INC) P::inc(a.ctx, target, pe);
+    else if constexpr (kAmo == ROCSHMEM_AMD_AMO_COMPARE_SWAP)
+      out = P::compare_swap(a.ctx, target, a.conds[i], v, pe);
+    else if constexpr (kAmo == ROCSHMEM_AMD_AMO_FETCH) out = P::fetch(a.ctx, target, pe);
+    else if constexpr (kAmo == ROCSHMEM_AMD_AMO_SET) P::set(a.ctx, target, v, pe);
+    else if constexpr (kAmo == ROCSHMEM_AMD_AMO_SWAP) out = P::swap(a.ctx, target, v, pe);
+    else if constexpr (kAmo == ROCSHMEM_AMD_AMO_FETCH_AND) out = P::fetch_and(a.ctx, target, v, pe);
+    else if constexpr (kAmo == ROCSHMEM_AMD_AMO_FETCH_OR) out = P::fetch_or(a.ctx, target, v, pe);
+    else out = P::fetch_xor(a.ctx, target, v, pe);
+    if (a.fetched) a.fetched[i] = out;
+  }
+}
+
+template <typename T>
+int launch_amo(int amo_op, const AmoArgs<T> &a, int n_wgs, int wg_size, hipStream_t s) {
+  using P = PublicAmo<T>;
+  const dim3 g(n_wgs), b(wg_size);
+  const bool std_op = amo_op <= ROCSHMEM_AMD_AMO_COMPARE_SWAP;
+  const bool bit_op = amo_op >= ROCSHMEM_AMD_AMO_FETCH_AND;
+  if ((std_op && !P::kStd) || (bit_op && !P::kBit)) return -1;
+  switch (amo_op) {
+#define DRV_AMO_CASE(OP) \
+  case OP: hipLaunchKernelGGL((amo_kernel<T, OP>), g, b, 0, s, a); break;
+    DRV_AMO_CASE(ROCSHMEM_AMD_AMO_FETCH_ADD)
+    DRV_AMO_CASE(ROCSHMEM_AMD_AMO_ADD)
+    DRV_AMO_CASE(ROCSHMEM_AMD_AMO_FETCH_INC)
+    DRV_AMO_CASE(ROCSHMEM_AMD_AMO_INC)
+    DRV_AMO_CASE(ROCSHMEM_AMD_AMO_COMPARE_SWAP)
+    DRV_AMO_CASE(ROCSHMEM_AMD_AMO_FETCH)
+    DRV_AMO_CASE(ROCSHMEM_AMD_AMO_SET)
+    DRV_AMO_CASE(ROCSHMEM_AMD_AMO_SWAP)
+    DRV_AMO_CASE(ROCSHMEM_AMD_AMO_FETCH_AND)
+    DRV_AMO_CASE(ROCSHMEM_AMD_AMO_FETCH_OR)
+    DRV_AMO_CASE(ROCSHMEM_AMD_AMO_FETCH_XOR)
+#undef DRV_AMO_CASE
+    default: return -1;
+  }
+  DRV_CHECK_HIP(hipGetLastError());
+  return 0;
+}
+
+// ---------------------------------------------------------------------------
+// put-with-signal
+// ---------------------------------------------------------------------------
+struct SignalArgs {
+  char *dest;
+  const char *source;
+  size_t nbytes;
+  size_t tile;
+  uint64_t *sig_addr;
+  uint64_t signal;
+  int sig_op;
+  rocshmem_ctx_t ctx;
+  int pe;
+  int calls;
+};
+
+template <int kGran>
+__global__ void put_signal_kernel(SignalArgs a) {
+  size_t group;
+  const size_t tid = threadIdx.x, bs = blockDim.x;
+  if constexpr (kGran == ROCSHMEM_AMD_WG) group = blockIdx.x;
+  else if constexpr (kGran == ROCSHMEM_AMD_WAVE) group = blockIdx.x * ((bs + 63) / 64) + tid / 64;
+  else group = blockIdx.x * bs + tid;
+  const size_t off = group * a.tile;
+  // A group whose tile starts past the end has nothing to send: a zero-length
+  // call, which leaves the signal untouched.
+  const size_t len = off >= a.nbytes ? 0 : (a.nbytes - off < a.tile ? a.nbytes - off : a.tile);
+  for (int k = 0; k < a.calls; ++k) {
+    if constexpr (kGran == ROCSHMEM_AMD_WG)
+      rocshmem_ctx_putmem_signal_wg(a.ctx, a.dest + off, a.source + off, len, a.sig_addr,
+                                    a.signal, a.sig_op, a.pe);
+    else if constexpr (kGran == ROCSHMEM_AMD_WAVE)
+      rocshmem_ctx_putmem_signal_wave(a.ctx, a.dest + off, a.source + off, len, a.sig_addr,
+                                      a.signal, a.sig_op, a.pe);
+    else
+      rocshmem_ctx_putmem_signal(a.ctx, a.dest + off, a.source + off, len, a.sig_addr,
+                                 a.signal, a.sig_op, a.pe);
+  }
+}
+
+template <int kGran>
+__global__ void signal_fetch_kernel(const uint64_t *sig, uint64_t *out) {
+  uint64_t v;
+  if constexpr (kGran == ROCSHMEM_AMD_WG) v = rocshmem_signal_fetch_wg(sig);
+  else if constexpr (kGran == ROCSHMEM_AMD_WAVE) v = rocshmem_signal_fetch_wave(sig);
+  else v = rocshmem_signal_fetch(sig);
+  // Every thread must have received the value.
+  if (v != *reinterpret_cast<const volatile uint64_t *>(sig)) atomicAdd(reinterpret_cast<unsigned long long *>(out + 1), 1ull);
+  if (threadIdx.x == 0) out[0] = v;
+}
+
+// ---------------------------------------------------------------------------
+// ping-pong between two work-groups acting as two PEs
+// ---------------------------------------------------------------------------
+struct PingPongArgs {
+  char *buf_a;      // address on pe_a
+  uint64_t *sig_a;  // address on pe_a
+  size_t nbytes;
+  int iters;
+  int pe_a, pe_b;
+  uint64_t pe_stride;
+  detail::Context *ctx_row;
+  detail::Team *world_row;
+  unsigned long long *ticks;
+};
+
+__global__ void pingpong_kernel(PingPongArgs a) {
+  const bool is_a = blockIdx.x == 0;
+  const int me = is_a ? a.pe_a : a.pe_b;
+  const int peer = is_a ? a.pe_b : a.pe_a;
+  const int64_t shift = static_cast<int64_t>(me - a.pe_a) * static_cast<int64_t>(a.pe_stride);
+  char *buf = a.buf_a + shift;
+  uint64_t *sig = reinterpret_cast<uint64_t *>(reinterpret_cast<char *>(a.sig_a) + shift);
+  rocshmem_ctx_t ctx{a.ctx_row + me, &a.world_row[me].wrt_world};
+  const unsigned long long t0 = wall_clock64();
+  for (int r = 1; r <= a.iters; ++r) {
+    if (is_a) {
+      rocshmem_ctx_putmem_signal_wg(ctx, buf, buf, a.nbytes, sig, static_cast<uint64_t>(r),
+                                    ROCSHMEM_SIGNAL_SET, peer);
+      if (threadIdx.x == 0)
+        rocshmem_ulong_wait_until(reinterpret_cast<unsigned long *>(sig), ROCSHMEM_CMP_EQ,
+                                  static_cast<unsigned long>(r));
+      __syncthreads();
+    } else {
+      if (threadIdx.x == 0)
+        rocshmem_ulong_wait_until(reinterpret_cast<unsigned long *>(sig), ROCSHMEM_CMP_EQ,
+                                  static_cast<unsigned long>(r));
+      __syncthreads();
+      rocshmem_ctx_putmem_signal_wg(ctx, buf, buf, a.nbytes, sig, static_cast<uint64_t>(r),
+                                    ROCSHMEM_SIGNAL_SET, peer);
+    }
+  }
+  const unsigned long long t1 = wall_clock64();
+  if (is_a && threadIdx.x == 0) *a.ticks = t1 - t0;
+}
+
+// ---------------------------------------------------------------------------
+// MoE-style dispatch with put_signal
+// ---------------------------------------------------------------------------
+struct DispatchArgs {
+  char *recv0;          // addresses on PE 0
+  const char *send0;
+  uint64_t *sig0;
+  const uint32_t *count, *send_row, *recv_row;
+  size_t row_bytes;
+  uint64_t pe_stride;
+  int np;
+  int wgs_per_pair;
+  detail::Context *ctx_row;
+  detail::Team *world_row;
+};
+
+__global__ void dispatch_kernel(DispatchArgs a) {
+  const int P = a.np, W = a.wgs_per_pair;
+  const int senders = P * P * W;
+  const int b = blockIdx.x;
+  if (b < senders) {
+    const int w = b % W, pair = b / W;
+    const int d = pair % P, s = pair / P;
+    const uint32_t cnt = a.count[s * P + d];
+    // Rows of this pair are shared out over its W work-groups.
+    const uint32_t per = (cnt + W - 1) / W;
+    const uint32_t lo = per * w < cnt ? per * w : cnt;
+    const uint32_t hi = lo + per < cnt ? lo + per : cnt;
+    rocshmem_ctx_t ctx{a.ctx_row + s, &a.world_row[s].wrt_world};
+    char *recv_s = a.recv0 + static_cast<uint64_t>(s) * a.pe_stride;
+    const char *send_s = a.send0 + static_cast<uint64_t>(s) * a.pe_stride;
+    uint64_t *sig_s = reinterpret_cast<uint64_t *>(reinterpret_cast<char *>(a.sig0) +
+                                                   static_cast<uint64_t>(s) * a.pe_stride);
+    rocshmem_ctx_putmem_signal_wg(
+        ctx, recv_s + (static_cast<size_t>(a.recv_row[s * P + d]) + lo) * a.row_bytes,
+        send_s + (static_cast<size_t>(a.send_row[s * P + d]) + lo) * a.row_bytes,
+        static_cast<size_t>(hi - lo) * a.row_bytes, sig_s + s, static_cast<uint64_t>(hi - lo),
+        ROCSHMEM_SIGNAL_ADD, d);
+  } else {
+    const int d = b - senders;
+    uint64_t *sig_d = reinterpret_cast<uint64_t *>(reinterpret_cast<char *>(a.sig0) +
+                                                   static_cast<uint64_t>(d) * a.pe_stride);
+    // Lane s of the first wavefront waits for sender s.
+    for (int s = threadIdx.x; s < P; s += blockDim.x)
+      rocshmem_ulong_wait_until(reinterpret_cast<unsigned long *>(sig_d + s), ROCSHMEM_CMP_GE,
+                                static_cast<unsigned long>(a.count[s * P + d]));
+  }
+}
+
+// ---------------------------------------------------------------------------
+// wait / test
+// ---------------------------------------------------------------------------
+template <typename T>
+struct PublicWait;
+#define DRV_WAIT(T, TN)                                                                    \
+  template <>                                                                              \
+  struct PublicWait<T> {                                                                   \
+    __device__ static int test(T *p, int c, T v) { return rocshmem_##TN##_test(p, c, v); } \
+    __device__ static void wait(T *p, int c, T v) { rocshmem_##TN##_wait_until(p, c, v); } \
+    __device__ static size_t any(T *p, size_t n, const int *s, int c, T v) {               \
+      return rocshmem_##TN##_wait_until_any(p, n, s, c, v);                                \
+    }                                                                                      \
+    __device__ static void all(T *p, size_t n, const int *s, int c, T v) {                 \
+      rocshmem_##TN##_wait_until_all(p, n, s, c, v);                                       \
+    }                                                                                      \
+    __device__ static size_t some(T *p, size_t n, size_t *idx, const int *s, int c, T v) { \
+      return rocshmem_##TN##_wait_until_some(p, n, idx, s, c, v);                          \
+    }                                                                                      \
+  };
+DRV_WAIT(short, short)
+DRV_WAIT(int, int)
+DRV_WAIT(long, long)
+DRV_WAIT(long long, longlong)
+DRV_WAIT(float, float)
+DRV_WAIT(double, double)
+DRV_WAIT(unsigned int, uint)
+DRV_WAIT(unsigned long, ulong)
+DRV_WAIT(unsigned long long, ulonglong)
+
+template <typename T>
+struct WaitArgs {
+  int fn;
+  T *ivars;
+  size_t nelems;
+  const int *status;
+  int cmp;
+  T value;
+  size_t *ret;
+  size_t *indices;
+  // waker
+  int woken;
+  size_t wake_index;
+  T wake_value;
+  unsigned long long delay_ticks;
+};
+
+template <typename T>
+__global__ void wait_kernel(WaitArgs<T> a) {
+  using P = PublicWait<T>;
+  if (blockIdx.x == 0) {
+    if (threadIdx.x != 0) return;
+    size_t r = 0;
+    switch (a.fn) {
+      case ROCSHMEM_AMD_TEST: r = static_cast<size_t>(P::test(a.ivars, a.cmp, a.value)); break;
+      case ROCSHMEM_AMD_WAIT_UNTIL: P::wait(a.ivars, a.cmp, a.value); break;
+      case ROCSHMEM_AMD_WAIT_UNTIL_ANY: r = P::any(a.ivars, a.nelems, a.status, a.cmp, a.value); break;
+      case ROCSHMEM_AMD_WAIT_UNTIL_ALL: P::all(a.ivars, a.nelems, a.status, a.cmp, a.value); break;
+      default: r = P::some(a.ivars, a.nelems, a.indices, a.status, a.cmp, a.value); break;
+    }
+    *a.ret = r;
+  } else if (a.woken && threadIdx.x == 0) {
+    const unsigned long long t0 = wall_clock64();
+    while (wall_clock64() - t0 < a.delay_ticks) __builtin_amdgcn_s_sleep(8);
+    detail::amo_set(a.ivars + a.wake_index, a.wake_value);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// context lifecycle
+// ---------------------------------------------------------------------------
+struct CtxCycleArgs {
+  rocshmem_team_t team;  // may be null
+  int per_wg;
+  int *status, *pe, *npes;
+};
+
+__global__ void ctx_cycle_kernel(CtxCycleArgs a) {
+  constexpr int kMaxPerWg = 64;
+  __shared__ rocshmem_ctx_t ctxs[kMaxPerWg];
+  rocshmem_wg_init();
+  for (int k = 0; k < a.per_wg; ++k) {
+    int rc;
+    if (a.team) rc = rocshmem_wg_team_create_ctx(a.team, 0, &ctxs[k]);
+    else rc = rocshmem_wg_ctx_create(0, &ctxs[k]);
+    if (threadIdx.x == 0) {
+      const int slot = blockIdx.x * a.per_wg + k;
+      a.status[slot] = rc;
+      a.pe[slot] = rc == 0 ? rocshmem_ctx_my_pe(ctxs[k]) : -2;
+      a.npes[slot] = rc == 0 ? rocshmem_ctx_n_pes(ctxs[k]) : -2;
+    }
+  }
+  __syncthreads();
+  for (int k = 0; k < a.per_wg; ++k) {
+    if (ctxs[k].ctx_opaque) rocshmem_wg_ctx_destroy(&ctxs[k]);
+  }
+  rocshmem_wg_finalize();
+}
+
+template <typename Fn>
+bool for_amo_dtype(int dtype, Fn &&fn) {
+  switch (dtype) {
+    case ROCSHMEM_AMD_INT: fn(static_cast<int *>(nullptr)); return true;
+    case ROCSHMEM_AMD_LONG: fn(static_cast<long *>(nullptr)); return true;
+    case ROCSHMEM_AMD_LONGLONG: fn(static_cast<long long *>(nullptr)); return true;
+    case ROCSHMEM_AMD_UINT: fn(static_cast<unsigned int *>(nullptr)); return true;
+    case ROCSHMEM_AMD_ULONG: fn(static_cast<unsigned long *>(nullptr)); return true;
+    case ROCSHMEM_AMD_ULONGLONG: fn(static_cast<unsigned long long *>(nullptr)); return true;
+    case ROCSHMEM_AMD_FLOAT: fn(static_cast<float *>(nullptr)); return true;
+    case ROCSHMEM_AMD_DOUBLE: fn(static_cast<double *>(nullptr)); return true;
+    default: return false;
+  }
+}
+template <typename Fn>
+bool for_wait_dtype(int dtype, Fn &&fn) {
+  if (dtype == ROCSHMEM_AMD_SHORT) {
+    fn(static_cast<short *>(nullptr));
+    return true;
+  }
+  return for_amo_dtype(dtype, fn);
+}
+
+template <typename T>
+int run_wait(int wait_fn, void *ivars, size_t nelems, const int *status, int cmp,
+             const void *value, int woken, size_t wake_index, const void *wake_value,
+             uint64_t delay_ticks, size_t *ret_out, size_t *indices_out) {
+  WaitArgs<T> a;
+  a.fn = wait_fn;
+  a.ivars = static_cast<T *>(ivars);
+  a.nelems = nelems;
+  a.cmp = cmp;
+  a.value = *static_cast<const T *>(value);
+  a.woken = woken;
+  a.wake_index = wake_index;
+  a.wake_value = woken ? *static_cast<const T *>(wake_value) : zero_of<T>();
+  a.delay_ticks = delay_ticks;
+  int *d_status = nullptr;
+  size_t *d_ret, *d_idx;
+  const size_t nidx = nelems ? nelems : 1;
+  if (status) {
+    DRV_CHECK_HIP(hipMalloc(&d_status, nidx * sizeof(int)));
+    DRV_CHECK_HIP(hipMemcpy(d_status, status, nelems * sizeof(int), hipMemcpyHostToDevice));
+  }
+  DRV_CHECK_HIP(hipMalloc(&d_ret, sizeof(size_t)));
+  DRV_CHECK_HIP(hipMalloc(&d_idx, nidx * sizeof(size_t)));
+  DRV_CHECK_HIP(hipMemset(d_ret, 0, sizeof(size_t)));
+  DRV_CHECK_HIP(hipMemset(d_idx, 0xff, nidx * sizeof(size_t)));
+  a.status = d_status;
+  a.ret = d_ret;
+  a.indices = d_idx;
+  hipLaunchKernelGGL(wait_kernel<T>, dim3(woken ? 2 : 1), dim3(64), 0, 0, a);
+  DRV_CHECK_HIP(hipGetLastError());
+  DRV_CHECK_HIP(hipDeviceSynchronize());
+  if (ret_out) DRV_CHECK_HIP(hipMemcpy(ret_out, d_ret, sizeof(size_t), hipMemcpyDeviceToHost));
+  if (indices_out && nelems)
+    DRV_CHECK_HIP(hipMemcpy(indices_out, d_idx, nelems * sizeof(size_t), hipMemcpyDeviceToHost));
+  if (d_status) DRV_CHECK_HIP(hipFree(d_status));
+  DRV_CHECK_HIP(hipFree(d_ret));
+  DRV_CHECK_HIP(hipFree(d_idx));
+  return 0;
+}
+
+}  // namespace drv
+}  // namespace rocshmem
+
+using namespace rocshmem;
+using namespace rocshmem::drv;
+
+extern "C" {
+
+int rocshmem_amd_amo(int amo_op, int dtype, void *counters, uint32_t n_slots,
+                     const uint32_t *ids, const void *values, const void *conds, void *fetched,
+                     size_t n_ops, int my_pe, int n_wgs, int wg_size,
+                     rocshmem_amd_stream_t stream) {
+  if (!valid_pe(my_pe) || !valid_launch(n_wgs, wg_size) || !n_slots || !ids) return -1;
+  if (amo_op == ROCSHMEM_AMD_AMO_COMPARE_SWAP && !conds) return -1;
+  int rc = -1;
+  const bool known = for_amo_dtype(dtype, [&](auto *tag) {
+    using T = typename std::remove_pointer<decltype(tag)>::type;
+    AmoArgs<T> a;
+    a.counters = static_cast<T *>(counters);
+    a.n_slots = n_slots;
+    a.ids = ids;
+    a.values = static_cast<const T *>(values);
+    a.conds = static_cast<const T *>(conds);
+    a.fetched = static_cast<T *>(fetched);
+    a.n_ops = n_ops;
+    a.ctx = runtime::rt().default_ctx_handle(my_pe);
+    rc = launch_amo<T>(amo_op, a, n_wgs, wg_size, as_stream(stream));
+  });
+  return known ? rc : -1;
+}
+
+int rocshmem_amd_put_signal(int gran, void *dest, const void *source, size_t nbytes,
+                            uint64_t *sig_addr, uint64_t signal, int sig_op, int my_pe, int pe,
+                            int n_wgs, int wg_size, int calls, rocshmem_amd_stream_t stream) {
+  if (!valid_pe(my_pe) || !valid_pe(pe) || !valid_launch(n_wgs, wg_size) || calls < 0) return -1;
+  if (gran < ROCSHMEM_AMD_THREAD || gran > ROCSHMEM_AMD_WG) return -1;
+  size_t groups = n_wgs;
+  if (gran == ROCSHMEM_AMD_WAVE) groups *= (wg_size + 63) / 64;
+  if (gran == ROCSHMEM_AMD_THREAD) groups *= wg_size;
+  SignalArgs a;
+  a.dest = static_cast<char *>(dest);
+  a.source = static_cast<const char *>(source);
+  a.nbytes = nbytes;
+  a.tile = auto_tile(nbytes, groups);
+  a.sig_addr = sig_addr;
+  a.signal = signal;
+  a.sig_op = sig_op;
+  a.ctx = runtime::rt().default_ctx_handle(my_pe);
+  a.pe = pe;
+  a.calls = calls;
+  hipStream_t s = as_stream(stream);
+  const dim3 g(n_wgs), b(wg_size);
+  if (gran == ROCSHMEM_AMD_WG) hipLaunchKernelGGL(put_signal_kernel<ROCSHMEM_AMD_WG>, g, b, 0, s, a);
+  else if (gran == ROCSHMEM_AMD_WAVE) hipLaunchKernelGGL(put_signal_kernel<ROCSHMEM_AMD_WAVE>, g, b, 0, s, a);
+  else hipLaunchKernelGGL(put_signal_kernel<ROCSHMEM_AMD_THREAD>, g, b, 0, s, a);
+  DRV_CHECK_HIP(hipGetLastError());
+  return 0;
+}
+
+int rocshmem_amd_signal_fetch(int gran, const uint64_t *sig_addr, int my_pe, uint64_t *value_out) {
+  if (!valid_pe(my_pe) || !value_out) return -1;
+  uint64_t *d_out;
+  DRV_CHECK_HIP(hipMalloc(&d_out, 2 * sizeof(uint64_t)));
+  DRV_CHECK_HIP(hipMemset(d_out, 0, 2 * sizeof(uint64_t)));
+  const dim3 g(1), b(gran == ROCSHMEM_AMD_THREAD ? 1 : (gran == ROCSHMEM_AMD_WAVE ? 64 : 256));
+  if (gran == ROCSHMEM_AMD_WG) hipLaunchKernelGGL(signal_fetch_kernel<ROCSHMEM_AMD_WG>, g, b, 0, 0, sig_addr, d_out);
+  else if (gran == ROCSHMEM_AMD_WAVE) hipLaunchKernelGGL(signal_fetch_kernel<ROCSHMEM_AMD_WAVE>, g, b, 0, 0, sig_addr, d_out);
+  else if (gran == ROCSHMEM_AMD_THREAD) hipLaunchKernelGGL(signal_fetch_kernel<ROCSHMEM_AMD_THREAD>, g, b, 0, 0, sig_addr, d_out);
+  else { DRV_CHECK_HIP(hipFree(d_out)); return -1; }
+  DRV_CHECK_HIP(hipGetLastError());
+  uint64_t out[2];
+  DRV_CHECK_HIP(hipMemcpy(out, d_out, sizeof(out), hipMemcpyDeviceToHost));
+  DRV_CHECK_HIP(hipFree(d_out));
+  *value_out = out[0];
+  return out[1] == 0 ? 0 : -2;
+}
+
+int rocshmem_amd_pingpong(void *buf, uint64_t *sig, size_t nbytes, int iters, int pe_a, int pe_b,
+                          int wg_size, uint64_t *ticks_out, double *tick_hz_out,
+                          rocshmem_amd_stream_t stream) {
+  if (!valid_pe(pe_a) || !valid_pe(pe_b) || pe_a == pe_b || !valid_launch(2, wg_size) ||
+      iters < 0 || nbytes == 0)
+    return -1;
+  auto &r = runtime::rt();
+  unsigned long long *d_ticks;
+  DRV_CHECK_HIP(hipMalloc(&d_ticks, sizeof(unsigned long long)));
+  DRV_CHECK_HIP(hipMemset(d_ticks, 0, sizeof(unsigned long long)));
+  PingPongArgs a;
+  a.buf_a = static_cast<char *>(buf);
+  a.sig_a = sig;
+  a.nbytes = nbytes;
+  a.iters = iters;
+  a.pe_a = pe_a;
+  a.pe_b = pe_b;
+  a.pe_stride = r.pe_stride;
+  a.ctx_row = r.d_default_ctx;
+  a.world_row = r.d_teams;
+  a.ticks = d_ticks;
+  hipStream_t s = as_stream(stream);
+  hipLaunchKernelGGL(pingpong_kernel, dim3(2), dim3(wg_size), 0, s, a);
+  DRV_CHECK_HIP(hipGetLastError());
+  DRV_CHECK_HIP(hipStreamSynchronize(s));
+  unsigned long long ticks = 0;
+  DRV_CHECK_HIP(hipMemcpy(&ticks, d_ticks, sizeof(ticks), hipMemcpyDeviceToHost));
+  DRV_CHECK_HIP(hipFree(d_ticks));
+  if (ticks_out) *ticks_out = ticks;
+  if (tick_hz_out) {
+    int khz = 0, dev = 0;
+    DRV_CHECK_HIP(hipGetDevice(&dev));
+    DRV_CHECK_HIP(hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev));
+    *tick_hz_out = static_cast<double>(khz) * 1e3;
+  }
+  return 0;
+}
+
+int rocshmem_amd_dispatch_put_signal(void *recv, const void *send, uint64_t *sig,
+                                     const uint32_t *count, const uint32_t *send_row,
+                                     const uint32_t *recv_row, size_t row_bytes,
+                                     int wgs_per_pair, int wg_size,
+                                     rocshmem_amd_stream_t stream) {
+  auto &r = runtime::rt();
+  if (!r.live || wgs_per_pair < 1 || !valid_launch(1, wg_size) || !row_bytes) return -1;
+  if (r.pe_of(recv) != 0 || r.pe_of(send) != 0 || r.pe_of(sig) != 0) return -1;
+  DispatchArgs a;
+  a.recv0 = static_cast<char *>(recv);
+  a.send0 = static_cast<const char *>(send);
+  a.sig0 = sig;
+  a.count = count;
+  a.send_row = send_row;
+  a.recv_row = recv_row;
+  a.row_bytes = row_bytes;
+  a.pe_stride = r.pe_stride;
+  a.np = r.npes;
+  a.wgs_per_pair = wgs_per_pair;
+  a.ctx_row = r.d_default_ctx;
+  a.world_row = r.d_teams;
+  const int grid = r.npes * r.npes * wgs_per_pair + r.npes;
+  hipLaunchKernelGGL(dispatch_kernel, dim3(grid), dim3(wg_size), 0, as_stream(stream), a);
+  DRV_CHECK_HIP(hipGetLastError());
+  return 0;
+}
+
+int rocshmem_amd_wait_test(int wait_fn, int dtype, void *ivars, size_t nelems, const int *status,
+                           int cmp, const void *value, size_t *ret_out, size_t *indices_out) {
+  if (!runtime::rt().live || !ivars || !value) return -1;
+  if (wait_fn < ROCSHMEM_AMD_TEST || wait_fn > ROCSHMEM_AMD_WAIT_UNTIL_SOME) return -1;
+  int rc = -1;
+  const bool known = for_wait_dtype(dtype, [&](auto *tag) {
+    using T = typename std::remove_pointer<decltype(tag)>::type;
+    rc = run_wait<T>(wait_fn, ivars, nelems, status, cmp, value, 0, 0, nullptr, 0, ret_out,
+                     indices_out);
+  });
+  return known ? rc : -1;
+}
+
+int rocshmem_amd_wait_test_woken(int wait_fn, int dtype, void *ivars, size_t nelems,
+                                 const int *status, int cmp, const void *value,
+                                 size_t wake_index, const void *wake_value,
+                                 uint64_t delay_ticks, size_t *ret_out, size_t *indices_out) {
+  if (!runtime::rt().live || !ivars || !value || !wake_value) return -1;
+  if (wait_fn < ROCSHMEM_AMD_WAIT_UNTIL || wait_fn > ROCSHMEM_AMD_WAIT_UNTIL_SOME) return -1;
+  if (wake_index >= (nelems ? nelems : 1)) return -1;
+  int rc = -1;
+  const bool known = for_wait_dtype(dtype, [&](auto *tag) {
+    using T = typename std::remove_pointer<decltype(tag)>::type;
+    rc = run_wait<T>(wait_fn, ivars, nelems, status, cmp, value, 1, wake_index, wake_value,
+                     delay_ticks, ret_out, indices_out);
+  });
+  return known ? rc : -1;
+}
+
+int rocshmem_amd_ctx_cycle(rocshmem_amd_team_t team, int n_wgs, int wg_size, int per_wg,
+                           int *status_out, int *pe_out, int *npes_out) {
+  if (!runtime::rt().live || !valid_launch(n_wgs, wg_size) || per_wg < 1 || per_wg > 64)
+    return -1;
+  if (!status_out || !pe_out || !npes_out) return -1;
+  const size_t n = static_cast<size_t>(n_wgs) * per_wg;
+  int *d;
+  DRV_CHECK_HIP(hipMalloc(&d, 3 * n * sizeof(int)));
+  DRV_CHECK_HIP(hipMemset(d, 0xff, 3 * n * sizeof(int)));
+  CtxCycleArgs a{static_cast<rocshmem_team_t>(team), per_wg, d, d + n, d + 2 * n};
+  hipLaunchKernelGGL(ctx_cycle_kernel, dim3(n_wgs), dim3(wg_size), 0, 0, a);
+  DRV_CHECK_HIP(hipGetLastError());
+  DRV_CHECK_HIP(hipDeviceSynchronize());
+  DRV_CHECK_HIP(hipMemcpy(status_out, d, n * sizeof(int), hipMemcpyDeviceToHost));
+  DRV_CHECK_HIP(hipMemcpy(pe_out, d + n, n * sizeof(int), hipMemcpyDeviceToHost));
+  DRV_CHECK_HIP(hipMemcpy(npes_out, d + 2 * n, n * sizeof(int), hipMemcpyDeviceToHost));
+  DRV_CHECK_HIP(hipFree(d));
+  return 0;
+}
+
+}  // extern "C"

@@ -1,0 +1,445 @@
+// Host runtime: symmetric heap, PE slices, teams, context pools and the
+// work/sync area, for P processing elements hosted by one process on one GPU.
+//
+// Plays the part of the reference's rocshmem_init -> IPCBackend bring-up
+// (src/rocshmem.cpp:73-140, src/ipc/backend_ipc.cpp:56-165,274-490) without
+// MPI or HIP IPC: there is one heap allocation of P slices at a fixed stride,
+// so the table of peer base addresses collapses to (base, stride).
+#include "runtime.hpp"
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <vector>
+
+#include "rocshmem/rocshmem.hpp"
+
+namespace rocshmem {
+
+rocshmem_team_t ROCSHMEM_TEAM_WORLD = ROCSHMEM_TEAM_INVALID;
+
+namespace runtime {
+
+#define RT_CHECK_HIP(expr)                                                        \
+  do {                                                                            \
+    hipError_t rt_err_ = (expr);                                                  \
+    if (rt_err_ != hipSuccess) {                                                  \
+      fprintf(stderr, "rocshmem: HIP error %d (%s) at %s:%d\n", (int)rt_err_,     \
+              hipGetErrorString(rt_err_), __FILE__, __LINE__);                    \
+      exit(EXIT_FAILURE);                                                         \
+    }                                                                             \
+  } while (0)
+
+namespace {
+
+std::vector<detail::StateUploader> &uploaders() {
+  static std::vector<detail::StateUploader> v;
+  return v;
+}
+
+Runtime g_rt;
+int g_requested_npes = 0;
+
+size_t env_size(const char *name, size_t fallback) {
+  const char *v = getenv(name);
+  if (!v || !*v) return fallback;
+  char *end = nullptr;
+  unsigned long long x = strtoull(v, &end, 10);
+  if (end == v) return fallback;
+  return static_cast<size_t>(x);
+}
+
+size_t round_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+int ilog2(int x) {
+  int l = 0;
+  while ((1 << (l + 1)) <= x) ++l;
+  return l;
+}
+
+}  // namespace
+
+Runtime &rt() { return g_rt; }
+
+void Runtime::push_state() {
+  for (auto fn : uploaders()) fn(&state);
+  RT_CHECK_HIP(hipDeviceSynchronize());
+}
+
+size_t Runtime::ws_bytes_per_pe() const {
+  // [world pad][per team: SYNC_KINDS pads + pWrk]
+  const size_t per_team = sizeof(detail::SyncPad) * detail::SYNC_KINDS +
+                          ROCSHMEM_REDUCE_MIN_WRKDATA_SIZE * sizeof(double);
+  return round_up(sizeof(detail::SyncPad) + per_team * max_teams, 4096);
+}
+
+detail::SyncPad *Runtime::team_pads(int pool_index, int pe) const {
+  const size_t per_team = sizeof(detail::SyncPad) * detail::SYNC_KINDS +
+                          ROCSHMEM_REDUCE_MIN_WRKDATA_SIZE * sizeof(double);
+  char *p = d_ws + static_cast<size_t>(pe) * ws_stride + sizeof(detail::SyncPad) +
+            per_team * pool_index;
+  return reinterpret_cast<detail::SyncPad *>(p);
+}
+
+void Runtime::write_team(int pool_index, int pe, const detail::TeamInfo &world,
+                         const detail::TeamInfo &parent, int my_pe_in_team) {
+  detail::Team t{};
+  t.wrt_world = world;
+  t.wrt_parent = parent;
+  t.my_pe = my_pe_in_team;
+  t.my_pe_in_world = pe;
+  t.num_pes = world.size;
+  t.world_size = npes;
+  t.pool_index = pool_index;
+  t.sync = team_pads(pool_index, pe);
+  t.pWrk = reinterpret_cast<char *>(t.sync) + sizeof(detail::SyncPad) * detail::SYNC_KINDS;
+  h_teams[static_cast<size_t>(pool_index) * npes + pe] = t;
+  RT_CHECK_HIP(hipMemcpy(d_teams + static_cast<size_t>(pool_index) * npes + pe, &t,
+                         sizeof(t), hipMemcpyHostToDevice));
+}
+
+int Runtime::init(int want_npes, size_t want_heap) {
+  if (live) return 0;
+  int ndev = 0;
+  if (hipGetDeviceCount(&ndev) != hipSuccess || ndev == 0) {
+    fprintf(stderr, "rocshmem: no GPU available\n");
+    abort();
+  }
+  npes = want_npes > 0 ? want_npes
+                       : (g_requested_npes > 0
+                              ? g_requested_npes
+                              : static_cast<int>(env_size("ROCSHMEM_EMU_NPES", 1)));
+  if (npes < 1 || npes > detail::SyncPad::kMaxPes) {
+    fprintf(stderr, "rocshmem: number of PEs must be in [1, %d]\n", detail::SyncPad::kMaxPes);
+    abort();
+  }
+  heap_size = want_heap ? want_heap : env_size("ROCSHMEM_HEAP_SIZE", size_t{1} << 30);
+  max_ctxs = static_cast<int>(env_size("ROCSHMEM_MAX_NUM_CONTEXTS", 1024));
+  if (max_ctxs > detail::CtxPool::kMaxWords * 64) max_ctxs = detail::CtxPool::kMaxWords * 64;
+  max_teams = static_cast<int>(env_size("ROCSHMEM_MAX_NUM_TEAMS", 40));
+  if (max_teams < 1) max_teams = 1;
+  // Slices start on 2 MiB boundaries; an optional pad staggers them further.
+  pe_stride = round_up(heap_size, size_t{2} << 20) + env_size("ROCSHMEM_EMU_SLICE_PAD", 0);
+  acting_pe = 0;
+
+  RT_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&heap_base), pe_stride * npes));
+  allocator.reset(reinterpret_cast<uint64_t>(heap_base), heap_size);
+
+  ws_stride = ws_bytes_per_pe();
+  RT_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&d_ws), ws_stride * npes));
+  RT_CHECK_HIP(hipMemset(d_ws, 0, ws_stride * npes));
+
+  // Teams: slot 0 is the world team.
+  h_teams.assign(static_cast<size_t>(max_teams) * npes, detail::Team{});
+  team_slot_used.assign(max_teams, false);
+  RT_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&d_teams),
+                         sizeof(detail::Team) * max_teams * npes));
+  RT_CHECK_HIP(hipMemset(d_teams, 0, sizeof(detail::Team) * max_teams * npes));
+  team_slot_used[0] = true;
+  num_user_teams = 0;
+  const detail::TeamInfo world{0, 1, npes, 0};
+  for (int pe = 0; pe < npes; ++pe) write_team(0, pe, world, world, pe);
+
+  // Contexts: one default context and one pool per PE.
+  auto fill_ctx = [&](detail::Context &c, int pe, int slot) {
+    c.heap_base = heap_base;
+    c.pe_stride = pe_stride;
+    c.ws_stride = ws_stride;
+    c.my_pe = pe;
+    c.num_pes = npes;
+    c.tinfo = &d_teams[pe].wrt_world;
+    c.world_sync = reinterpret_cast<detail::SyncPad *>(d_ws + static_cast<size_t>(pe) * ws_stride);
+    c.options = 0;
+    c.pool_slot = slot;
+  };
+  std::vector<detail::Context> ctxs(npes);
+  for (int pe = 0; pe < npes; ++pe) fill_ctx(ctxs[pe], pe, -1);
+  RT_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&d_default_ctx), sizeof(detail::Context) * npes));
+  RT_CHECK_HIP(hipMemcpy(d_default_ctx, ctxs.data(), sizeof(detail::Context) * npes,
+                         hipMemcpyHostToDevice));
+
+  RT_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&d_ctx_slots),
+                         sizeof(detail::Context) * max_ctxs * npes));
+  RT_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&d_pools), sizeof(detail::CtxPool) * npes));
+  std::vector<detail::Context> slots(static_cast<size_t>(max_ctxs) * npes);
+  std::vector<detail::CtxPool> pools(npes);
+  for (int pe = 0; pe < npes; ++pe) {
+    for (int s = 0; s < max_ctxs; ++s) fill_ctx(slots[static_cast<size_t>(pe) * max_ctxs + s], pe, s);
+    detail::CtxPool &p = pools[pe];
+    memset(&p, 0, sizeof(p));
+    for (int s = 0; s < max_ctxs; ++s) p.free_mask[s >> 6] |= 1ull << (s & 63);
+    p.capacity = max_ctxs;
+    p.slots = d_ctx_slots + static_cast<size_t>(pe) * max_ctxs;
+  }
+  RT_CHECK_HIP(hipMemcpy(d_ctx_slots, slots.data(), sizeof(detail::Context) * slots.size(),
+                         hipMemcpyHostToDevice));
+  RT_CHECK_HIP(hipMemcpy(d_pools, pools.data(), sizeof(detail::CtxPool) * npes,
+                         hipMemcpyHostToDevice));
+
+  state.heap_base = heap_base;
+  state.pe_stride = pe_stride;
+  state.heap_size = heap_size;
+  state.ws_stride = ws_stride;
+  state.n_pes = npes;
+  state.pe_rule = detail::PE_RULE_FIXED;
+  state.fixed_pe = 0;
+  state.max_teams = max_teams;
+  state.default_ctx = d_default_ctx;
+  state.world_team = d_teams;
+  state.ctx_pool = d_pools;
+  state.ws_base = d_ws;
+  state.nt_bytes = env_size("ROCSHMEM_NT_THRESHOLD", size_t{1} << 20);
+  live = true;
+  push_state();
+  ROCSHMEM_TEAM_WORLD = team_handle(0, acting_pe);
+  return 0;
+}
+
+void Runtime::finalize() {
+  if (!live) return;
+  RT_CHECK_HIP(hipDeviceSynchronize());
+  RT_CHECK_HIP(hipFree(d_pools));
+  RT_CHECK_HIP(hipFree(d_ctx_slots));
+  RT_CHECK_HIP(hipFree(d_default_ctx));
+  RT_CHECK_HIP(hipFree(d_teams));
+  RT_CHECK_HIP(hipFree(d_ws));
+  RT_CHECK_HIP(hipFree(heap_base));
+  heap_base = nullptr;
+  d_ws = nullptr;
+  d_teams = nullptr;
+  h_teams.clear();
+  team_slot_used.clear();
+  live = false;
+  memset(&state, 0, sizeof(state));
+  ROCSHMEM_TEAM_WORLD = ROCSHMEM_TEAM_INVALID;
+}
+
+void Runtime::require_live(const char *what) const {
+  if (!live) {
+    fprintf(stderr, "rocshmem: %s called before rocshmem_init\n", what);
+    abort();
+  }
+}
+
+rocshmem_team_t Runtime::team_handle(int pool_index, int pe) const {
+  return reinterpret_cast<rocshmem_team_t>(d_teams + static_cast<size_t>(pool_index) * npes + pe);
+}
+
+const detail::Team *Runtime::host_team(rocshmem_team_t team) const {
+  if (team == ROCSHMEM_TEAM_INVALID || !live) return nullptr;
+  const detail::Team *p = reinterpret_cast<const detail::Team *>(team);
+  if (p < d_teams || p >= d_teams + static_cast<size_t>(max_teams) * npes) return nullptr;
+  const size_t idx = static_cast<size_t>(p - d_teams);
+  if (!team_slot_used[idx / npes]) return nullptr;
+  return &h_teams[idx];
+}
+
+void *Runtime::sym_malloc(size_t size) {
+  require_live("rocshmem_malloc");
+  const uint64_t off = allocator.alloc(size);
+  if (off == Pow2Allocator::kNoBlock) return nullptr;
+  return heap_base + static_cast<size_t>(acting_pe) * pe_stride + off;
+}
+
+void Runtime::sym_free(void *ptr) {
+  require_live("rocshmem_free");
+  if (!ptr) return;
+  const uint64_t off = offset_of(ptr);
+  if (off == Pow2Allocator::kNoBlock || !allocator.free(off)) {
+    fprintf(stderr, "rocshmem: rocshmem_free of an address that was not allocated\n");
+    abort();
+  }
+}
+
+uint64_t Runtime::offset_of(const void *ptr) const {
+  const char *p = static_cast<const char *>(ptr);
+  if (p < heap_base || p >= heap_base + pe_stride * npes) return Pow2Allocator::kNoBlock;
+  return static_cast<uint64_t>(p - heap_base) % pe_stride;
+}
+
+int Runtime::pe_of(const void *ptr) const {
+  const char *p = static_cast<const char *>(ptr);
+  if (p < heap_base || p >= heap_base + pe_stride * npes) return -1;
+  return static_cast<int>(static_cast<uint64_t>(p - heap_base) / pe_stride);
+}
+
+void *Runtime::pe_ptr(const void *ptr, int pe) const {
+  const uint64_t off = offset_of(ptr);
+  if (off == Pow2Allocator::kNoBlock || pe < 0 || pe >= npes) return nullptr;
+  return heap_base + static_cast<size_t>(pe) * pe_stride + off;
+}
+
+// src/rocshmem.cpp:221-303.  One call creates the team object of every member.
+int Runtime::team_split_strided(rocshmem_team_t parent, int start, int stride, int size,
+                                rocshmem_team_t *new_team) {
+  require_live("rocshmem_team_split_strided");
+  *new_team = ROCSHMEM_TEAM_INVALID;
+  if (num_user_teams >= max_teams - 1) return -1;
+  if (parent == ROCSHMEM_TEAM_INVALID) return 0;
+  const detail::Team *pt = host_team(parent);
+  if (!pt) return -1;
+  if (start < 0 || start >= pt->num_pes || size < 1 || size > pt->num_pes || stride < 1)
+    return -1;
+  const int start_world = pt->wrt_world.pe_start + pt->wrt_world.stride * start;
+  const int stride_world = stride * pt->wrt_world.stride;
+  const int end_world = start_world + stride_world * (size - 1);
+  // The reference compares with '>' (src/rocshmem.cpp:253-255), which lets a
+  // team end one past the last PE; every member must exist here.
+  if (end_world >= npes) return -1;
+
+  int slot = -1;
+  for (int i = 1; i < max_teams; ++i)
+    if (!team_slot_used[i]) { slot = i; break; }
+  if (slot < 0) return -1;
+  team_slot_used[slot] = true;
+  ++num_user_teams;
+
+  // Fresh sync pads for the new team on every PE.
+  const size_t pad_bytes = sizeof(detail::SyncPad) * detail::SYNC_KINDS;
+  for (int pe = 0; pe < npes; ++pe) RT_CHECK_HIP(hipMemset(team_pads(slot, pe), 0, pad_bytes));
+
+  const detail::TeamInfo world{start_world, stride_world, size, ilog2(stride_world)};
+  const detail::TeamInfo wrt_parent{start, stride, size, ilog2(stride)};
+  for (int pe = 0; pe < npes; ++pe) {
+    const int off = pe - start_world;
+    int mine = -1;
+    if (off >= 0 && off % stride_world == 0 && off / stride_world < size) mine = off / stride_world;
+    write_team(slot, pe, world, wrt_parent, mine);
+  }
+  RT_CHECK_HIP(hipDeviceSynchronize());
+  if (h_teams[static_cast<size_t>(slot) * npes + acting_pe].my_pe >= 0)
+    *new_team = team_handle(slot, acting_pe);
+  last_created_slot = slot;
+  return 0;
+}
+
+void Runtime::team_destroy(rocshmem_team_t team) {
+  if (team == ROCSHMEM_TEAM_INVALID || !live) return;
+  const detail::Team *t = host_team(team);
+  if (!t || t->pool_index == 0) return;
+  team_slot_used[t->pool_index] = false;
+  --num_user_teams;
+}
+
+rocshmem_team_t Runtime::team_on(rocshmem_team_t team, int pe) const {
+  const detail::Team *t = host_team(team);
+  if (!t || pe < 0 || pe >= npes) return ROCSHMEM_TEAM_INVALID;
+  if (h_teams[static_cast<size_t>(t->pool_index) * npes + pe].my_pe < 0) return ROCSHMEM_TEAM_INVALID;
+  return team_handle(t->pool_index, pe);
+}
+
+void Runtime::set_pe(int pe) {
+  require_live("rocshmem_emu_set_pe");
+  if (pe < 0 || pe >= npes) {
+    fprintf(stderr, "rocshmem: PE %d out of range\n", pe);
+    abort();
+  }
+  acting_pe = pe;
+  ROCSHMEM_TEAM_WORLD = team_handle(0, pe);
+  if (state.fixed_pe != pe) {
+    state.fixed_pe = pe;
+    push_state();
+  }
+}
+
+void Runtime::set_pe_rule(int rule) {
+  require_live("rocshmem_emu_set_pe_rule");
+  if (rule < detail::PE_RULE_FIXED || rule > detail::PE_RULE_BLOCK_Z) {
+    fprintf(stderr, "rocshmem: unknown PE rule %d\n", rule);
+    abort();
+  }
+  if (state.pe_rule != rule) {
+    state.pe_rule = rule;
+    push_state();
+  }
+}
+
+}  // namespace runtime
+
+namespace detail {
+void register_state_uploader(StateUploader fn) {
+  runtime::uploaders().push_back(fn);
+  if (runtime::rt().live) fn(&runtime::rt().state);
+}
+}  // namespace detail
+
+// ============================ public host API ===============================
+using runtime::rt;
+
+__host__ void rocshmem_init(MPI_Comm) { rt().init(0, 0); }
+__host__ void rocshmem_init_thread(int, int *provided, MPI_Comm) {
+  rt().init(0, 0);
+  rocshmem_query_thread(provided);
+}
+__host__ void rocshmem_query_thread(int *provided) { *provided = ROCSHMEM_THREAD_MULTIPLE; }
+__host__ void rocshmem_dump_stats() {}
+__host__ void rocshmem_reset_stats() {}
+__host__ void rocshmem_finalize() { rt().finalize(); }
+__host__ void *rocshmem_malloc(size_t size) { return rt().sym_malloc(size); }
+__host__ void rocshmem_free(void *ptr) { rt().sym_free(ptr); }
+// Usable before rocshmem_init, as in the reference (src/rocshmem.cpp:113-121).
+__host__ int rocshmem_n_pes() {
+  if (rt().live) return rt().npes;
+  if (runtime::g_requested_npes > 0) return runtime::g_requested_npes;
+  return static_cast<int>(runtime::env_size("ROCSHMEM_EMU_NPES", 1));
+}
+__host__ int rocshmem_my_pe() { return rt().live ? rt().acting_pe : 0; }
+__host__ int rocshmem_ctx_create(int64_t, rocshmem_ctx_t *ctx) {
+  rt().require_live("rocshmem_ctx_create");
+  ctx->ctx_opaque = rt().d_default_ctx + rt().acting_pe;
+  ctx->team_opaque = &rt().d_teams[rt().acting_pe].wrt_world;
+  return 0;
+}
+__host__ void rocshmem_ctx_destroy(rocshmem_ctx_t) {}
+
+// src/team.cpp:51-111
+__host__ int rocshmem_team_translate_pe(rocshmem_team_t src_team, int src_pe,
+                                        rocshmem_team_t dest_team) {
+  const detail::Team *s = rt().host_team(src_team);
+  const detail::Team *d = rt().host_team(dest_team);
+  if (!s || !d) return -1;
+  const int world = s->wrt_world.pe_start + s->wrt_world.stride * src_pe;
+  const int off = world - d->wrt_world.pe_start;
+  if (off < 0 || off % d->wrt_world.stride) return -1;
+  const int rel = off / d->wrt_world.stride;
+  return rel >= d->num_pes ? -1 : rel;
+}
+__host__ int rocshmem_team_n_pes(rocshmem_team_t team) {
+  const detail::Team *t = rt().host_team(team);
+  return t ? t->num_pes : -1;
+}
+__host__ int rocshmem_team_my_pe(rocshmem_team_t team) {
+  const detail::Team *t = rt().host_team(team);
+  return t ? t->my_pe : -1;
+}
+__host__ int rocshmem_team_split_strided(rocshmem_team_t parent_team, int start, int stride,
+                                         int size, const rocshmem_team_config_t *, long,
+                                         rocshmem_team_t *new_team) {
+  return rt().team_split_strided(parent_team, start, stride, size, new_team);
+}
+__host__ void rocshmem_team_destroy(rocshmem_team_t team) {
+  if (team == ROCSHMEM_TEAM_WORLD) return;
+  rt().team_destroy(team);
+}
+// With every PE in this process, host-side ordering and barriers reduce to
+// draining the device.
+__host__ void rocshmem_ctx_fence(rocshmem_ctx_t) { RT_CHECK_HIP(hipDeviceSynchronize()); }
+__host__ void rocshmem_fence() { RT_CHECK_HIP(hipDeviceSynchronize()); }
+__host__ void rocshmem_ctx_quiet(rocshmem_ctx_t) { RT_CHECK_HIP(hipDeviceSynchronize()); }
+__host__ void rocshmem_quiet() { RT_CHECK_HIP(hipDeviceSynchronize()); }
+__host__ void rocshmem_barrier_all() { RT_CHECK_HIP(hipDeviceSynchronize()); }
+__host__ void rocshmem_sync_all() { RT_CHECK_HIP(hipDeviceSynchronize()); }
+__host__ void rocshmem_global_exit(int status) { exit(status); }
+
+void rocshmem_emu_set_npes(int npes) { runtime::g_requested_npes = npes; }
+void rocshmem_emu_set_pe(int pe) { rt().set_pe(pe); }
+void rocshmem_emu_set_pe_rule(int rule) { rt().set_pe_rule(rule); }
+void *rocshmem_emu_pe_ptr(const void *ptr, int pe) { return rt().pe_ptr(ptr, pe); }
+rocshmem_team_t rocshmem_emu_team_on(rocshmem_team_t team, int pe) { return rt().team_on(team, pe); }
+size_t rocshmem_emu_pe_stride() { return rt().pe_stride; }
+
+}  // namespace rocshmem

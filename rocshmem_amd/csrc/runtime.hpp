@@ -1,0 +1,77 @@
+// Host-side runtime object shared by the C++ host API, the C entry points and
+// the kernel launchers.
+#ifndef ROCSHMEM_AMD_RUNTIME_HPP_
+#define ROCSHMEM_AMD_RUNTIME_HPP_
+
+#include <cstddef>
+#include <cstdint>
+#include <vector>
+
+#include "pow2_allocator.hpp"
+#include "rocshmem/detail/state.hpp"
+
+namespace rocshmem {
+namespace runtime {
+
+struct Runtime {
+  bool live = false;
+  int npes = 0;
+  int acting_pe = 0;
+  int max_ctxs = 0;
+  int max_teams = 0;
+  int num_user_teams = 0;
+  int last_created_slot = -1;
+  size_t heap_size = 0;
+  size_t pe_stride = 0;
+  size_t ws_stride = 0;
+  char *heap_base = nullptr;
+  char *d_ws = nullptr;
+  detail::Team *d_teams = nullptr;         // [max_teams][npes]
+  detail::Context *d_default_ctx = nullptr;  // [npes]
+  detail::Context *d_ctx_slots = nullptr;  // [npes][max_ctxs]
+  detail::CtxPool *d_pools = nullptr;      // [npes]
+  std::vector<detail::Team> h_teams;       // host mirror of d_teams
+  std::vector<bool> team_slot_used;
+  Pow2Allocator allocator;
+  detail::DeviceState state{};
+
+  int init(int want_npes, size_t want_heap);
+  void finalize();
+  void require_live(const char *what) const;
+  void push_state();
+
+  void *sym_malloc(size_t size);
+  void sym_free(void *ptr);
+  uint64_t offset_of(const void *ptr) const;
+  int pe_of(const void *ptr) const;
+  void *pe_ptr(const void *ptr, int pe) const;
+
+  int team_split_strided(rocshmem_team_t parent, int start, int stride, int size,
+                         rocshmem_team_t *new_team);
+  void team_destroy(rocshmem_team_t team);
+  rocshmem_team_t team_handle(int pool_index, int pe) const;
+  rocshmem_team_t team_on(rocshmem_team_t team, int pe) const;
+  const detail::Team *host_team(rocshmem_team_t team) const;
+
+  void set_pe(int pe);
+  void set_pe_rule(int rule);
+
+  // Context handle of PE `pe` bound to its member object of team slot `slot`.
+  rocshmem_ctx_t default_ctx_handle(int pe, int slot = 0) const {
+    return rocshmem_ctx_t{d_default_ctx + pe,
+                          &d_teams[static_cast<size_t>(slot) * npes + pe].wrt_world};
+  }
+
+ private:
+  size_t ws_bytes_per_pe() const;
+  detail::SyncPad *team_pads(int pool_index, int pe) const;
+  void write_team(int pool_index, int pe, const detail::TeamInfo &world,
+                  const detail::TeamInfo &parent, int my_pe_in_team);
+};
+
+Runtime &rt();
+
+}  // namespace runtime
+}  // namespace rocshmem
+
+#endif  // ROCSHMEM_AMD_RUNTIME_HPP_
