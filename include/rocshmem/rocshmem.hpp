@@ -14,6 +14,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+
 #if __has_include(<mpi.h>) && !defined(ROCSHMEM_AMD_NO_MPI_HEADER)
 #include <mpi.h>
 #else
@@ -28,6 +30,11 @@ typedef int MPI_Comm;
 #ifndef MPI_COMM_NULL
 #define MPI_COMM_NULL (-1)
 #endif
+// Programs written for the reference end a failed run with MPI_Abort.
+static inline int MPI_Abort(MPI_Comm, int errorcode) {
+  exit(errorcode);
+  return 0;
+}
 #endif
 #endif
 

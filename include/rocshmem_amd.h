@@ -124,6 +124,19 @@ size_t rocshmem_amd_heap_used(void);
 size_t rocshmem_amd_heap_avail(void);
 size_t rocshmem_amd_pe_stride(void);
 
+/* The allocator on its own, usable without a GPU (planning and host-side
+ * tests): a model heap of heap_bytes whose base has the alignment of
+ * base_address.  Same algorithm as rocshmem_amd_malloc: SingleHeap / Pow2Bins
+ * (src/memory/single_heap.cpp:29-64, pow2_bins.hpp:90-152).  alloc returns the
+ * block's offset from the base, or UINT64_MAX for "nullptr". */
+void *rocshmem_amd_heap_model_create(uint64_t base_address, uint64_t heap_bytes);
+void rocshmem_amd_heap_model_destroy(void *model);
+uint64_t rocshmem_amd_heap_model_alloc(void *model, uint64_t size);
+int rocshmem_amd_heap_model_free(void *model, uint64_t offset);
+uint64_t rocshmem_amd_heap_model_used(void *model);
+uint64_t rocshmem_amd_heap_model_num_bins(void *model);
+uint64_t rocshmem_amd_heap_model_bin_population(void *model, uint64_t block_bytes);
+
 /* Teams (rocshmem.hpp:165-236; src/rocshmem.cpp:193-319, src/team.cpp:51-111). */
 rocshmem_amd_team_t rocshmem_amd_team_world(void);
 int rocshmem_amd_team_split_strided(rocshmem_amd_team_t parent, int start, int stride,

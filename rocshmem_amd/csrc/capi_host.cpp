@@ -44,6 +44,28 @@ size_t rocshmem_amd_heap_used(void) { return rt().allocator.used(); }
 size_t rocshmem_amd_heap_avail(void) { return rt().allocator.avail(); }
 size_t rocshmem_amd_pe_stride(void) { return rt().pe_stride; }
 
+void *rocshmem_amd_heap_model_create(uint64_t base_address, uint64_t heap_bytes) {
+  return new rocshmem::runtime::Pow2Allocator(base_address, heap_bytes);
+}
+void rocshmem_amd_heap_model_destroy(void *model) {
+  delete static_cast<rocshmem::runtime::Pow2Allocator *>(model);
+}
+uint64_t rocshmem_amd_heap_model_alloc(void *model, uint64_t size) {
+  return static_cast<rocshmem::runtime::Pow2Allocator *>(model)->alloc(size);
+}
+int rocshmem_amd_heap_model_free(void *model, uint64_t offset) {
+  return static_cast<rocshmem::runtime::Pow2Allocator *>(model)->free(offset) ? 0 : -1;
+}
+uint64_t rocshmem_amd_heap_model_used(void *model) {
+  return static_cast<rocshmem::runtime::Pow2Allocator *>(model)->used();
+}
+uint64_t rocshmem_amd_heap_model_num_bins(void *model) {
+  return static_cast<rocshmem::runtime::Pow2Allocator *>(model)->num_bins();
+}
+uint64_t rocshmem_amd_heap_model_bin_population(void *model, uint64_t block_bytes) {
+  return static_cast<rocshmem::runtime::Pow2Allocator *>(model)->bin_population(block_bytes);
+}
+
 rocshmem_amd_team_t rocshmem_amd_team_world(void) { return rocshmem::ROCSHMEM_TEAM_WORLD; }
 int rocshmem_amd_team_split_strided(rocshmem_amd_team_t parent, int start, int stride,
                                     int size, rocshmem_amd_team_t *new_team) {
@@ -83,14 +105,17 @@ int rocshmem_amd_dev_free(void *ptr) {
   return 0;
 }
 int rocshmem_amd_copy_in(void *dst_dev, const void *src_host, size_t n) {
+  if (n && (!dst_dev || !src_host)) return -1;
   if (n) DRV_CHECK_HIP(hipMemcpy(dst_dev, src_host, n, hipMemcpyHostToDevice));
   return 0;
 }
 int rocshmem_amd_copy_out(void *dst_host, const void *src_dev, size_t n) {
+  if (n && (!dst_host || !src_dev)) return -1;
   if (n) DRV_CHECK_HIP(hipMemcpy(dst_host, src_dev, n, hipMemcpyDeviceToHost));
   return 0;
 }
 int rocshmem_amd_fill(void *dst_dev, int byte, size_t n) {
+  if (n && !dst_dev) return -1;
   if (n) DRV_CHECK_HIP(hipMemset(dst_dev, byte, n));
   return 0;
 }

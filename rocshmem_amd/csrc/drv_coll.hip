@@ -387,7 +387,13 @@ int wg_move_common(int elem_size, rocshmem_amd_team_t team, void *dest, const vo
                    int nelems, int root, int wg_size, hipStream_t s) {
   TeamView v;
   if (!view_team(team, &v) || !valid_launch(1, wg_size) || nelems < 0) return -1;
-  if (!in_heap(dest) || !in_heap(source)) return -1;
+  {
+    const size_t blk = static_cast<size_t>(nelems) * elem_size;
+    const size_t all = blk * v.host->num_pes;
+    const int me = runtime::rt().acting_pe;
+    if (!sym_ok_on(dest, kMove == MOVE_BROADCAST ? blk : all, me)) return -1;
+    if (!sym_ok_on(source, kMove == MOVE_ALLTOALL ? all : blk, me)) return -1;
+  }
   if (kMove == MOVE_BROADCAST && (root < 0 || root >= v.host->num_pes)) return -1;
   const WgCollArgs a = make_wg_args(v, dest, source, nelems, root, nullptr);
   const dim3 g(v.host->num_pes), b(wg_size);
@@ -407,7 +413,12 @@ int grid_move_common(rocshmem_amd_team_t team, void *dest, const void *source, s
                      int root, hipStream_t s) {
   TeamView v;
   if (!view_team(team, &v)) return -1;
-  if (!in_heap(dest) || !in_heap(source)) return -1;
+  {
+    const size_t all = nbytes * v.host->num_pes;
+    const int me = runtime::rt().acting_pe;
+    if (!sym_ok_on(dest, kMove == MOVE_BROADCAST ? nbytes : all, me)) return -1;
+    if (!sym_ok_on(source, kMove == MOVE_ALLTOALL ? all : nbytes, me)) return -1;
+  }
   if (kMove == MOVE_BROADCAST && (root < 0 || root >= v.host->num_pes)) return -1;
   auto &r = runtime::rt();
   const int64_t first = static_cast<int64_t>(v.host->wrt_world.pe_start) * r.pe_stride;
@@ -426,7 +437,11 @@ int rocshmem_amd_wg_reduce(int dtype, int op, rocshmem_amd_team_t team, void *de
                            rocshmem_amd_stream_t stream) {
   TeamView v;
   if (!view_team(team, &v) || !valid_launch(1, wg_size) || nreduce < 0) return -1;
-  if (!in_heap(dest) || !in_heap(source)) return -1;
+  {
+    const size_t bytes = static_cast<size_t>(nreduce) * dtype_size(dtype);
+    const int me = runtime::rt().acting_pe;
+    if (!sym_ok_on(dest, bytes, me) || !sym_ok_on(source, bytes, me)) return -1;
+  }
   int *d_status;
   DRV_CHECK_HIP(hipMalloc(&d_status, sizeof(int)));
   DRV_CHECK_HIP(hipMemset(d_status, 0, sizeof(int)));
@@ -468,7 +483,7 @@ int rocshmem_amd_wg_fcollect(int elem_size, rocshmem_amd_team_t team, void *dest
 int rocshmem_amd_wg_sync(int sync_fn, rocshmem_amd_team_t team, uint64_t *scratch, int rounds,
                          int wg_size, rocshmem_amd_stream_t stream) {
   auto &r = runtime::rt();
-  if (!r.live || rounds < 0 || !valid_launch(1, wg_size) || !in_heap(scratch)) return -1;
+  if (!r.live || rounds < 0 || !valid_launch(1, wg_size) || !sym_ok_on(scratch, 8, r.acting_pe)) return -1;
   if (sync_fn < ROCSHMEM_AMD_BARRIER_ALL || sync_fn > ROCSHMEM_AMD_TEAM_SYNC) return -1;
   TeamView v;
   if (sync_fn == ROCSHMEM_AMD_TEAM_SYNC) {
@@ -507,10 +522,9 @@ int rocshmem_amd_to_all(int dtype, int op, void *dest, const void *source, int n
   if (!r.live || PE_start < 0 || logPE_stride < 0 || logPE_stride > 30 || PE_size < 1) return -1;
   const int stride = 1 << logPE_stride;
   if (PE_start + static_cast<long>(stride) * (PE_size - 1) >= r.npes) return -1;
-  if (!in_heap(dest) || !in_heap(source)) return -1;
-  if (r.pe_of(dest) != PE_start || r.pe_of(source) != PE_start) return -1;
-  const size_t bytes = static_cast<size_t>(nreduce < 0 ? 0 : nreduce) * dtype_size(dtype);
-  if (r.offset_of(dest) + bytes > r.heap_size || r.offset_of(source) + bytes > r.heap_size) return -1;
+  if (nreduce < 0) return -1;
+  const size_t bytes = static_cast<size_t>(nreduce) * dtype_size(dtype);
+  if (!sym_ok_on(dest, bytes, PE_start) || !sym_ok_on(source, bytes, PE_start)) return -1;
   return grid_reduce_common(dtype, op, dest, source, static_cast<int64_t>(stride) * r.pe_stride,
                             PE_size, nreduce, as_stream(stream));
 }
@@ -518,10 +532,10 @@ int rocshmem_amd_to_all(int dtype, int op, void *dest, const void *source, int n
 int rocshmem_amd_reduce(int dtype, int op, rocshmem_amd_team_t team, void *dest,
                         const void *source, int nreduce, rocshmem_amd_stream_t stream) {
   TeamView v;
-  if (!view_team(team, &v) || !in_heap(dest) || !in_heap(source)) return -1;
+  if (!view_team(team, &v) || nreduce < 0) return -1;
   auto &r = runtime::rt();
-  const size_t bytes = static_cast<size_t>(nreduce < 0 ? 0 : nreduce) * dtype_size(dtype);
-  if (r.offset_of(dest) + bytes > r.heap_size || r.offset_of(source) + bytes > r.heap_size) return -1;
+  const size_t bytes = static_cast<size_t>(nreduce) * dtype_size(dtype);
+  if (!sym_ok_on(dest, bytes, r.acting_pe) || !sym_ok_on(source, bytes, r.acting_pe)) return -1;
   const int64_t first = static_cast<int64_t>(v.host->wrt_world.pe_start) * r.pe_stride;
   const int64_t hop = static_cast<int64_t>(v.host->wrt_world.stride) * r.pe_stride;
   return grid_reduce_common(dtype, op, on_pe0(dest) + first, on_pe0(source) + first, hop,

@@ -32,6 +32,28 @@ inline bool valid_pe(int pe) {
 }
 inline hipStream_t as_stream(void *s) { return static_cast<hipStream_t>(s); }
 
+// [p, p+bytes) lies inside the usable part of one PE's slice.
+inline bool sym_ok(const void *p, size_t bytes) {
+  auto &r = runtime::rt();
+  if (!r.live || !p) return false;
+  const uint64_t off = r.offset_of(p);
+  return off != runtime::Pow2Allocator::kNoBlock && off <= r.heap_size &&
+         bytes <= r.heap_size - off;
+}
+// As sym_ok, and the address belongs to PE `pe`.
+inline bool sym_ok_on(const void *p, size_t bytes, int pe) {
+  return sym_ok(p, bytes) && runtime::rt().pe_of(p) == pe;
+}
+// A caller-local buffer: any non-null device address outside the heap is taken
+// on trust; one inside the heap must stay inside its slice.
+inline bool local_ok(const void *p, size_t bytes) {
+  auto &r = runtime::rt();
+  if (!p) return bytes == 0;
+  const char *c = static_cast<const char *>(p);
+  if (r.live && c >= r.heap_base && c < r.heap_base + r.pe_stride * r.npes) return sym_ok(p, bytes);
+  return true;
+}
+
 // Bytes per tile when the caller leaves the choice to the driver: an equal
 // share per group, rounded up to 16 bytes.
 inline size_t auto_tile(size_t nbytes, size_t groups) {

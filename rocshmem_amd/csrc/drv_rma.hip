@@ -129,6 +129,13 @@ int rocshmem_amd_rma(int rma_op, int gran, void *dest, const void *source, size_
     return -1;
   if (rma_op != ROCSHMEM_AMD_PUT && rma_op != ROCSHMEM_AMD_GET) return -1;
   if (gran < ROCSHMEM_AMD_THREAD || gran > ROCSHMEM_AMD_WG) return -1;
+  // The remote side must be a symmetric address of my_pe; the local side may
+  // be any device buffer.
+  if (rma_op == ROCSHMEM_AMD_PUT) {
+    if (!sym_ok_on(dest, nbytes, my_pe) || !local_ok(source, nbytes)) return -1;
+  } else {
+    if (!sym_ok_on(source, nbytes, my_pe) || !local_ok(dest, nbytes)) return -1;
+  }
   size_t groups = n_wgs;
   if (gran == ROCSHMEM_AMD_WAVE) groups *= (wg_size + 63) / 64;
   if (gran == ROCSHMEM_AMD_THREAD) groups *= wg_size;
@@ -158,6 +165,7 @@ int rocshmem_amd_rma(int rma_op, int gran, void *dest, const void *source, size_
 int rocshmem_amd_putmem(void *dest, const void *source, size_t nbytes, int my_pe, int pe,
                         rocshmem_amd_stream_t stream) {
   if (!valid_pe(my_pe) || !valid_pe(pe)) return -1;
+  if (!sym_ok_on(dest, nbytes, my_pe) || !local_ok(source, nbytes)) return -1;
   char *target = static_cast<char *>(dest) +
                  static_cast<int64_t>(pe - my_pe) * static_cast<int64_t>(runtime::rt().pe_stride);
   launch_bulk(target, static_cast<const char *>(source), nbytes, as_stream(stream));
@@ -167,6 +175,7 @@ int rocshmem_amd_putmem(void *dest, const void *source, size_t nbytes, int my_pe
 int rocshmem_amd_getmem(void *dest, const void *source, size_t nbytes, int my_pe, int pe,
                         rocshmem_amd_stream_t stream) {
   if (!valid_pe(my_pe) || !valid_pe(pe)) return -1;
+  if (!sym_ok_on(source, nbytes, my_pe) || !local_ok(dest, nbytes)) return -1;
   const char *origin = static_cast<const char *>(source) +
                        static_cast<int64_t>(pe - my_pe) * static_cast<int64_t>(runtime::rt().pe_stride);
   launch_bulk(static_cast<char *>(dest), origin, nbytes, as_stream(stream));
@@ -176,7 +185,7 @@ int rocshmem_amd_getmem(void *dest, const void *source, size_t nbytes, int my_pe
 int rocshmem_amd_wf_coalesce(const int *pe, const uint64_t *src, const uint64_t *dst,
                              const uint64_t *size, uint64_t active_mask, int *sends_out,
                              uint64_t *size_out) {
-  if (!runtime::rt().live) return -1;
+  if (!runtime::rt().live || !pe || !src || !dst || !size || !sends_out || !size_out) return -1;
   int *d_pe, *d_sends;
   uint64_t *d_src, *d_dst, *d_size, *d_size_out;
   DRV_CHECK_HIP(hipMalloc(&d_pe, 64 * sizeof(int)));

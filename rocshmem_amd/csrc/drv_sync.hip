@@ -3,6 +3,9 @@
 #include "drv_common.hpp"
 #include "rocshmem_amd.h"
 
+#include <algorithm>
+#include <vector>
+
 namespace rocshmem {
 namespace drv {
 
@@ -486,6 +489,11 @@ int rocshmem_amd_amo(int amo_op, int dtype, void *counters, uint32_t n_slots,
                      rocshmem_amd_stream_t stream) {
   if (!valid_pe(my_pe) || !valid_launch(n_wgs, wg_size) || !n_slots || !ids) return -1;
   if (amo_op == ROCSHMEM_AMD_AMO_COMPARE_SWAP && !conds) return -1;
+  {
+    const size_t es = (dtype == ROCSHMEM_AMD_INT || dtype == ROCSHMEM_AMD_UINT ||
+                       dtype == ROCSHMEM_AMD_FLOAT) ? 4 : 8;
+    if (!sym_ok_on(counters, es * n_slots, my_pe)) return -1;
+  }
   int rc = -1;
   const bool known = for_amo_dtype(dtype, [&](auto *tag) {
     using T = typename std::remove_pointer<decltype(tag)>::type;
@@ -508,6 +516,9 @@ int rocshmem_amd_put_signal(int gran, void *dest, const void *source, size_t nby
                             int n_wgs, int wg_size, int calls, rocshmem_amd_stream_t stream) {
   if (!valid_pe(my_pe) || !valid_pe(pe) || !valid_launch(n_wgs, wg_size) || calls < 0) return -1;
   if (gran < ROCSHMEM_AMD_THREAD || gran > ROCSHMEM_AMD_WG) return -1;
+  if (!sym_ok_on(dest, nbytes, my_pe) || !local_ok(source, nbytes) ||
+      !sym_ok_on(sig_addr, 8, my_pe))
+    return -1;
   size_t groups = n_wgs;
   if (gran == ROCSHMEM_AMD_WAVE) groups *= (wg_size + 63) / 64;
   if (gran == ROCSHMEM_AMD_THREAD) groups *= wg_size;
@@ -532,7 +543,7 @@ int rocshmem_amd_put_signal(int gran, void *dest, const void *source, size_t nby
 }
 
 int rocshmem_amd_signal_fetch(int gran, const uint64_t *sig_addr, int my_pe, uint64_t *value_out) {
-  if (!valid_pe(my_pe) || !value_out) return -1;
+  if (!valid_pe(my_pe) || !value_out || !sym_ok_on(sig_addr, 8, my_pe)) return -1;
   uint64_t *d_out;
   DRV_CHECK_HIP(hipMalloc(&d_out, 2 * sizeof(uint64_t)));
   DRV_CHECK_HIP(hipMemset(d_out, 0, 2 * sizeof(uint64_t)));
@@ -555,6 +566,7 @@ int rocshmem_amd_pingpong(void *buf, uint64_t *sig, size_t nbytes, int iters, in
   if (!valid_pe(pe_a) || !valid_pe(pe_b) || pe_a == pe_b || !valid_launch(2, wg_size) ||
       iters < 0 || nbytes == 0)
     return -1;
+  if (!sym_ok_on(buf, nbytes, pe_a) || !sym_ok_on(sig, 8, pe_a)) return -1;
   auto &r = runtime::rt();
   unsigned long long *d_ticks;
   DRV_CHECK_HIP(hipMalloc(&d_ticks, sizeof(unsigned long long)));
@@ -594,7 +606,23 @@ int rocshmem_amd_dispatch_put_signal(void *recv, const void *send, uint64_t *sig
                                      rocshmem_amd_stream_t stream) {
   auto &r = runtime::rt();
   if (!r.live || wgs_per_pair < 1 || !valid_launch(1, wg_size) || !row_bytes) return -1;
-  if (r.pe_of(recv) != 0 || r.pe_of(send) != 0 || r.pe_of(sig) != 0) return -1;
+  if (!count || !send_row || !recv_row) return -1;
+  {
+    // Bounds of every pair's rows, from a host copy of the three tables.
+    const size_t pp = static_cast<size_t>(r.npes) * r.npes;
+    std::vector<uint32_t> h(3 * pp);
+    DRV_CHECK_HIP(hipMemcpy(h.data(), count, pp * 4, hipMemcpyDeviceToHost));
+    DRV_CHECK_HIP(hipMemcpy(h.data() + pp, send_row, pp * 4, hipMemcpyDeviceToHost));
+    DRV_CHECK_HIP(hipMemcpy(h.data() + 2 * pp, recv_row, pp * 4, hipMemcpyDeviceToHost));
+    size_t max_send = 0, max_recv = 0;
+    for (size_t i = 0; i < pp; ++i) {
+      max_send = std::max<size_t>(max_send, static_cast<size_t>(h[pp + i]) + h[i]);
+      max_recv = std::max<size_t>(max_recv, static_cast<size_t>(h[2 * pp + i]) + h[i]);
+    }
+    if (!sym_ok_on(send, max_send * row_bytes, 0) || !sym_ok_on(recv, max_recv * row_bytes, 0) ||
+        !sym_ok_on(sig, 8 * static_cast<size_t>(r.npes), 0))
+      return -1;
+  }
   DispatchArgs a;
   a.recv0 = static_cast<char *>(recv);
   a.send0 = static_cast<const char *>(send);

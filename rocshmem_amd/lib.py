@@ -36,6 +36,13 @@ SIGNATURES = {
     "rocshmem_amd_heap_used": (_sz, []),
     "rocshmem_amd_heap_avail": (_sz, []),
     "rocshmem_amd_pe_stride": (_sz, []),
+    "rocshmem_amd_heap_model_create": (_vp, [_u64, _u64]),
+    "rocshmem_amd_heap_model_destroy": (None, [_vp]),
+    "rocshmem_amd_heap_model_alloc": (_u64, [_vp, _u64]),
+    "rocshmem_amd_heap_model_free": (_i, [_vp, _u64]),
+    "rocshmem_amd_heap_model_used": (_u64, [_vp]),
+    "rocshmem_amd_heap_model_num_bins": (_u64, [_vp]),
+    "rocshmem_amd_heap_model_bin_population": (_u64, [_vp, _u64]),
     "rocshmem_amd_team_world": (_vp, []),
     "rocshmem_amd_team_split_strided": (_i, [_vp, _i, _i, _i, C.POINTER(_vp)]),
     "rocshmem_amd_team_destroy": (None, [_vp]),
