@@ -1,0 +1,344 @@
+#!/usr/bin/env python3
+"""Throughput of the symmetric-heap data path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick]
+
+Prints ONE JSON line.  The headline (`metric`/`value`) is the bulk putmem
+workload of BASELINE.json's configs[1]: one 256 MiB message between two of
+P=8 PE slices of one symmetric heap, moved by the whole GPU; a step is one such
+message and `value` counts algorithmic bytes (N read + N written).  The same
+line carries the other configurations (all-reduce, alltoall, put_signal
+dispatch, atomics, ping-pong) under `all_configs`, the roofline of the
+headline kernel measured with HIP events on the launch stream, and a CPU
+baseline (the oracle's threaded routines on the host cores, bounded sample).
+
+Inputs are resident in HBM before any timed region starts.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X, published
+P = 8
+MiB = 1 << 20
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--quick", action="store_true", help="headline only, no CPU baseline")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    return ap.parse_args()
+
+
+class Bench:
+    def __init__(self, L):
+        self.L = L
+        self.l = L.load()
+        self.timer = self.l.timer_create()
+
+    def time_ms(self, fn, steps, warmup):
+        """Average milliseconds per call of fn over `steps` calls, HIP events
+        on the stream the kernels are launched on (the null stream)."""
+        l = self.l
+        for _ in range(warmup):
+            fn()
+        l.stream_sync(None)
+        l.timer_start(self.timer, None)
+        for _ in range(steps):
+            fn()
+        l.timer_stop(self.timer, None)
+        return l.timer_elapsed_ms(self.timer) / steps
+
+    def fill_random(self, ptr, nbytes, pe, seed):
+        """Random payload resident on the device: a seeded 4 MiB tile uploaded
+        once and doubled in place by on-device copies."""
+        l = self.l
+        tile = min(nbytes, 4 * MiB)
+        rng = np.random.default_rng(seed)
+        host = rng.integers(0, 256, tile, dtype=np.uint8)
+        l.copy_in(ptr, host.ctypes.data, tile)
+        done = tile
+        while done < nbytes:
+            step = min(done, nbytes - done)
+            assert l.putmem(ptr + done, ptr, step, pe, pe, None) == 0
+            done += step
+        l.stream_sync(None)
+
+
+def headline(b, steps, warmup):
+    """configs[1]: bulk putmem, 256 MiB, PE 0 -> PE 1, all CUs."""
+    l = b.l
+    n = 256 * MiB
+    src, dst = l.malloc(n), l.malloc(n)
+    assert src and dst
+    b.fill_random(src, n, 0, 1)
+    ms = b.time_ms(lambda: l.putmem(dst, src, n, 0, 1, None), steps, warmup)
+    out = {"bytes_per_step": 2 * n, "ms": ms, "gbs": 2 * n / ms / 1e6}
+    # the rest of the bandwidth curve (device API, one work-group and all CUs)
+    curve = {}
+    for k in (3, 6, 10, 13, 16, 20, 24, 28):
+        m = 1 << k
+        reps = max(3, min(steps, 20))
+        t1 = b.time_ms(lambda: l.rma(b.L.PUT, b.L.WG, dst, src, m, 0, 0, 1, 1, 1024, 1, None),
+                       reps if k < 24 else 3, 2)
+        tg = b.time_ms(lambda: l.putmem(dst, src, m, 0, 1, None), reps, 2)
+        tget = b.time_ms(lambda: l.getmem(dst, src, m, 0, 1, None), reps, 2)
+        curve[str(m)] = {"putmem_wg_1wg_gbs": round(2 * m / t1 / 1e6, 3),
+                         "putmem_all_cus_gbs": round(2 * m / tg / 1e6, 3),
+                         "getmem_all_cus_gbs": round(2 * m / tget / 1e6, 3)}
+    out["curve"] = curve
+    l.free(src)
+    l.free(dst)
+    return out
+
+
+def to_all_configs(b, steps, warmup):
+    """configs[2]: all-reduce over P=8 slices x 64 Mi elements."""
+    l, L = b.l, b.L
+    n = 1 << 26
+    res = {}
+    # largest buffers first: freed blocks are never merged by the allocator
+    for name, dt, op, es in (("int64_xor", L.LONG, L.XOR, 8), ("fp32_sum", L.FLOAT, L.SUM, 4),
+                             ("fp32_max", L.FLOAT, L.MAX, 4), ("bf16_sum", L.BF16, L.SUM, 2)):
+        src, dst = l.malloc(n * es), l.malloc(n * es)
+        assert src and dst, name
+        for p in range(P):
+            b.fill_random(l.pe_ptr(src, p), n * es, p, 10 + p)
+            if dt in (L.FLOAT, L.BF16):
+                pass  # random bit patterns: NaNs cost the same as numbers here
+        ms = b.time_ms(lambda: l.to_all(dt, op, dst, src, n, 0, 0, P, None), max(5, steps // 5), 3)
+        alg = 2 * P * n * es
+        res[name] = {"ms": round(ms, 4), "gbs": round(alg / ms / 1e6, 1),
+                     "frac": round(alg / ms / 1e6 / HBM_PEAK_GBS, 4)}
+        l.free(src)
+        l.free(dst)
+    return res
+
+
+def alltoall_config(b, steps):
+    """configs[4] part 1: alltoall, 512 tokens x 7168 bf16 per PE pair."""
+    l = b.l
+    blk = 512 * 7168 * 2
+    src, dst = l.malloc(P * blk), l.malloc(P * blk)
+    assert src and dst
+    for p in range(P):
+        b.fill_random(l.pe_ptr(src, p), P * blk, p, 30 + p)
+    ms = b.time_ms(lambda: l.alltoallmem(l.team_world(), dst, src, blk, None), max(5, steps // 5), 3)
+    alg = 2 * P * P * blk
+    l.free(src)
+    l.free(dst)
+    return {"ms": round(ms, 4), "gbs": round(alg / ms / 1e6, 1),
+            "frac": round(alg / ms / 1e6 / HBM_PEAK_GBS, 4)}
+
+
+def zipf_table(K, s):
+    w = 1.0 / np.power(np.arange(1, K + 1, dtype=np.float64), s)
+    return np.cumsum(w / w.sum())
+
+
+def dispatch_config(b, steps):
+    """configs[4] part 2: put_signal dispatch, 4096 tokens/PE, top-8 of 256
+    experts by Zipf(1.1), rows of 7168 bf16."""
+    l = b.l
+    tokens, experts, topk, row = 4096, 256, 8, 7168 * 2
+    rng = np.random.default_rng(0)
+    cdf = zipf_table(experts, 1.1)
+    counts = np.zeros((P, P), np.uint32)
+    for s in range(P):
+        # top-k distinct by Gumbel-free sequential redraw on a vectorised batch
+        chosen = np.full((tokens, topk), -1, np.int64)
+        for k in range(topk):
+            pick = np.searchsorted(cdf, rng.random(tokens))
+            dup = (chosen[:, :k] == pick[:, None]).any(1)
+            while dup.any():
+                pick[dup] = np.searchsorted(cdf, rng.random(int(dup.sum())))
+                dup = (chosen[:, :k] == pick[:, None]).any(1)
+            chosen[:, k] = np.minimum(pick, experts - 1)
+        counts[s] = np.bincount((chosen // (experts // P)).ravel(), minlength=P)
+    send_row = np.zeros((P, P), np.uint32)
+    recv_row = np.zeros((P, P), np.uint32)
+    for s in range(P):
+        send_row[s] = np.r_[0, np.cumsum(counts[s])[:-1]]
+    for d in range(P):
+        recv_row[:, d] = np.r_[0, np.cumsum(counts[:, d])[:-1]]
+    rows_out = tokens * topk
+    rows_in = int(counts.sum(0).max())
+    send, recv, sig = l.malloc(rows_out * row), l.malloc(rows_in * row), l.malloc(8 * P)
+    assert send and recv and sig
+    for p in range(P):
+        b.fill_random(l.pe_ptr(send, p), rows_out * row, p, 40 + p)
+    dev = []
+    for a in (counts, send_row, recv_row):
+        d = l.dev_alloc(a.nbytes)
+        l.copy_in(d, np.ascontiguousarray(a).ctypes.data, a.nbytes)
+        dev.append(d)
+
+    def step():
+        for p in range(P):  # signals start from zero each dispatch
+            l.fill(l.pe_ptr(sig, p), 0, 8 * P)
+        assert l.dispatch_put_signal(recv, send, sig, dev[0], dev[1], dev[2], row, 32, 256, None) == 0
+
+    ms = b.time_ms(step, max(5, steps // 10), 2)
+    alg = 2 * int(counts.sum()) * row
+    for d in dev:
+        l.dev_free(d)
+    for x in (send, recv, sig):
+        l.free(x)
+    return {"ms": round(ms, 4), "gbs": round(alg / ms / 1e6, 1),
+            "frac": round(alg / ms / 1e6 / HBM_PEAK_GBS, 4), "rows": int(counts.sum())}
+
+
+def amo_config(b, steps):
+    """configs[5] part 1: 16 Mi int64 fetch_add onto 4096 counters."""
+    l, L = b.l, b.L
+    K, n = 4096, 1 << 24
+    ctr = l.malloc(K // P * 8)
+    res = {}
+    rng = np.random.default_rng(0)
+    cdf = zipf_table(K, 1.1)
+    for dist in ("uniform", "zipf"):
+        if dist == "uniform":
+            ids = rng.integers(0, K, n, dtype=np.uint32)
+        else:
+            ids = np.minimum(np.searchsorted(cdf, rng.random(n)), K - 1).astype(np.uint32)
+        d_ids = l.dev_alloc(n * 4)
+        d_out = l.dev_alloc(n * 8)
+        l.copy_in(d_ids, ids.ctypes.data, n * 4)
+        for p in range(P):
+            l.fill(l.pe_ptr(ctr, p), 0, K // P * 8)
+        ms = b.time_ms(lambda: l.amo(L.AMO_FETCH_ADD, L.LONG, ctr, K // P, d_ids, None, None, d_out,
+                                     n, 0, 4096, 256, None), max(3, steps // 10), 1)
+        res[dist] = {"ms": round(ms, 4), "mops": round(n / ms / 1e3, 1)}
+        l.dev_free(d_ids)
+        l.dev_free(d_out)
+    l.free(ctr)
+    return res
+
+
+def pingpong_config(b):
+    """configs[5] part 2: put_signal / wait_until ping-pong between two
+    work-groups acting as two PEs."""
+    l = b.l
+    buf, sig = l.malloc(65536), l.malloc(8)
+    res = {}
+    iters = 2000
+    for k in range(3, 17):
+        n = 1 << k
+        for p in (0, 1):
+            l.fill(l.pe_ptr(sig, p), 0, 8)
+        ticks, hz = C.c_uint64(), C.c_double()
+        assert l.pingpong(buf, sig, n, iters, 0, 1, 256, C.byref(ticks), C.byref(hz), None) == 0
+        one_way_us = ticks.value / hz.value / iters / 2 * 1e6
+        res[str(n)] = {"latency_us": round(one_way_us, 3), "msg_per_s": round(1e6 / one_way_us, 1)}
+    l.free(buf)
+    l.free(sig)
+    return res
+
+
+def cpu_baseline():
+    """The oracle's threaded routines on this host's cores, bounded samples.
+    (The only place outside tests/ and smoke() that touches oracle/.)"""
+    from oracle import pyoracle as orc
+    cores = orc.lib.orc_hardware_threads()
+    threads = max(1, cores)
+    out = {}
+    # bulk copy: 256 MiB message, as the headline
+    n = 256 * MiB
+    src = np.random.default_rng(0).integers(0, 256, n, dtype=np.uint8)
+    dst = np.empty_like(src)
+    orc.lib.orc_copy_threaded(dst.ctypes.data, src.ctypes.data, n, threads)
+    t0 = time.perf_counter()
+    reps = 0
+    while time.perf_counter() - t0 < 4.0:
+        orc.lib.orc_copy_threaded(dst.ctypes.data, src.ctypes.data, n, threads)
+        reps += 1
+    copy_gbs = 2 * n * reps / (time.perf_counter() - t0) / 1e9
+    # fp32 sum all-reduce, P=8 x 4 Mi elements (1/16 of the GPU workload)
+    m = 1 << 22
+    srcs = [np.random.default_rng(p).standard_normal(m).astype(np.float32) for p in range(P)]
+    t0 = time.perf_counter()
+    reps = 0
+    while time.perf_counter() - t0 < 4.0:
+        orc.to_all(orc.FLOAT, orc.SUM, srcs, ndst=P, nthreads=threads)
+        reps += 1
+    red_gbs = 2 * P * m * 4 * reps / (time.perf_counter() - t0) / 1e9
+    # atomics: 4 Mi fetch_adds onto 4096 counters
+    k = 1 << 22
+    ids = np.random.default_rng(1).integers(0, 4096, k, dtype=np.uint32)
+    counters = np.zeros(4096, np.int64)
+    fetched = np.zeros(k, np.int64)
+    sec = orc.lib.orc_amo_fetch_add_threaded(counters.ctypes.data, ids.ctypes.data, None,
+                                             fetched.ctypes.data, k, threads)
+    pp = orc.lib.orc_pingpong_threaded(8, 200000) / 200000 / 2 * 1e6
+    out = {"value": round(copy_gbs, 2), "unit": "GB/s", "cores": threads, "kind": "port",
+           "sample": "threaded memcpy of one 256 MiB message repeated for 4 s (2N bytes per pass)",
+           "other": {"fp32_sum_to_all_gbs": round(red_gbs, 2),
+                     "fp32_sum_sample": "P=8 x 4 Mi elements, ascending fold, 4 s",
+                     "amo_fetch_add_mops": round(k / sec / 1e6, 1),
+                     "amo_sample": "4 Mi seq_cst fetch_add on 4096 counters, uniform",
+                     "pingpong_8B_latency_us": round(pp, 3)}}
+    return out
+
+
+def main():
+    a = parse()
+    if a.gpus != 1:
+        print("bench.py measures one GPU: every PE is a slice of one symmetric heap on a single "
+              "MI355X; --gpus %d is not supported (use --gpus 1)." % a.gpus, file=sys.stderr)
+        sys.exit(2)
+    from rocshmem_amd import lib as L
+    b = Bench(L)
+    # 8 slices of 4 GiB: the dispatch receive buffer of the busiest PE needs a
+    # 2 GiB block, int64 x 64 Mi needs 2 x 512 MiB.  Largest requests go first
+    # because the allocator never merges freed blocks.
+    assert b.l.init(P, 4 << 30) == 0
+    head = headline(b, a.steps, a.warmup)
+    allc = {}
+    if not a.quick:
+        allc["dispatch_put_signal"] = dispatch_config(b, a.steps)
+        allc["to_all_P8_64Mi"] = to_all_configs(b, a.steps, a.warmup)
+        allc["alltoall_512x7168_bf16"] = alltoall_config(b, a.steps)
+        allc["atomic_fetch_add_16Mi"] = amo_config(b, a.steps)
+        allc["pingpong"] = pingpong_config(b)
+    allc["putmem_curve"] = head["curve"]
+    b.l.finalize()
+    cpu = None if (a.quick or a.no_cpu) else cpu_baseline()
+    line = {
+        "metric": "HBM GB/s (% of MI355X peak) for to_all/alltoall/putmem; atomic Mops/s",
+        "value": round(head["gbs"], 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": a.steps,
+        "warmup": a.warmup,
+        "ms_per_step": round(head["ms"], 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "u8",
+        "data": "synthetic",
+        "config": {"workload": "bulk putmem, one 256 MiB message PE0->PE1 of P=8 slices in one "
+                               "symmetric heap, all CUs (BASELINE configs[1], largest size)",
+                   "n_pes": P, "message_bytes": 256 * MiB, "heap_bytes_per_pe": 4 << 30},
+        "roofline": {"bound": "hbm", "achieved": round(head["gbs"], 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(head["gbs"] / HBM_PEAK_GBS, 4),
+                     "traffic": None, "kernel": "bulk_copy_kernel<true>",
+                     "algorithmic_bytes_per_launch": head["bytes_per_step"]},
+        "cpu_baseline": cpu,
+        "all_configs": allc,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

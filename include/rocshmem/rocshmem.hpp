@@ -117,13 +117,16 @@ __device__ ATTR_NO_INLINE inline void rocshmem_wg_ctx_destroy(rocshmem_ctx_t *ct
 }
 
 // fence / quiet are ordering points, not completion waits
-// (src/ipc/context_ipc_device.cpp:90-102).
-__device__ ATTR_NO_INLINE inline void rocshmem_ctx_fence(rocshmem_ctx_t) { detail::fence_full(); }
-__device__ ATTR_NO_INLINE inline void rocshmem_fence() { detail::fence_full(); }
-__device__ ATTR_NO_INLINE inline void rocshmem_ctx_fence(rocshmem_ctx_t, int) { detail::fence_full(); }
-__device__ ATTR_NO_INLINE inline void rocshmem_fence(int) { detail::fence_full(); }
-__device__ ATTR_NO_INLINE inline void rocshmem_ctx_quiet(rocshmem_ctx_t) { detail::fence_full(); }
-__device__ ATTR_NO_INLINE inline void rocshmem_quiet() { detail::fence_full(); }
+// (src/ipc/context_ipc_device.cpp:90-102, where both are a sequentially
+// consistent store per PE).  Every operation of this library has already
+// performed its loads and stores when it returns, so what is left to do is to
+// publish them: a release at agent scope.
+__device__ ATTR_NO_INLINE inline void rocshmem_ctx_fence(rocshmem_ctx_t) { detail::fence_release(); }
+__device__ ATTR_NO_INLINE inline void rocshmem_fence() { detail::fence_release(); }
+__device__ ATTR_NO_INLINE inline void rocshmem_ctx_fence(rocshmem_ctx_t, int) { detail::fence_release(); }
+__device__ ATTR_NO_INLINE inline void rocshmem_fence(int) { detail::fence_release(); }
+__device__ ATTR_NO_INLINE inline void rocshmem_ctx_quiet(rocshmem_ctx_t) { detail::fence_release(); }
+__device__ ATTR_NO_INLINE inline void rocshmem_quiet() { detail::fence_release(); }
 __device__ ATTR_NO_INLINE inline void rocshmem_ctx_threadfence_system(rocshmem_ctx_t) {
   __threadfence_system();
 }

@@ -56,7 +56,8 @@ __global__ void rma_kernel(RmaArgs a) {
       }
     }
   }
-  rocshmem_ctx_quiet(a.ctx);
+  // One quiet per group, as a kernel that batches its puts would issue it.
+  if (kGran != ROCSHMEM_AMD_WG || threadIdx.x == 0) rocshmem_ctx_quiet(a.ctx);
 }
 
 // Whole-GPU copy: every thread of the grid is one lane of a single

@@ -1,0 +1,268 @@
+"""R1-R6, R-CPU: all-reduce through the device API (one work-group per PE) and
+through the host-called whole-GPU form, bit-exact against the oracle's
+ascending-PE fold.  Through the C entry points."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+HEAP = 1 << 30
+INT_OPS = ["SUM", "MAX", "MIN", "PROD", "AND", "OR", "XOR"]
+FLT_OPS = ["SUM", "MAX", "MIN", "PROD"]
+TYPES = {"SHORT": INT_OPS, "INT": INT_OPS, "LONG": INT_OPS, "LONGLONG": INT_OPS,
+         "FLOAT": FLT_OPS, "DOUBLE": FLT_OPS, "BF16": ["SUM"]}
+
+
+def make_inputs(orc, dtype_name, P, n, seed):
+    rng = np.random.default_rng(seed)
+    np_t = orc.NP_DTYPE[getattr(orc, dtype_name)]
+    if dtype_name == "BF16":
+        return [orc.f32_to_bf16(orc.fill_normal_f32(n, seed, p)) for p in range(P)]
+    if dtype_name in ("FLOAT", "DOUBLE"):
+        return [orc.fill_normal_f32(n, seed, p).astype(np_t) for p in range(P)]
+    info = np.iinfo(np_t)
+    return [rng.integers(info.min, info.max, n, dtype=np_t, endpoint=True) for _ in range(P)]
+
+
+class Buffers:
+    def __init__(self, rt, l, nbytes):
+        self.rt, self.l = rt, l
+        self.src = l.malloc(nbytes)
+        self.dst = l.malloc(nbytes)
+        assert self.src and self.dst
+
+    def free(self):
+        self.l.free(self.src)
+        self.l.free(self.dst)
+
+
+def check_all(rt, l, orc, L, P, dtype_name, op_name, n, mode, seed=0, off=0, wg=256, pes=None,
+              team=None):
+    """pes: world PEs taking part (default all); off: element offset into the
+    buffers (exercises unaligned starts)."""
+    pes = list(range(P)) if pes is None else pes
+    dt, op = getattr(L, dtype_name), getattr(L, op_name)
+    np_t = orc.NP_DTYPE[getattr(orc, dtype_name)]
+    es = np.dtype(np_t).itemsize
+    b = Buffers(rt, l, (n + off + 8) * es)
+    srcs = make_inputs(orc, dtype_name, len(pes), n, seed)
+    for p in range(P):
+        l.fill(l.pe_ptr(b.dst, p), 0x5A, (n + off + 8) * es)
+    for k, p in enumerate(pes):
+        rt.put_bytes(l.pe_ptr(b.src, p) + off * es, srcs[k])
+    me = l.my_pe()
+    d = l.pe_ptr(b.dst, me) + off * es
+    s = l.pe_ptr(b.src, me) + off * es
+    if mode == "wg":
+        rc = l.wg_reduce(dt, op, team if team else l.team_world(), d, s, n, wg, None)
+    elif mode == "to_all":
+        stride = pes[1] - pes[0] if len(pes) > 1 else 1
+        log = int(np.log2(stride))
+        rc = l.to_all(dt, op, l.pe_ptr(b.dst, pes[0]) + off * es, l.pe_ptr(b.src, pes[0]) + off * es,
+                      n, pes[0], log, len(pes), None)
+    else:
+        rc = l.reduce(dt, op, team if team else l.team_world(), d, s, n, None)
+    assert rc == 0, (dtype_name, op_name, n, mode)
+    l.stream_sync(None)
+    want = orc.to_all(getattr(orc, dtype_name), getattr(orc, op_name), srcs)
+    for p in range(P):
+        got = rt.get_bytes(l.pe_ptr(b.dst, p), (n + off + 8) * es, np_t)
+        if p in pes:
+            assert np.array_equal(got[off:off + n].view(np.uint8), want.view(np.uint8)), \
+                (dtype_name, op_name, n, mode, p)
+            rest = np.concatenate([got[:off], got[off + n:]]).view(np.uint8)
+        else:
+            rest = got.view(np.uint8)
+        assert (rest == 0x5A).all(), (dtype_name, op_name, n, mode, p, "guard")
+    b.free()
+
+
+@pytest.mark.parametrize("mode", ["wg", "to_all"])
+@pytest.mark.parametrize("dtype_name", list(TYPES))
+def test_every_type_and_op(rt, L, orc, dtype_name, mode):
+    l = rt.up(8, HEAP)
+    for op_name in TYPES[dtype_name]:
+        for n in (1, 37, 1000, 4099):
+            check_all(rt, l, orc, L, 8, dtype_name, op_name, n, mode, seed=n)
+
+
+@pytest.mark.parametrize("mode", ["wg", "to_all"])
+@pytest.mark.parametrize("P", [1, 2, 3, 4, 5, 8])
+def test_pe_counts_and_ragged_sizes(rt, L, orc, P, mode):
+    l = rt.up(P, 64 << 20)
+    for n in (1, 2, 3, 5, 7, 8, 9, 63, 64, 65, 127, 1025, 20001):
+        check_all(rt, l, orc, L, P, "FLOAT", "SUM", n, mode, seed=n)
+        check_all(rt, l, orc, L, P, "LONG", "XOR", n, mode, seed=n)
+        check_all(rt, l, orc, L, P, "BF16", "SUM", n, mode, seed=n)
+    rt.up(8, HEAP)
+
+
+@pytest.mark.parametrize("mode", ["wg", "to_all"])
+def test_unaligned_starts(rt, L, orc, mode):
+    l = rt.up(8, HEAP)
+    for off in (1, 2, 3, 5):
+        for dtype_name in ("SHORT", "INT", "FLOAT", "LONG", "BF16"):
+            check_all(rt, l, orc, L, 8, dtype_name, "SUM", 3001, mode, seed=off, off=off)
+
+
+@pytest.mark.parametrize("wg", [1, 64, 100, 1024])
+def test_work_group_sizes(rt, L, orc, wg):
+    l = rt.up(8, HEAP)
+    check_all(rt, l, orc, L, 8, "FLOAT", "SUM", 5003, "wg", wg=wg)
+    check_all(rt, l, orc, L, 8, "INT", "MAX", 333, "wg", wg=wg)
+
+
+def test_zero_elements_is_a_no_op(rt, L, orc):
+    l = rt.up(8, HEAP)
+    b = Buffers(rt, l, 256)
+    l.fill(b.dst, 0x11, 256)
+    assert l.wg_reduce(L.INT, L.SUM, l.team_world(), b.dst, b.src, 0, 64, None) == 0
+    assert l.to_all(L.INT, L.SUM, b.dst, b.src, 0, 0, 0, 8, None) == 0
+    l.stream_sync(None)
+    assert (rt.get_bytes(b.dst, 256) == 0x11).all()
+    b.free()
+
+
+def test_in_place(rt, L, orc):
+    """dest == source is allowed on the host path (src/host/host_templates.hpp:353)."""
+    l = rt.up(8, HEAP)
+    n = 70001
+    srcs = make_inputs(orc, "FLOAT", 8, n, 9)
+    want = orc.to_all(orc.FLOAT, orc.SUM, srcs)
+    for mode in ("to_all", "wg"):
+        buf = l.malloc(n * 4)
+        for p in range(8):
+            rt.put_bytes(l.pe_ptr(buf, p), srcs[p])
+        if mode == "to_all":
+            assert l.to_all(L.FLOAT, L.SUM, buf, buf, n, 0, 0, 8, None) == 0
+        else:
+            assert l.wg_reduce(L.FLOAT, L.SUM, l.team_world(), buf, buf, n, 256, None) == 0
+        l.stream_sync(None)
+        for p in range(8):
+            got = rt.get_bytes(l.pe_ptr(buf, p), n * 4, np.float32)
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (mode, p)
+        l.free(buf)
+
+
+def test_active_sets_and_teams(rt, L, orc):
+    l = rt.up(8, HEAP)
+    import ctypes
+    # host to_all over (PE_start, logPE_stride, PE_size)
+    for pes in ([0, 2, 4, 6], [1, 3, 5, 7], [2, 3, 4], [4], [0, 4]):
+        check_all(rt, l, orc, L, 8, "INT", "SUM", 2049, "to_all", seed=len(pes), pes=pes)
+    # strided team through the device API and the host team form
+    for start, stride, size in [(0, 2, 4), (1, 3, 2), (2, 1, 5)]:
+        team = ctypes.c_void_p()
+        pes = [start + stride * k for k in range(size)]
+        l.set_pe(pes[0])
+        assert l.team_split_strided(l.team_world(), start, stride, size, ctypes.byref(team)) == 0
+        assert team.value and l.team_n_pes(team) == size
+        for mode in ("wg", "reduce"):
+            check_all(rt, l, orc, L, 8, "FLOAT", "SUM", 1234, mode, seed=start, pes=pes, team=team)
+            check_all(rt, l, orc, L, 8, "LONGLONG", "MIN", 77, mode, seed=start, pes=pes, team=team)
+        l.team_destroy(team)
+    l.set_pe(0)
+
+
+def test_closed_forms_of_the_reference_tests(rt, L, orc):
+    """examples/rocshmem_allreduce_test.cc:49-70 (src[i] = pe + i%9) and
+    tests/functional_tests/tester.cpp:147-159 (all ones -> P)."""
+    l = rt.up(8, HEAP)
+    P, n = 8, 256
+    b = Buffers(rt, l, n * 4)
+    for p in range(P):
+        rt.put_bytes(l.pe_ptr(b.src, p), np.array([p + i % 9 for i in range(n)], np.int32))
+    assert l.wg_reduce(L.INT, L.SUM, l.team_world(), b.dst, b.src, n, 256, None) == 0
+    expect = np.array([P * (P - 1) // 2 + P * (i % 9) for i in range(n)], np.int32)
+    for p in range(P):
+        assert np.array_equal(rt.get_bytes(l.pe_ptr(b.dst, p), n * 4, np.int32), expect)
+    for p in range(P):
+        rt.put_bytes(l.pe_ptr(b.src, p), np.ones(n, np.float32))
+    assert l.wg_reduce(L.FLOAT, L.SUM, l.team_world(), b.dst, b.src, n, 64, None) == 0
+    for p in range(P):
+        assert (rt.get_bytes(l.pe_ptr(b.dst, p), n * 4, np.float32) == P).all()
+    b.free()
+
+
+def test_config1_int32_sum_two_pes_one_mi(rt, L, orc):
+    """int32 sum, P=2, 1,048,576 elements per PE, uniform in [-1000,1000], seed 0."""
+    l = rt.up(2, 64 << 20)
+    n = 1 << 20
+    srcs = [orc.fill_i32_pm1000(n, 0, p) for p in range(2)]
+    want = orc.to_all(orc.INT, orc.SUM, srcs, nthreads=4)
+    assert np.array_equal(want, srcs[0] + srcs[1])
+    b = Buffers(rt, l, n * 4)
+    for p in range(2):
+        rt.put_bytes(l.pe_ptr(b.src, p), srcs[p])
+    for mode in ("wg", "to_all"):
+        for p in range(2):
+            l.fill(l.pe_ptr(b.dst, p), 0, n * 4)
+        if mode == "wg":
+            assert l.wg_reduce(L.INT, L.SUM, l.team_world(), b.dst, b.src, n, 1024, None) == 0
+        else:
+            assert l.to_all(L.INT, L.SUM, b.dst, b.src, n, 0, 0, 2, None) == 0
+        l.stream_sync(None)
+        for p in range(2):
+            assert np.array_equal(rt.get_bytes(l.pe_ptr(b.dst, p), n * 4, np.int32), want), (mode, p)
+    b.free()
+    rt.up(8, HEAP)
+
+
+def test_team_too_large_for_reduce_is_an_error(rt, L, orc):
+    """2*P > ROCSHMEM_REDUCE_SYNC_SIZE -> ROCSHMEM_ERROR
+    (src/ipc/context_ipc_tmpl_device.hpp:412-415)."""
+    l = rt.up(130, 2 << 20)
+    buf = l.malloc(1024)
+    l.fill(buf, 0, 1024)
+    assert l.wg_reduce(L.INT, L.SUM, l.team_world(), buf, buf, 16, 64, None) == 1
+    l.free(buf)
+    rt.up(8, HEAP)
+
+
+def test_unsupported_combinations_are_rejected(rt, L):
+    l = rt.up(8, HEAP)
+    buf = l.malloc(1024)
+    assert l.to_all(L.FLOAT, L.XOR, buf, buf, 4, 0, 0, 8, None) == -1
+    assert l.to_all(L.BF16, L.MAX, buf, buf, 4, 0, 0, 8, None) == -1
+    assert l.to_all(L.INT, L.SUM, buf, buf, 4, 0, 1, 8, None) == -1   # active set leaves the world
+    assert l.to_all(L.INT, L.SUM, buf, buf, 1 << 30, 0, 0, 8, None) == -1
+    assert l.wg_reduce(L.INT, 9, l.team_world(), buf, buf, 4, 64, None) == -1
+    l.free(buf)
+
+
+@pytest.mark.parametrize("dtype_name,op_name", [("FLOAT", "SUM"), ("BF16", "SUM"), ("FLOAT", "MAX"),
+                                                ("LONG", "XOR")])
+def test_full_size_64mi_properties(rt, L, orc, dtype_name, op_name):
+    """P=8 x 64 Mi elements.  Inputs are made on the CPU for windows only; the
+    bulk is checked through size-independent properties: all P destinations are
+    identical, the windows match the oracle, and for xor reducing the result
+    with itself gives zero / reducing twice with P even returns to zero."""
+    l = rt.up(8, 2 << 30)
+    n = 1 << 26
+    np_t = orc.NP_DTYPE[getattr(orc, dtype_name)]
+    es = np.dtype(np_t).itemsize
+    b = Buffers(rt, l, n * es)
+    # fill sources on the device by replicating a seeded 4 Mi-element tile
+    tile = 1 << 22
+    tiles = make_inputs(orc, dtype_name, 8, tile, 123)
+    for p in range(8):
+        base = l.pe_ptr(b.src, p)
+        rt.put_bytes(base, tiles[p])
+        done = tile
+        while done < n:  # doubling copy inside the slice
+            step = min(done, n - done)
+            assert l.putmem(base + done * es, base, step * es, p, p, None) == 0
+            done += step
+    l.stream_sync(None)
+    dt, op = getattr(L, dtype_name), getattr(L, op_name)
+    assert l.to_all(dt, op, b.dst, b.src, n, 0, 0, 8, None) == 0
+    l.stream_sync(None)
+    want_tile = orc.to_all(getattr(orc, dtype_name), getattr(orc, op_name), tiles, nthreads=4)
+    first = rt.get_bytes(l.pe_ptr(b.dst, 0), n * es, np_t)
+    assert np.array_equal(first.reshape(-1, tile).view(np.uint8),
+                          np.broadcast_to(want_tile, (n // tile, tile)).copy().view(np.uint8))
+    for p in range(1, 8):
+        other = rt.get_bytes(l.pe_ptr(b.dst, p), n * es, np_t)
+        assert np.array_equal(other.view(np.uint8), first.view(np.uint8)), p
+    b.free()
+    rt.up(8, HEAP)

@@ -1,0 +1,161 @@
+"""C1-C3, H3: putmem/getmem at thread, wavefront and work-group granularity,
+and the host-initiated whole-GPU copy, byte-exact against the oracle's copy
+with guard bytes either side.  Through the C entry points."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+P, HEAP = 8, 1 << 30
+GUARD = 64
+
+
+@pytest.fixture(scope="module")
+def env(rt, L, orc):
+    l = rt.up(P, HEAP)
+    size = 8 << 20
+    src = l.malloc(size)
+    dst = l.malloc(size)
+    assert src and dst
+    host = orc.fill_u8(size, 0, 11)
+    rt.put_bytes(src, host)
+    yield dict(l=l, src=src, dst=dst, size=size, host=host)
+    l.free(src)
+    l.free(dst)
+
+
+def run_case(rt, L, orc, env, op, gran, n, soff, doff, n_wgs, wg_size, my_pe=0, pe=1, tile=0):
+    """Copies n bytes from src+soff to dst+doff across PEs and checks the
+    destination window including GUARD bytes on both sides."""
+    l = env["l"]
+    src, dst, host = env["src"], env["dst"], env["host"]
+    base = GUARD + 16  # room for the low guard
+    if op == L.PUT:
+        local = l.pe_ptr(src, my_pe) + soff
+        remote_mine = l.pe_ptr(dst, my_pe) + base + doff
+        landing = l.pe_ptr(dst, pe) + base + doff
+        d_arg, s_arg = remote_mine, local
+        if my_pe != 0:
+            rt.put_bytes(l.pe_ptr(src, my_pe), host[:soff + n + 1])
+    else:
+        remote_mine = l.pe_ptr(src, my_pe) + soff
+        origin = l.pe_ptr(src, pe)
+        rt.put_bytes(origin, host[:soff + n + 1])
+        landing = l.pe_ptr(dst, my_pe) + base + doff
+        d_arg, s_arg = landing, remote_mine
+    l.fill(landing - GUARD, 0xA5, n + 2 * GUARD)
+    rc = l.rma(op, gran, d_arg, s_arg, n, tile, my_pe, pe, n_wgs, wg_size, 1, None)
+    assert rc == 0
+    l.stream_sync(None)
+    got = rt.get_bytes(landing - GUARD, n + 2 * GUARD)
+    want = np.full(n + 2 * GUARD, 0xA5, np.uint8)
+    if n:
+        exp = np.empty(n, np.uint8)
+        orc.lib.orc_copy(exp.ctypes.data, host[soff:soff + n].ctypes.data, n)
+        want[GUARD:GUARD + n] = exp
+    assert np.array_equal(got, want), (op, gran, n, soff, doff, n_wgs, wg_size)
+
+
+GRANS = ["THREAD", "WAVE", "WG"]
+
+
+@pytest.mark.parametrize("gran", GRANS)
+@pytest.mark.parametrize("op", ["PUT", "GET"])
+def test_every_size_up_to_300(rt, L, orc, env, op, gran):
+    for n in range(0, 301):
+        run_case(rt, L, orc, env, getattr(L, op), getattr(L, gran), n, 3, 5, 1, 64)
+
+
+@pytest.mark.parametrize("gran", GRANS)
+def test_all_256_alignment_pairs(rt, L, orc, env, gran):
+    for n in (1, 15, 16, 17, 100, 1000):
+        for soff in range(16):
+            for doff in range(16):
+                run_case(rt, L, orc, env, L.PUT, getattr(L, gran), n, soff, doff, 1, 128)
+
+
+def test_sizes_to_4096_one_alignment_each(rt, L, orc, env):
+    rng = np.random.default_rng(0)
+    for n in range(301, 4097, 7):
+        run_case(rt, L, orc, env, L.PUT, L.WG, n, int(rng.integers(16)), int(rng.integers(16)), 1, 256)
+        run_case(rt, L, orc, env, L.GET, L.WAVE, n, int(rng.integers(16)), int(rng.integers(16)), 1, 64)
+
+
+@pytest.mark.parametrize("wg_size", [1, 2, 4, 8, 16, 32, 64, 128, 256, 512, 768, 1024])
+def test_block_sizes_iota(rt, L, orc, env, wg_size):
+    """tests/unit_tests/ipc_impl_simple_fine_gtest.cpp:71-177: work-group copies
+    with block sizes 1..1024 (and 768)."""
+    for n in (32 * 4, 4099):
+        run_case(rt, L, orc, env, L.PUT, L.WG, n, 0, 0, 1, wg_size)
+        run_case(rt, L, orc, env, L.GET, L.WG, n, 0, 0, 1, wg_size)
+
+
+@pytest.mark.parametrize("lanes", [1, 2, 3, 7, 31, 32, 33, 63, 64])
+def test_wave_lane_counts(rt, L, orc, env, lanes):
+    """Wavefront copies with 1..64 active lanes (same gtest, wave fixtures)."""
+    for n in (128, 1027):
+        run_case(rt, L, orc, env, L.PUT, L.WAVE, n, 1, 2, 1, lanes)
+        run_case(rt, L, orc, env, L.GET, L.WAVE, n, 1, 2, 1, lanes)
+
+
+@pytest.mark.parametrize("gran", GRANS)
+def test_tiled_multi_group_transfers(rt, L, orc, env, gran):
+    """tests/functional_tests/extended_primitives.cpp:49-51: several groups each
+    moving their own tile."""
+    for n, n_wgs, wg, tile in [(1 << 16, 8, 256, 0), (100001, 7, 192, 0), (1 << 20, 64, 256, 4096),
+                               (5000, 4, 64, 17)]:
+        run_case(rt, L, orc, env, L.PUT, getattr(L, gran), n, 1, 9, n_wgs, wg, tile=tile)
+        run_case(rt, L, orc, env, L.GET, getattr(L, gran), n, 6, 0, n_wgs, wg, tile=tile)
+
+
+def test_every_pe_pair(rt, L, orc, env):
+    for me in range(P):
+        for pe in range(P):
+            run_case(rt, L, orc, env, L.PUT, L.WG, 777, 1, 1, 2, 128, my_pe=me, pe=pe)
+    for me in (0, 3, 7):
+        for pe in (0, 5):
+            run_case(rt, L, orc, env, L.GET, L.WG, 777, 1, 1, 2, 128, my_pe=me, pe=pe)
+
+
+def test_powers_of_two_to_256mib(rt, L, orc):
+    """The bandwidth curve's message sizes, 8 B .. 256 MiB, checked whole:
+    device-API work-group put from all CUs, and the host-initiated copy."""
+    l = rt.up(P, HEAP)
+    big = 256 << 20
+    src, dst = l.malloc(big), l.malloc(big)
+    assert src and dst
+    host = orc.fill_u8(big, 0, 5)
+    rt.put_bytes(src, host)
+    for k in range(3, 29):
+        n = 1 << k
+        for mode in ("device", "host"):
+            l.fill(l.pe_ptr(dst, 2), 0, n + 16)
+            if mode == "device":
+                assert l.rma(L.PUT, L.WG, dst, src, n, 0, 0, 2, min(1024, max(1, n // 4096)), 256, 1, None) == 0
+            else:
+                assert l.putmem(dst, src, n, 0, 2, None) == 0
+            l.stream_sync(None)
+            got = rt.get_bytes(l.pe_ptr(dst, 2), n + 16)
+            assert np.array_equal(got[:n], host[:n]), (k, mode)
+            assert not got[n:].any(), (k, mode)
+    # getmem, misaligned, large
+    n = (64 << 20) + 13
+    l.fill(dst, 0, n + 32)
+    assert l.getmem(dst + 3, l.pe_ptr(src, 0) + 5, n, 0, 0, None) == 0
+    l.stream_sync(None)
+    got = rt.get_bytes(dst, n + 32)
+    assert np.array_equal(got[3:3 + n], host[5:5 + n]) and not got[:3].any() and not got[3 + n:].any()
+    l.free(src)
+    l.free(dst)
+
+
+def test_argument_errors_launch_nothing(rt, L, env):
+    l = env["l"]
+    src, dst = env["src"], env["dst"]
+    assert l.rma(L.PUT, L.WG, dst, src, 16, 0, 0, P, 1, 64, 1, None) == -1       # bad PE
+    assert l.rma(L.PUT, L.WG, dst, src, 16, 0, 0, 1, 1, 2048, 1, None) == -1     # bad block
+    assert l.rma(L.PUT, L.WG, None, src, 16, 0, 0, 1, 1, 64, 1, None) == -1      # null dest
+    assert l.rma(L.PUT, L.WG, dst, src, HEAP + 1, 0, 0, 1, 1, 64, 1, None) == -1 # beyond the slice
+    assert l.rma(L.PUT, L.WG, l.pe_ptr(dst, 1), src, 16, 0, 0, 1, 1, 64, 1, None) == -1  # not my_pe's address
+    assert l.putmem(dst, src, HEAP, 0, 1, None) == -1
+    assert l.rma(7, L.WG, dst, src, 16, 0, 0, 1, 1, 64, 1, None) == -1

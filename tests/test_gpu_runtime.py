@@ -1,0 +1,130 @@
+"""H1-H3, X2: bring-up, symmetric allocation on the device heap, PE
+addressing and teams through the C entry points."""
+import ctypes
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def test_malloc_matches_the_oracle_allocator(rt, L, orc):
+    l = rt.up(4, 1 << 26)
+    base = l.malloc(1)
+    l.free(base)
+    model = orc.Heap(base, 1 << 26)
+    assert model.alloc(1) == base  # replay what the device heap has seen so far
+    model.free(base)
+    rng = np.random.default_rng(0)
+    live = []
+    for _ in range(300):
+        if live and rng.random() < 0.4:
+            p = live.pop(int(rng.integers(len(live))))
+            l.free(p)
+            model.free(p)
+        else:
+            req = int(rng.integers(0, 1 << int(rng.integers(1, 25))))
+            got = l.malloc(req) or 0
+            assert got == model.alloc(req), req
+            if got:
+                live.append(got)
+        assert l.heap_used() == model.used()
+        assert l.heap_avail() == (1 << 26) - model.used()
+    assert l.heap_size() == 1 << 26
+    for p in live:
+        l.free(p)
+    assert l.heap_used() == 0
+    assert l.malloc(0) is None and l.malloc((1 << 26) + 1) is None
+    l.free(None)  # ignored
+
+
+def test_same_offset_on_every_pe_and_slices_do_not_overlap(rt, L):
+    l = rt.up(8, 1 << 24)
+    stride = l.pe_stride()
+    assert stride >= 1 << 24 and stride % (2 << 20) == 0
+    a = l.malloc(1000)
+    ptrs = [l.pe_ptr(a, p) for p in range(8)]
+    assert ptrs == [a + p * stride for p in range(8)]
+    for p in range(8):
+        l.set_pe(p)
+        b = l.malloc(64)
+        assert b == l.pe_ptr(b, p) and (b - a) % stride == (l.pe_ptr(b, 0) - a)
+        assert l.my_pe() == p
+        l.free(b)
+    l.set_pe(0)
+    assert l.pe_ptr(a, 8) is None and l.pe_ptr(a + 8 * stride, 0) is None
+    # a write through one PE's address is seen only there
+    for p in range(8):
+        l.fill(ptrs[p], p + 1, 1000)
+    for p in range(8):
+        buf = np.empty(1000, np.uint8)
+        l.copy_out(buf.ctypes.data, ptrs[p], 1000)
+        assert (buf == p + 1).all()
+    l.free(a)
+
+
+def test_teams(rt, L, orc):
+    """src/rocshmem.cpp:193-319 and tests/sos_tests/shmem_team_translate.cpp."""
+    l = rt.up(8, 1 << 24)
+    world = l.team_world()
+    assert l.team_n_pes(world) == 8 and l.team_my_pe(world) == 0
+    assert l.team_n_pes(None) == -1 and l.team_my_pe(None) == -1
+    t2, t3, bad = ctypes.c_void_p(), ctypes.c_void_p(), ctypes.c_void_p()
+    assert l.team_split_strided(world, 0, 2, 4, ctypes.byref(t2)) == 0
+    assert l.team_split_strided(world, 0, 3, 3, ctypes.byref(t3)) == 0
+    for args in [(-1, 1, 2), (8, 1, 1), (0, 0, 2), (0, 1, 0), (0, 1, 9), (2, 3, 3)]:
+        assert l.team_split_strided(world, *args, ctypes.byref(bad)) == -1 and not bad.value
+    for me in range(8):
+        l.set_pe(me)
+        a, b = l.team_on(t2, me), l.team_on(t3, me)
+        assert (a is not None) == (me % 2 == 0) and (b is not None) == (me % 3 == 0)
+        if a:
+            assert l.team_my_pe(a) == me // 2 and l.team_n_pes(a) == 4
+        if a and b:
+            assert l.team_translate_pe(a, l.team_my_pe(a), b) == me // 3
+        elif a:
+            assert l.team_translate_pe(a, l.team_my_pe(a), t3) == -1
+    l.set_pe(0)
+    assert l.team_translate_pe(None, 0, t2) == -1
+    # a split of a strided parent composes with it
+    t22 = ctypes.c_void_p()
+    assert l.team_split_strided(t2, 1, 2, 2, ctypes.byref(t22)) == 0   # world PEs 2, 6
+    assert not t22.value  # PE 0 is not a member
+    l.set_pe(6)
+    assert l.team_split_strided(l.team_on(t2, 6), 1, 2, 2, ctypes.byref(t22)) == 0
+    assert l.team_n_pes(t22) == 2 and l.team_my_pe(t22) == 1
+    assert l.team_translate_pe(t22, 0, l.team_world()) == 2
+    l.set_pe(0)
+    for t in (t2, t3):
+        l.team_destroy(t)
+
+
+def test_team_pool_exhaustion(rt, L):
+    """ROCSHMEM_MAX_NUM_TEAMS - 1 user teams (39 by default), then -1
+    (tests/functional_tests/team_ctx_infra_tester.cpp:31-32, src/rocshmem.cpp:229-234)."""
+    l = rt.up(2, 1 << 22)
+    teams = []
+    for _ in range(39):
+        t = ctypes.c_void_p()
+        assert l.team_split_strided(l.team_world(), 0, 1, 2, ctypes.byref(t)) == 0 and t.value
+        teams.append(t)
+    assert len({t.value for t in teams}) == 39
+    t = ctypes.c_void_p()
+    assert l.team_split_strided(l.team_world(), 0, 1, 2, ctypes.byref(t)) == -1 and not t.value
+    l.team_destroy(teams.pop())
+    assert l.team_split_strided(l.team_world(), 0, 1, 2, ctypes.byref(t)) == 0 and t.value
+    for x in teams + [t]:
+        l.team_destroy(x)
+
+
+def test_reinit_and_environment_defaults(rt, L, monkeypatch):
+    rt.down()
+    l = L.load()
+    monkeypatch.setenv("ROCSHMEM_EMU_NPES", "3")
+    monkeypatch.setenv("ROCSHMEM_HEAP_SIZE", str(1 << 22))
+    assert l.n_pes() == 3           # before init
+    assert l.init(0, 0) == 0
+    assert l.n_pes() == 3 and l.heap_size() == 1 << 22
+    l.finalize()
+    monkeypatch.delenv("ROCSHMEM_EMU_NPES")
+    monkeypatch.delenv("ROCSHMEM_HEAP_SIZE")
