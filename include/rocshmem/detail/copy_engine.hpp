@@ -34,7 +34,7 @@ typedef uint32_t u32_any __attribute__((aligned(1)));
 typedef uint16_t u16_any __attribute__((aligned(1)));
 
 // Messages at least this large are stored with the non-temporal hint.
-constexpr size_t kNonTemporalBytes = size_t{1} << 20;
+constexpr size_t kNonTemporalBytes = size_t{64} << 10;
 
 template <bool kNonTemporal>
 __device__ __forceinline__ void store16(char *p, u32x4 v) {

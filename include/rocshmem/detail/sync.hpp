@@ -63,13 +63,125 @@ __device__ __forceinline__ void store_through(T *p, T v) {
 // ---- atomic memory operations on an already-translated address -----------
 // Each is one device-wide RMW; the memory order is acquire-release so an AMO
 // can publish or consume data the way the reference's seq_cst ones do.
+// One RMW per lane, straight to memory.
 template <typename T>
-__device__ __forceinline__ T amo_fetch_add(T *p, T v) {
+__device__ __forceinline__ T amo_fetch_add_each(T *p, T v) {
   return __hip_atomic_fetch_add(p, v, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
 }
 template <typename T>
-__device__ __forceinline__ void amo_add(T *p, T v) {
+__device__ __forceinline__ void amo_add_each(T *p, T v) {
   (void)__hip_atomic_fetch_add(p, v, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+__device__ __forceinline__ unsigned lane_index() {
+  return __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+}
+template <typename T>
+__device__ __forceinline__ T read_lane(T v, int lane) {
+  if constexpr (sizeof(T) == 8) {
+    unsigned long long b;
+    __builtin_memcpy(&b, &v, 8);
+    const unsigned lo = __builtin_amdgcn_readlane(static_cast<unsigned>(b), lane);
+    const unsigned hi = __builtin_amdgcn_readlane(static_cast<unsigned>(b >> 32), lane);
+    b = (static_cast<unsigned long long>(hi) << 32) | lo;
+    T out;
+    __builtin_memcpy(&out, &b, 8);
+    return out;
+  } else {
+    unsigned b;
+    __builtin_memcpy(&b, &v, 4);
+    b = __builtin_amdgcn_readlane(b, lane);
+    T out;
+    __builtin_memcpy(&out, &b, 4);
+    return out;
+  }
+}
+// Value of `v` in lane `lane` (which must be active), lane index per lane.
+template <typename T>
+__device__ __forceinline__ T from_lane(T v, int lane) {
+  if constexpr (sizeof(T) == 8) {
+    unsigned long long b;
+    __builtin_memcpy(&b, &v, 8);
+    const unsigned lo = __builtin_amdgcn_ds_bpermute(lane << 2, static_cast<int>(b));
+    const unsigned hi = __builtin_amdgcn_ds_bpermute(lane << 2, static_cast<int>(b >> 32));
+    b = (static_cast<unsigned long long>(hi) << 32) | lo;
+    T out;
+    __builtin_memcpy(&out, &b, 8);
+    return out;
+  } else {
+    int b;
+    __builtin_memcpy(&b, &v, 4);
+    b = __builtin_amdgcn_ds_bpermute(lane << 2, b);
+    T out;
+    __builtin_memcpy(&out, &b, 4);
+    return out;
+  }
+}
+
+// Wavefront-aggregated add.  Lanes of the calling wavefront that target the
+// same word are merged: the lowest such lane issues ONE RMW with the sum, and
+// every lane of the group receives base + (sum of the group's lower lanes) —
+// exactly what it would have fetched had the group's operations run back to
+// back in lane order, so the fetched values remain a valid serialisation.
+// A hot word (skewed address streams) then costs one memory-side atomic per
+// wavefront instead of one per lane.  Groups are found by peeling: take the
+// first unassigned lane, ballot for its address, repeat; the search stops
+// early once kMissBudget lanes in a row turned out to be alone, which keeps
+// the cost flat for address streams without collisions.
+template <typename T, bool kFetch>
+__device__ __forceinline__ T amo_add_wave(T *p, T v) {
+  constexpr int kMissBudget = 6;
+  const unsigned lane = lane_index();
+  const unsigned long long addr = reinterpret_cast<unsigned long long>(p);
+  unsigned long long rem = __ballot(1);
+  int leader = static_cast<int>(lane);
+  T prefix = static_cast<T>(0);
+  T total = v;
+  int misses = 0;
+  while (rem && misses < kMissBudget) {
+    const int l = __ffsll(static_cast<long long>(rem)) - 1;
+    const unsigned long long a = read_lane(addr, l);
+    const bool mine = addr == a;
+    const unsigned long long same = __ballot(mine);
+    if (same & (same - 1)) {  // two or more lanes share this word
+      misses = 0;
+      T run = static_cast<T>(0);
+      unsigned long long m = same;
+      while (m) {
+        const int j = __ffsll(static_cast<long long>(m)) - 1;
+        const T vj = read_lane(v, j);
+        if (static_cast<int>(lane) == j) prefix = run;
+        run = static_cast<T>(run + vj);
+        m &= m - 1;
+      }
+      if (mine) {
+        leader = l;
+        total = run;
+      }
+    } else {
+      ++misses;
+    }
+    rem &= ~same;
+  }
+  T base = static_cast<T>(0);
+  if (leader == static_cast<int>(lane)) {
+    if constexpr (kFetch) base = amo_fetch_add_each(p, total);
+    else amo_add_each(p, total);
+  }
+  if constexpr (kFetch) {
+    base = from_lane(base, leader);
+    return static_cast<T>(base + prefix);
+  }
+  return base;
+}
+
+template <typename T>
+__device__ __forceinline__ T amo_fetch_add(T *p, T v) {
+  return amo_add_wave<T, true>(p, v);
+}
+template <typename T>
+__device__ __forceinline__ void amo_add(T *p, T v) {
+  (void)amo_add_wave<T, false>(p, v);
 }
 template <typename T>
 __device__ __forceinline__ T amo_fetch_cas(T *p, T cond, T v) {

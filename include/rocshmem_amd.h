@@ -284,17 +284,18 @@ int rocshmem_amd_pingpong(void *buf, uint64_t *sig, size_t nbytes, int iters, in
                           rocshmem_amd_stream_t stream);
 
 /* MoE-style dispatch with put_signal.  For every ordered pair (s, d) of the P
- * world PEs, `wgs_per_pair` work-groups acting for s send rows
- * [send_row[s*P+d], +count[s*P+d]) of s's `send` buffer to rows starting at
- * recv_row[s*P+d] of d's `recv` buffer with rocshmem_putmem_signal_wg, adding
- * the number of rows they sent to d's sig[s]; one more work-group per PE d
- * waits with rocshmem_ulong_wait_until(sig[s], GE, count[s*P+d]) for every s.
+ * world PEs, rows [send_row[s*P+d], +count[s*P+d]) of s's `send` buffer go to
+ * rows starting at recv_row[s*P+d] of d's `recv` buffer, rows_per_call rows per
+ * rocshmem_putmem_signal_wg call, each call adding the number of rows it sent
+ * to d's sig[s]; work-groups acting for the sources share out the list of all
+ * calls, and one more work-group per PE d waits with
+ * rocshmem_ulong_wait_until(sig[s], GE, count[s*P+d]) for every s.
  * count/send_row/recv_row: device arrays of P*P uint32.  send/recv/sig:
- * addresses on PE 0. */
+ * addresses on PE 0.  sig must be zero when the kernel starts. */
 int rocshmem_amd_dispatch_put_signal(void *recv, const void *send, uint64_t *sig,
                                      const uint32_t *count, const uint32_t *send_row,
                                      const uint32_t *recv_row, size_t row_bytes,
-                                     int wgs_per_pair, int wg_size,
+                                     int rows_per_call, int wg_size,
                                      rocshmem_amd_stream_t stream);
 
 /* rocshmem_<T>_test / _wait_until / _wait_until_any / _all / _some

@@ -272,41 +272,50 @@ struct DispatchArgs {
   const char *send0;
   uint64_t *sig0;
   const uint32_t *count, *send_row, *recv_row;
+  const uint32_t *call_start;  // [P*P+1] first call number of every pair
   size_t row_bytes;
   uint64_t pe_stride;
   int np;
-  int wgs_per_pair;
+  uint32_t rows_per_call;
+  uint32_t n_calls;
   detail::Context *ctx_row;
   detail::Team *world_row;
 };
 
+// Work-groups walk the list of all calls (a call = up to rows_per_call rows of
+// one (source, destination) pair), so a skewed routing table still keeps every
+// CU busy; the last P work-groups are the receivers.
 __global__ void dispatch_kernel(DispatchArgs a) {
-  const int P = a.np, W = a.wgs_per_pair;
-  const int senders = P * P * W;
-  const int b = blockIdx.x;
-  if (b < senders) {
-    const int w = b % W, pair = b / W;
-    const int d = pair % P, s = pair / P;
-    const uint32_t cnt = a.count[s * P + d];
-    // Rows of this pair are shared out over its W work-groups.
-    const uint32_t per = (cnt + W - 1) / W;
-    const uint32_t lo = per * w < cnt ? per * w : cnt;
-    const uint32_t hi = lo + per < cnt ? lo + per : cnt;
-    rocshmem_ctx_t ctx{a.ctx_row + s, &a.world_row[s].wrt_world};
-    char *recv_s = a.recv0 + static_cast<uint64_t>(s) * a.pe_stride;
-    const char *send_s = a.send0 + static_cast<uint64_t>(s) * a.pe_stride;
-    uint64_t *sig_s = reinterpret_cast<uint64_t *>(reinterpret_cast<char *>(a.sig0) +
-                                                   static_cast<uint64_t>(s) * a.pe_stride);
-    rocshmem_ctx_putmem_signal_wg(
-        ctx, recv_s + (static_cast<size_t>(a.recv_row[s * P + d]) + lo) * a.row_bytes,
-        send_s + (static_cast<size_t>(a.send_row[s * P + d]) + lo) * a.row_bytes,
-        static_cast<size_t>(hi - lo) * a.row_bytes, sig_s + s, static_cast<uint64_t>(hi - lo),
-        ROCSHMEM_SIGNAL_ADD, d);
+  const int P = a.np;
+  const unsigned senders = gridDim.x - P;
+  if (blockIdx.x < senders) {
+    for (uint32_t c = blockIdx.x; c < a.n_calls; c += senders) {
+      // pair whose call range holds c: P*P+1 sorted entries, binary search
+      int lo = 0, hi = P * P;
+      while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (a.call_start[mid] <= c) lo = mid; else hi = mid;
+      }
+      const int pair = lo, s = pair / P, d = pair % P;
+      const uint32_t first = (c - a.call_start[pair]) * a.rows_per_call;
+      const uint32_t cnt = a.count[pair];
+      const uint32_t rows = cnt - first < a.rows_per_call ? cnt - first : a.rows_per_call;
+      rocshmem_ctx_t ctx{a.ctx_row + s, &a.world_row[s].wrt_world};
+      char *recv_s = a.recv0 + static_cast<uint64_t>(s) * a.pe_stride;
+      const char *send_s = a.send0 + static_cast<uint64_t>(s) * a.pe_stride;
+      uint64_t *sig_s = reinterpret_cast<uint64_t *>(reinterpret_cast<char *>(a.sig0) +
+                                                     static_cast<uint64_t>(s) * a.pe_stride);
+      rocshmem_ctx_putmem_signal_wg(
+          ctx, recv_s + (static_cast<size_t>(a.recv_row[pair]) + first) * a.row_bytes,
+          send_s + (static_cast<size_t>(a.send_row[pair]) + first) * a.row_bytes,
+          static_cast<size_t>(rows) * a.row_bytes, sig_s + s, static_cast<uint64_t>(rows),
+          ROCSHMEM_SIGNAL_ADD, d);
+    }
   } else {
-    const int d = b - senders;
+    const int d = blockIdx.x - senders;
     uint64_t *sig_d = reinterpret_cast<uint64_t *>(reinterpret_cast<char *>(a.sig0) +
                                                    static_cast<uint64_t>(d) * a.pe_stride);
-    // Lane s of the first wavefront waits for sender s.
+    // Lane s of the receiver waits for sender s.
     for (int s = threadIdx.x; s < P; s += blockDim.x)
       rocshmem_ulong_wait_until(reinterpret_cast<unsigned long *>(sig_d + s), ROCSHMEM_CMP_GE,
                                 static_cast<unsigned long>(a.count[s * P + d]));
@@ -602,27 +611,31 @@ int rocshmem_amd_pingpong(void *buf, uint64_t *sig, size_t nbytes, int iters, in
 int rocshmem_amd_dispatch_put_signal(void *recv, const void *send, uint64_t *sig,
                                      const uint32_t *count, const uint32_t *send_row,
                                      const uint32_t *recv_row, size_t row_bytes,
-                                     int wgs_per_pair, int wg_size,
+                                     int rows_per_call, int wg_size,
                                      rocshmem_amd_stream_t stream) {
   auto &r = runtime::rt();
-  if (!r.live || wgs_per_pair < 1 || !valid_launch(1, wg_size) || !row_bytes) return -1;
+  if (!r.live || rows_per_call < 1 || !valid_launch(1, wg_size) || !row_bytes) return -1;
   if (!count || !send_row || !recv_row) return -1;
-  {
-    // Bounds of every pair's rows, from a host copy of the three tables.
-    const size_t pp = static_cast<size_t>(r.npes) * r.npes;
-    std::vector<uint32_t> h(3 * pp);
-    DRV_CHECK_HIP(hipMemcpy(h.data(), count, pp * 4, hipMemcpyDeviceToHost));
-    DRV_CHECK_HIP(hipMemcpy(h.data() + pp, send_row, pp * 4, hipMemcpyDeviceToHost));
-    DRV_CHECK_HIP(hipMemcpy(h.data() + 2 * pp, recv_row, pp * 4, hipMemcpyDeviceToHost));
-    size_t max_send = 0, max_recv = 0;
-    for (size_t i = 0; i < pp; ++i) {
-      max_send = std::max<size_t>(max_send, static_cast<size_t>(h[pp + i]) + h[i]);
-      max_recv = std::max<size_t>(max_recv, static_cast<size_t>(h[2 * pp + i]) + h[i]);
-    }
-    if (!sym_ok_on(send, max_send * row_bytes, 0) || !sym_ok_on(recv, max_recv * row_bytes, 0) ||
-        !sym_ok_on(sig, 8 * static_cast<size_t>(r.npes), 0))
-      return -1;
+  // Bounds of every pair's rows and the call list, from a host copy of the tables.
+  const size_t pp = static_cast<size_t>(r.npes) * r.npes;
+  std::vector<uint32_t> h(3 * pp);
+  DRV_CHECK_HIP(hipMemcpy(h.data(), count, pp * 4, hipMemcpyDeviceToHost));
+  DRV_CHECK_HIP(hipMemcpy(h.data() + pp, send_row, pp * 4, hipMemcpyDeviceToHost));
+  DRV_CHECK_HIP(hipMemcpy(h.data() + 2 * pp, recv_row, pp * 4, hipMemcpyDeviceToHost));
+  size_t max_send = 0, max_recv = 0;
+  std::vector<uint32_t> call_start(pp + 1, 0);
+  for (size_t i = 0; i < pp; ++i) {
+    max_send = std::max<size_t>(max_send, static_cast<size_t>(h[pp + i]) + h[i]);
+    max_recv = std::max<size_t>(max_recv, static_cast<size_t>(h[2 * pp + i]) + h[i]);
+    call_start[i + 1] = call_start[i] + (h[i] + rows_per_call - 1) / rows_per_call;
   }
+  if (!sym_ok_on(send, max_send * row_bytes, 0) || !sym_ok_on(recv, max_recv * row_bytes, 0) ||
+      !sym_ok_on(sig, 8 * static_cast<size_t>(r.npes), 0))
+    return -1;
+  uint32_t *d_calls;
+  hipStream_t s = as_stream(stream);
+  DRV_CHECK_HIP(hipMallocAsync(reinterpret_cast<void **>(&d_calls), (pp + 1) * 4, s));
+  DRV_CHECK_HIP(hipMemcpyAsync(d_calls, call_start.data(), (pp + 1) * 4, hipMemcpyHostToDevice, s));
   DispatchArgs a;
   a.recv0 = static_cast<char *>(recv);
   a.send0 = static_cast<const char *>(send);
@@ -630,15 +643,20 @@ int rocshmem_amd_dispatch_put_signal(void *recv, const void *send, uint64_t *sig
   a.count = count;
   a.send_row = send_row;
   a.recv_row = recv_row;
+  a.call_start = d_calls;
   a.row_bytes = row_bytes;
   a.pe_stride = r.pe_stride;
   a.np = r.npes;
-  a.wgs_per_pair = wgs_per_pair;
+  a.rows_per_call = static_cast<uint32_t>(rows_per_call);
+  a.n_calls = call_start[pp];
   a.ctx_row = r.d_default_ctx;
   a.world_row = r.d_teams;
-  const int grid = r.npes * r.npes * wgs_per_pair + r.npes;
-  hipLaunchKernelGGL(dispatch_kernel, dim3(grid), dim3(wg_size), 0, as_stream(stream), a);
+  const uint32_t max_senders = 256 * 16;
+  const uint32_t senders = a.n_calls < max_senders ? (a.n_calls ? a.n_calls : 1) : max_senders;
+  hipLaunchKernelGGL(dispatch_kernel, dim3(senders + r.npes), dim3(wg_size), 0, s, a);
   DRV_CHECK_HIP(hipGetLastError());
+  // call_start is pageable host memory: the copy above has completed by now.
+  DRV_CHECK_HIP(hipFreeAsync(d_calls, s));
   return 0;
 }
 

@@ -192,7 +192,7 @@ int Runtime::init(int want_npes, size_t want_heap) {
   state.world_team = d_teams;
   state.ctx_pool = d_pools;
   state.ws_base = d_ws;
-  state.nt_bytes = env_size("ROCSHMEM_NT_THRESHOLD", size_t{1} << 20);
+  state.nt_bytes = env_size("ROCSHMEM_NT_THRESHOLD", size_t{64} << 10);
   live = true;
   push_state();
   ROCSHMEM_TEAM_WORLD = team_handle(0, acting_pe);

@@ -307,8 +307,8 @@ def zipf_routing(orc, P, tokens, experts, topk, seed):
     return counts, dest_of
 
 
-@pytest.mark.parametrize("wgs_per_pair", [1, 4])
-def test_dispatch_put_signal(rt, L, orc, wgs_per_pair):
+@pytest.mark.parametrize("rows_per_call", [1, 7, 64, 100000])
+def test_dispatch_put_signal(rt, L, orc, rows_per_call):
     """MoE-dispatch pattern at reduced size: per-pair row counts from top-8 of
     256 Zipf(1.1) routing; rows packed per destination; receivers wait on the
     per-source signal.  Rows byte-exact, signals equal the counts."""
@@ -331,7 +331,7 @@ def test_dispatch_put_signal(rt, L, orc, wgs_per_pair):
         l.fill(l.pe_ptr(recv, s), 0, max_rows * row)
         l.fill(l.pe_ptr(sig, s), 0, 8 * P)
     d_cnt, d_srow, d_rrow = rt.dev_array(counts), rt.dev_array(send_row), rt.dev_array(recv_row)
-    assert l.dispatch_put_signal(recv, send, sig, d_cnt, d_srow, d_rrow, row, wgs_per_pair, 256,
+    assert l.dispatch_put_signal(recv, send, sig, d_cnt, d_srow, d_rrow, row, rows_per_call, 256,
                                  None) == 0
     l.stream_sync(None)
     for d in range(P):
