@@ -38,6 +38,9 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--quick", action="store_true", help="headline only, no CPU baseline")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also run three 256 MiB device-to-device hipMemcpy calls (the HIP "
+                         "runtime's copy kernel) for calibrating FETCH_SIZE / WRITE_SIZE")
     return ap.parse_args()
 
 
@@ -321,6 +324,12 @@ def main():
     allc = {}
     if not a.quick:
         allc["dispatch_put_signal"] = dispatch_config(b, a.steps)
+    if a.calibrate:
+        cs, cd = b.l.malloc(256 * MiB), b.l.malloc(256 * MiB)
+        for _ in range(3):
+            b.l.copy_dev(cd, cs, 256 * MiB)
+        b.l.free(cs)
+        b.l.free(cd)
     head = headline(b, a.steps, a.warmup)
     if not a.quick:
         allc["to_all_P8_64Mi"] = to_all_configs(b, a.steps, a.warmup)

@@ -155,6 +155,9 @@ int rocshmem_amd_dev_free(void *ptr);
 int rocshmem_amd_copy_in(void *dst_dev, const void *src_host, size_t n);
 int rocshmem_amd_copy_out(void *dst_host, const void *src_dev, size_t n);
 int rocshmem_amd_fill(void *dst_dev, int byte, size_t n);
+/* hipMemcpy device-to-device by the HIP runtime's own copy kernel: a plain copy
+ * of known size to calibrate hardware byte counters against. */
+int rocshmem_amd_copy_dev(void *dst_dev, const void *src_dev, size_t n);
 int rocshmem_amd_stream_sync(rocshmem_amd_stream_t stream);
 /* hipEvent pair on `stream`; elapsed time in milliseconds. */
 void *rocshmem_amd_timer_create(void);

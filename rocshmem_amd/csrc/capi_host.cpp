@@ -119,6 +119,11 @@ int rocshmem_amd_fill(void *dst_dev, int byte, size_t n) {
   if (n) DRV_CHECK_HIP(hipMemset(dst_dev, byte, n));
   return 0;
 }
+int rocshmem_amd_copy_dev(void *dst_dev, const void *src_dev, size_t n) {
+  if (n && (!dst_dev || !src_dev)) return -1;
+  if (n) DRV_CHECK_HIP(hipMemcpy(dst_dev, src_dev, n, hipMemcpyDeviceToDevice));
+  return 0;
+}
 int rocshmem_amd_stream_sync(rocshmem_amd_stream_t stream) {
   DRV_CHECK_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
   return 0;

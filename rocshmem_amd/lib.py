@@ -55,6 +55,7 @@ SIGNATURES = {
     "rocshmem_amd_copy_in": (_i, [_vp, _vp, _sz]),
     "rocshmem_amd_copy_out": (_i, [_vp, _vp, _sz]),
     "rocshmem_amd_fill": (_i, [_vp, _i, _sz]),
+    "rocshmem_amd_copy_dev": (_i, [_vp, _vp, _sz]),
     "rocshmem_amd_stream_sync": (_i, [_vp]),
     "rocshmem_amd_timer_create": (_vp, []),
     "rocshmem_amd_timer_start": (_i, [_vp, _vp]),

@@ -9,6 +9,12 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 
+# Slices are packed (stride = heap size) in the tests so that bring-up stays
+# quick; the spread 16 GiB layout only changes bandwidth, not results, and is
+# exercised by the full-size test and by bench.py.
+os.environ.setdefault("ROCSHMEM_EMU_PE_STRIDE", "1")
+
+
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 

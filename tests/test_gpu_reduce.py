@@ -232,12 +232,15 @@ def test_unsupported_combinations_are_rejected(rt, L):
 
 @pytest.mark.parametrize("dtype_name,op_name", [("FLOAT", "SUM"), ("BF16", "SUM"), ("FLOAT", "MAX"),
                                                 ("LONG", "XOR")])
-def test_full_size_64mi_properties(rt, L, orc, dtype_name, op_name):
-    """P=8 x 64 Mi elements.  Inputs are made on the CPU for windows only; the
+def test_full_size_64mi_properties(rt, L, orc, dtype_name, op_name, monkeypatch):
+    """P=8 x 64 Mi elements, slices in the default spread layout.  Inputs are made on the CPU for windows only; the
     bulk is checked through size-independent properties: all P destinations are
     identical, the windows match the oracle, and for xor reducing the result
     with itself gives zero / reducing twice with P even returns to zero."""
+    monkeypatch.delenv("ROCSHMEM_EMU_PE_STRIDE", raising=False)
+    rt.down()
     l = rt.up(8, 2 << 30)
+    assert l.pe_stride() >= 2 << 30
     n = 1 << 26
     np_t = orc.NP_DTYPE[getattr(orc, dtype_name)]
     es = np.dtype(np_t).itemsize
@@ -265,4 +268,4 @@ def test_full_size_64mi_properties(rt, L, orc, dtype_name, op_name):
         other = rt.get_bytes(l.pe_ptr(b.dst, p), n * es, np_t)
         assert np.array_equal(other.view(np.uint8), first.view(np.uint8)), p
     b.free()
-    rt.up(8, HEAP)
+    rt.down()

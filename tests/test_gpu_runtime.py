@@ -117,6 +117,23 @@ def test_team_pool_exhaustion(rt, L):
         l.team_destroy(x)
 
 
+def test_default_slice_stride_spreads_the_pes(rt, L, monkeypatch):
+    """Without an override the slices sit 16 GiB apart (or as far as half of
+    the device memory allows), never closer than the heap size."""
+    monkeypatch.delenv("ROCSHMEM_EMU_PE_STRIDE", raising=False)
+    rt.down()
+    l = L.load()
+    assert l.init(4, 1 << 24) == 0
+    assert l.pe_stride() == 16 << 30
+    a = l.malloc(64)
+    assert l.pe_ptr(a, 3) - a == 3 * (16 << 30)
+    l.finalize()
+    monkeypatch.setenv("ROCSHMEM_EMU_PE_STRIDE", str(6 << 20))
+    assert l.init(4, 1 << 22) == 0
+    assert l.pe_stride() == 6 << 20
+    l.finalize()
+
+
 def test_reinit_and_environment_defaults(rt, L, monkeypatch):
     rt.down()
     l = L.load()
