@@ -358,7 +358,9 @@ def main():
                    "n_pes": P, "message_bytes": 256 * MiB, "heap_bytes_per_pe": 8 << 30},
         "roofline": {"bound": "hbm", "achieved": round(head["gbs"], 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(head["gbs"] / HBM_PEAK_GBS, 4),
-                     "traffic": None, "kernel": "bulk_copy_kernel<true>",
+                     # FETCH_SIZE + WRITE_SIZE per launch under rocprofv3 --pmc, scaled by the
+                     # HIP runtime's own copy kernel (profiles/bulk_copy_256MiB_hbm_traffic.txt)
+                     "traffic": 536935029, "kernel": "bulk_copy_kernel<true>",
                      "algorithmic_bytes_per_launch": head["bytes_per_step"]},
         "cpu_baseline": cpu,
         "all_configs": allc,
