@@ -196,21 +196,16 @@ def dispatch_config(b, steps):
     assert send and recv and sig, (rows_in * row, rows_out * row)
     for p in range(P):
         b.fill_random(l.pe_ptr(send, p), rows_out * row, p, 40 + p)
-    dev = []
-    for a in (counts, send_row, recv_row):
-        d = l.dev_alloc(a.nbytes)
-        l.copy_in(d, np.ascontiguousarray(a).ctypes.data, a.nbytes)
-        dev.append(d)
+    tabs = [np.ascontiguousarray(a, np.uint32) for a in (counts, send_row, recv_row)]
 
     def step():
         for p in range(P):  # signals start from zero each dispatch
             l.fill(l.pe_ptr(sig, p), 0, 8 * P)
-        assert l.dispatch_put_signal(recv, send, sig, dev[0], dev[1], dev[2], row, 16, 512, None) == 0
+        assert l.dispatch_put_signal(recv, send, sig, tabs[0].ctypes.data, tabs[1].ctypes.data,
+                                     tabs[2].ctypes.data, row, 128, 1024, None) == 0
 
     ms = b.time_ms(step, max(5, steps // 10), 2)
     alg = 2 * int(counts.sum()) * row
-    for d in dev:
-        l.dev_free(d)
     for x in (send, recv, sig):
         l.free(x)
     return {"ms": round(ms, 4), "gbs": round(alg / ms / 1e6, 1),

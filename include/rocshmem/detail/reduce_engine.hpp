@@ -23,6 +23,7 @@
 #include <type_traits>
 
 #include "../rocshmem_common.hpp"
+#include "copy_engine.hpp"
 
 namespace rocshmem {
 
@@ -117,14 +118,35 @@ struct ElemTraits<Bf16Tag> {
   __device__ static uint16_t narrow(float a) { return f32_to_bf16(a); }
 };
 
+// One element of 2, 4 or 8 bytes as a write-through buffer store.
+template <typename S>
+__device__ __forceinline__ void store_elem(__amdgpu_buffer_rsrc_t w, uint32_t off, S v) {
+  if constexpr (sizeof(S) == 2) {
+    uint16_t b;
+    __builtin_memcpy(&b, &v, 2);
+    __builtin_amdgcn_raw_buffer_store_b16(b, w, static_cast<int>(off), 0, kAuxWriteThrough);
+  } else if constexpr (sizeof(S) == 4) {
+    uint32_t b;
+    __builtin_memcpy(&b, &v, 4);
+    __builtin_amdgcn_raw_buffer_store_b32(b, w, static_cast<int>(off), 0, kAuxWriteThrough);
+  } else {
+    typedef uint32_t b64_t __attribute__((ext_vector_type(2)));
+    b64_t b;
+    __builtin_memcpy(&b, &v, 8);
+    __builtin_amdgcn_raw_buffer_store_b64(b, w, static_cast<int>(off), 0, kAuxWriteThrough);
+  }
+}
+
 // Fold elements [lo, hi) across P team members and store the result on all P.
 //   src0 / dst0 : the buffers on team member 0
 //   hop         : bytes from one team member's buffer to the next member's
 //   kP          : P when known at compile time (loads fully unrolled), 0 when
 //                 only `np` is known
-// `lane` of `nlanes` dense cooperating lanes (a work-group or a whole grid).
+// `lane` of `nlanes` dense cooperating lanes (a work-group or a whole grid);
+// (hi - lo) * sizeof(element) must not exceed kWindowBytes.  Results leave as
+// write-through buffer stores, one resource per destination.
 template <typename E, ROCSHMEM_OP Op, int kP, bool kNonTemporal>
-__device__ __forceinline__ void fold_span(
+__device__ __forceinline__ void fold_window(
     typename ElemTraits<E>::storage *dst0,
     const typename ElemTraits<E>::storage *src0, int64_t hop, int np,
     size_t lo, size_t hi, size_t lane, size_t nlanes) {
@@ -133,18 +155,20 @@ __device__ __forceinline__ void fold_span(
   using A = typename Tr::accum;
   constexpr int V = Tr::kPerVec;
   const int P = kP ? kP : np;
+  const size_t win_bytes = (hi - lo) * sizeof(S);
 
   auto src_at = [&](int p, size_t i) -> const S * {
     return reinterpret_cast<const S *>(reinterpret_cast<const char *>(src0 + i) + p * hop);
   };
-  auto dst_at = [&](int p, size_t i) -> S * {
-    return reinterpret_cast<S *>(reinterpret_cast<char *>(dst0 + i) + p * hop);
+  auto dst_window = [&](int p) {
+    return window_of(reinterpret_cast<char *>(dst0 + lo) + p * hop, win_bytes);
   };
   auto scalar_one = [&](size_t i) {
     A acc = Tr::widen(*src_at(0, i));
     for (int p = 1; p < P; ++p) acc = combine<A, Op>(acc, Tr::widen(*src_at(p, i)));
     const S out = Tr::narrow(acc);
-    for (int p = 0; p < P; ++p) *dst_at(p, i) = out;
+    for (int p = 0; p < P; ++p)
+      store_elem<S>(dst_window(p), static_cast<uint32_t>((i - lo) * sizeof(S)), out);
   };
 
   // Elements before the first 16-byte boundary of the destination.
@@ -188,16 +212,31 @@ __device__ __forceinline__ void fold_span(
 #pragma unroll
       for (int e = 0; e < V; ++e) out.e[e] = Tr::narrow(acc[e]);
     }
-    for (int p = 0; p < P; ++p) {
-      if constexpr (kNonTemporal)
-        __builtin_nontemporal_store(out.raw, reinterpret_cast<r_u32x4 *>(dst_at(p, i)));
-      else
-        *reinterpret_cast<r_u32x4 *>(dst_at(p, i)) = out.raw;
+    const uint32_t off = static_cast<uint32_t>((i - lo) * sizeof(S));
+    if constexpr (kP != 0) {
+#pragma unroll
+      for (int p = 0; p < kP; ++p) store16<kNonTemporal>(dst_window(p), off, out.raw);
+    } else {
+      for (int p = 0; p < P; ++p) store16<kNonTemporal>(dst_window(p), off, out.raw);
     }
   }
 
   const size_t tlo = vlo + nvec * V;
   for (size_t k = tlo + lane; k < hi; k += nlanes) scalar_one(k);
+}
+
+// Any range: windows of at most kWindowBytes.
+template <typename E, ROCSHMEM_OP Op, int kP, bool kNonTemporal>
+__device__ __forceinline__ void fold_span(
+    typename ElemTraits<E>::storage *dst0,
+    const typename ElemTraits<E>::storage *src0, int64_t hop, int np,
+    size_t lo, size_t hi, size_t lane, size_t nlanes) {
+  constexpr size_t kWin = kWindowBytes / sizeof(typename ElemTraits<E>::storage);
+  while (hi - lo > kWin) {
+    fold_window<E, Op, kP, kNonTemporal>(dst0, src0, hop, np, lo, lo + kWin, lane, nlanes);
+    lo += kWin;
+  }
+  fold_window<E, Op, kP, kNonTemporal>(dst0, src0, hop, np, lo, hi, lane, nlanes);
 }
 
 // Dispatch on the team size so the common sizes get fully unrolled loads.

@@ -293,7 +293,8 @@ int rocshmem_amd_pingpong(void *buf, uint64_t *sig, size_t nbytes, int iters, in
  * to d's sig[s]; work-groups acting for the sources share out the list of all
  * calls, and one more work-group per PE d waits with
  * rocshmem_ulong_wait_until(sig[s], GE, count[s*P+d]) for every s.
- * count/send_row/recv_row: device arrays of P*P uint32.  send/recv/sig:
+ * count/send_row/recv_row: host arrays of P*P uint32 (a device copy is kept
+ * and reused while consecutive calls pass the same tables).  send/recv/sig:
  * addresses on PE 0.  sig must be zero when the kernel starts. */
 int rocshmem_amd_dispatch_put_signal(void *recv, const void *send, uint64_t *sig,
                                      const uint32_t *count, const uint32_t *send_row,

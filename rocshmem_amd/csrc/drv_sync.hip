@@ -608,6 +608,20 @@ int rocshmem_amd_pingpong(void *buf, uint64_t *sig, size_t nbytes, int iters, in
   return 0;
 }
 
+// Device copy of the last routing tables seen, so that a dispatch repeated
+// with the same tables only launches.
+namespace {
+struct DispatchTables {
+  std::vector<uint32_t> host;  // count | send_row | recv_row | call_start
+  uint32_t *dev = nullptr;
+  size_t pp = 0;
+  uint32_t rows_per_call = 0;
+  uint32_t n_calls = 0;
+  size_t max_send = 0, max_recv = 0;
+};
+DispatchTables g_tables;
+}  // namespace
+
 int rocshmem_amd_dispatch_put_signal(void *recv, const void *send, uint64_t *sig,
                                      const uint32_t *count, const uint32_t *send_row,
                                      const uint32_t *recv_row, size_t row_bytes,
@@ -616,47 +630,56 @@ int rocshmem_amd_dispatch_put_signal(void *recv, const void *send, uint64_t *sig
   auto &r = runtime::rt();
   if (!r.live || rows_per_call < 1 || !valid_launch(1, wg_size) || !row_bytes) return -1;
   if (!count || !send_row || !recv_row) return -1;
-  // Bounds of every pair's rows and the call list, from a host copy of the tables.
   const size_t pp = static_cast<size_t>(r.npes) * r.npes;
-  std::vector<uint32_t> h(3 * pp);
-  DRV_CHECK_HIP(hipMemcpy(h.data(), count, pp * 4, hipMemcpyDeviceToHost));
-  DRV_CHECK_HIP(hipMemcpy(h.data() + pp, send_row, pp * 4, hipMemcpyDeviceToHost));
-  DRV_CHECK_HIP(hipMemcpy(h.data() + 2 * pp, recv_row, pp * 4, hipMemcpyDeviceToHost));
-  size_t max_send = 0, max_recv = 0;
-  std::vector<uint32_t> call_start(pp + 1, 0);
-  for (size_t i = 0; i < pp; ++i) {
-    max_send = std::max<size_t>(max_send, static_cast<size_t>(h[pp + i]) + h[i]);
-    max_recv = std::max<size_t>(max_recv, static_cast<size_t>(h[2 * pp + i]) + h[i]);
-    call_start[i + 1] = call_start[i] + (h[i] + rows_per_call - 1) / rows_per_call;
+  DispatchTables &t = g_tables;
+  std::vector<uint32_t> h(4 * pp + 1);
+  std::copy(count, count + pp, h.begin());
+  std::copy(send_row, send_row + pp, h.begin() + pp);
+  std::copy(recv_row, recv_row + pp, h.begin() + 2 * pp);
+  const bool same = t.dev && t.pp == pp && t.rows_per_call == static_cast<uint32_t>(rows_per_call) &&
+                    std::equal(h.begin(), h.begin() + 3 * pp, t.host.begin());
+  if (!same) {
+    // Bounds of every pair's rows and the list of calls.
+    t.max_send = t.max_recv = 0;
+    uint32_t calls = 0;
+    for (size_t i = 0; i < pp; ++i) {
+      t.max_send = std::max<size_t>(t.max_send, static_cast<size_t>(h[pp + i]) + h[i]);
+      t.max_recv = std::max<size_t>(t.max_recv, static_cast<size_t>(h[2 * pp + i]) + h[i]);
+      h[3 * pp + i] = calls;
+      calls += (h[i] + rows_per_call - 1) / rows_per_call;
+    }
+    h[4 * pp] = calls;
+    DRV_CHECK_HIP(hipDeviceSynchronize());  // nobody is reading the old tables any more
+    if (t.dev) DRV_CHECK_HIP(hipFree(t.dev));
+    DRV_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&t.dev), h.size() * 4));
+    DRV_CHECK_HIP(hipMemcpy(t.dev, h.data(), h.size() * 4, hipMemcpyHostToDevice));
+    t.host = h;
+    t.pp = pp;
+    t.rows_per_call = static_cast<uint32_t>(rows_per_call);
+    t.n_calls = calls;
   }
-  if (!sym_ok_on(send, max_send * row_bytes, 0) || !sym_ok_on(recv, max_recv * row_bytes, 0) ||
+  if (!sym_ok_on(send, t.max_send * row_bytes, 0) || !sym_ok_on(recv, t.max_recv * row_bytes, 0) ||
       !sym_ok_on(sig, 8 * static_cast<size_t>(r.npes), 0))
     return -1;
-  uint32_t *d_calls;
-  hipStream_t s = as_stream(stream);
-  DRV_CHECK_HIP(hipMallocAsync(reinterpret_cast<void **>(&d_calls), (pp + 1) * 4, s));
-  DRV_CHECK_HIP(hipMemcpyAsync(d_calls, call_start.data(), (pp + 1) * 4, hipMemcpyHostToDevice, s));
   DispatchArgs a;
   a.recv0 = static_cast<char *>(recv);
   a.send0 = static_cast<const char *>(send);
   a.sig0 = sig;
-  a.count = count;
-  a.send_row = send_row;
-  a.recv_row = recv_row;
-  a.call_start = d_calls;
+  a.count = t.dev;
+  a.send_row = t.dev + pp;
+  a.recv_row = t.dev + 2 * pp;
+  a.call_start = t.dev + 3 * pp;
   a.row_bytes = row_bytes;
   a.pe_stride = r.pe_stride;
   a.np = r.npes;
   a.rows_per_call = static_cast<uint32_t>(rows_per_call);
-  a.n_calls = call_start[pp];
+  a.n_calls = t.n_calls;
   a.ctx_row = r.d_default_ctx;
   a.world_row = r.d_teams;
   const uint32_t max_senders = 256 * 16;
   const uint32_t senders = a.n_calls < max_senders ? (a.n_calls ? a.n_calls : 1) : max_senders;
-  hipLaunchKernelGGL(dispatch_kernel, dim3(senders + r.npes), dim3(wg_size), 0, s, a);
+  hipLaunchKernelGGL(dispatch_kernel, dim3(senders + r.npes), dim3(wg_size), 0, as_stream(stream), a);
   DRV_CHECK_HIP(hipGetLastError());
-  // call_start is pageable host memory: the copy above has completed by now.
-  DRV_CHECK_HIP(hipFreeAsync(d_calls, s));
   return 0;
 }
 

@@ -330,9 +330,9 @@ def test_dispatch_put_signal(rt, L, orc, rows_per_call):
         rt.put_bytes(l.pe_ptr(send, s), rows)
         l.fill(l.pe_ptr(recv, s), 0, max_rows * row)
         l.fill(l.pe_ptr(sig, s), 0, 8 * P)
-    d_cnt, d_srow, d_rrow = rt.dev_array(counts), rt.dev_array(send_row), rt.dev_array(recv_row)
-    assert l.dispatch_put_signal(recv, send, sig, d_cnt, d_srow, d_rrow, row, rows_per_call, 256,
-                                 None) == 0
+    counts, send_row, recv_row = (np.ascontiguousarray(a, np.uint32) for a in (counts, send_row, recv_row))
+    assert l.dispatch_put_signal(recv, send, sig, counts.ctypes.data, send_row.ctypes.data,
+                                 recv_row.ctypes.data, row, rows_per_call, 256, None) == 0
     l.stream_sync(None)
     for d in range(P):
         sigs = rt.get_bytes(l.pe_ptr(sig, d), 8 * P, np.uint64)
@@ -343,8 +343,6 @@ def test_dispatch_put_signal(rt, L, orc, rows_per_call):
             a = int(send_row[s, d]) * row
             b = int(recv_row[s, d]) * row
             assert np.array_equal(got[b:b + c * row], packed[s][a:a + c * row]), (s, d)
-    for x in (d_cnt, d_srow, d_rrow):
-        l.dev_free(x)
     for x in (send, recv, sig):
         l.free(x)
 
