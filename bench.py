@@ -31,6 +31,11 @@ P = 8
 MiB = 1 << 20
 
 
+# Contexts the device-API configurations run through: default, and created with
+# ROCSHMEM_CTX_NOSTORE (completion without the L2 write-back, relaxed AMOs).
+CTX_KINDS = (("default_ctx", 0), ("nostore_ctx", 1))
+
+
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -116,6 +121,17 @@ def headline(b, steps, warmup):
                          "putmem_all_cus_gbs": round(2 * m / tg / 1e6, 3),
                          "getmem_all_cus_gbs": round(2 * m / tget / 1e6, 3)}
     out["curve"] = curve
+    # Device API from every CU: rocshmem_ctx_putmem_wg on 64 KiB tiles, one
+    # quiet per work-group, through a default and a NOSTORE context.
+    tiled = {}
+    for name, opt in CTX_KINDS:
+        l.set_ctx_options(opt)
+        for n_wgs in (1024, 4096):
+            t = b.time_ms(rotating(lambda me, pe: l.rma(b.L.PUT, b.L.WG, dsts[me], srcs[me], n, 65536, me,
+                                                        pe, n_wgs, 1024, 1, None)), max(3, min(steps, 20)), 2)
+            tiled["%s_%dwgs_gbs" % (name, n_wgs)] = round(2 * n / t / 1e6, 1)
+    l.set_ctx_options(0)
+    out["tiled"] = tiled
     l.free(src)
     l.free(dst)
     return out
@@ -204,12 +220,17 @@ def dispatch_config(b, steps):
         assert l.dispatch_put_signal(recv, send, sig, tabs[0].ctypes.data, tabs[1].ctypes.data,
                                      tabs[2].ctypes.data, row, 128, 1024, None) == 0
 
-    ms = b.time_ms(step, max(5, steps // 10), 2)
     alg = 2 * int(counts.sum()) * row
+    res = {"rows": int(counts.sum())}
+    for name, opt in CTX_KINDS:
+        l.set_ctx_options(opt)
+        ms = b.time_ms(step, max(5, steps // 10), 2)
+        res[name] = {"ms": round(ms, 4), "gbs": round(alg / ms / 1e6, 1),
+                     "frac": round(alg / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    l.set_ctx_options(0)
     for x in (send, recv, sig):
         l.free(x)
-    return {"ms": round(ms, 4), "gbs": round(alg / ms / 1e6, 1),
-            "frac": round(alg / ms / 1e6 / HBM_PEAK_GBS, 4), "rows": int(counts.sum())}
+    return res
 
 
 def amo_config(b, steps):
@@ -230,9 +251,13 @@ def amo_config(b, steps):
         l.copy_in(d_ids, ids.ctypes.data, n * 4)
         for p in range(P):
             l.fill(l.pe_ptr(ctr, p), 0, K // P * 8)
-        ms = b.time_ms(lambda: l.amo(L.AMO_FETCH_ADD, L.LONG, ctr, K // P, d_ids, None, None, d_out,
-                                     n, 0, 4096, 256, None), max(3, steps // 10), 1)
-        res[dist] = {"ms": round(ms, 4), "mops": round(n / ms / 1e3, 1)}
+        res[dist] = {}
+        for name, opt in CTX_KINDS:
+            l.set_ctx_options(opt)
+            ms = b.time_ms(lambda: l.amo(L.AMO_FETCH_ADD, L.LONG, ctr, K // P, d_ids, None, None, d_out,
+                                         n, 0, 4096, 256, None), max(3, steps // 10), 1)
+            res[dist][name] = {"ms": round(ms, 4), "mops": round(n / ms / 1e3, 1)}
+        l.set_ctx_options(0)
         l.dev_free(d_ids)
         l.dev_free(d_out)
     l.free(ctr)
@@ -248,12 +273,17 @@ def pingpong_config(b):
     iters = 2000
     for k in range(3, 17):
         n = 1 << k
-        for p in (0, 1):
-            l.fill(l.pe_ptr(sig, p), 0, 8)
-        ticks, hz = C.c_uint64(), C.c_double()
-        assert l.pingpong(buf, sig, n, iters, 0, 1, 256, C.byref(ticks), C.byref(hz), None) == 0
-        one_way_us = ticks.value / hz.value / iters / 2 * 1e6
-        res[str(n)] = {"latency_us": round(one_way_us, 3), "msg_per_s": round(1e6 / one_way_us, 1)}
+        res[str(n)] = {}
+        for name, opt in CTX_KINDS:
+            l.set_ctx_options(opt)
+            for p in (0, 1):
+                l.fill(l.pe_ptr(sig, p), 0, 8)
+            ticks, hz = C.c_uint64(), C.c_double()
+            assert l.pingpong(buf, sig, n, iters, 0, 1, 256, C.byref(ticks), C.byref(hz), None) == 0
+            one_way_us = ticks.value / hz.value / iters / 2 * 1e6
+            res[str(n)][name] = {"latency_us": round(one_way_us, 3),
+                                 "msg_per_s": round(1e6 / one_way_us, 1)}
+    l.set_ctx_options(0)
     l.free(buf)
     l.free(sig)
     return res
@@ -332,6 +362,7 @@ def main():
         allc["atomic_fetch_add_16Mi"] = amo_config(b, a.steps)
         allc["pingpong"] = pingpong_config(b)
     allc["putmem_curve"] = head["curve"]
+    allc["putmem_wg_64KiB_tiles_256MiB"] = head["tiled"]
     b.l.finalize()
     cpu = None if (a.quick or a.no_cpu) else cpu_baseline()
     line = {

@@ -18,6 +18,24 @@ __device__ __forceinline__ int translate_pe(rocshmem_ctx_t ctx, int pe) {
   return ti ? ti->pe_start + ti->stride * pe : pe;
 }
 
+// A context created with ROCSHMEM_CTX_NOSTORE promises that its quiet / fence
+// need not order the caller's own plain stores (the reference turns its flush
+// off for such contexts, src/fence_policy.hpp:45-63).  Everything the library
+// itself writes for a _wave / _wg put is a write-through store, so on such a
+// context completion is a wait on the issuing wavefront's own counters and the
+// L2 write-back of a release is skipped.  That write-back is the expensive
+// part when many work-groups end a put each: the L2 of an XCD serves them one
+// after another, about 60 ns each when idle and a memory round trip each while
+// stores are in flight.
+__device__ __forceinline__ bool no_store_order(const Context *c) {
+  return (c->options & static_cast<unsigned>(ROCSHMEM_CTX_NOSTORE)) != 0;
+}
+// quiet / fence on context c.
+__device__ __forceinline__ void ctx_release(const Context *c) {
+  if (no_store_order(c)) drain_own_stores();
+  else fence_release();
+}
+
 // ---- thread granularity: copy, then order (context_ipc_device.cpp:62-88) ---
 __device__ __forceinline__ void putmem(Context *c, void *dest, const void *source,
                                        size_t n, int pe) {
@@ -34,7 +52,8 @@ __device__ __forceinline__ void getmem(Context *c, void *dest, const void *sourc
 __device__ __forceinline__ void putmem_wave(Context *c, void *dest, const void *source,
                                             size_t n, int pe) {
   copy_wave(remote_addr(c, static_cast<char *>(dest), pe), source, n, g_state.nt_bytes);
-  fence_full();
+  if (no_store_order(c)) drain_own_stores();
+  else fence_full();
 }
 __device__ __forceinline__ void getmem_wave(Context *c, void *dest, const void *source,
                                             size_t n, int pe) {
@@ -47,6 +66,9 @@ __device__ __forceinline__ void putmem_wg(Context *c, void *dest, const void *so
                                           size_t n, int pe) {
   copy_lanes(remote_addr(c, static_cast<char *>(dest), pe), source, n,
              flat_thread_id(), flat_block_size(), g_state.nt_bytes);
+  // Each wavefront completes its own share, so that after the barrier a quiet
+  // by any one thread covers the whole work-group's put.
+  if (no_store_order(c)) drain_own_stores();
   __syncthreads();
 }
 __device__ __forceinline__ void getmem_wg(Context *c, void *dest, const void *source,
@@ -57,18 +79,24 @@ __device__ __forceinline__ void getmem_wg(Context *c, void *dest, const void *so
 }
 
 // ---- signal update by the one lane that leads the call (:221-298) ---------
-// The store / add is a release at agent scope, which orders it after the
-// payload the caller's group wrote before it.
+// On a default context the store / add is a release at agent scope, which
+// orders it after the payload and after everything else the caller's group
+// wrote before it.  On a ROCSHMEM_CTX_NOSTORE context the payload of a _wave /
+// _wg put is already complete when the leader gets here (write-through
+// stores, drained by each wavefront), so a relaxed update suffices; the
+// thread-granularity put moves its payload with plain stores and keeps the
+// release.
 __device__ __forceinline__ void signal_update(Context *c, uint64_t *sig_addr,
-                                              uint64_t signal, int sig_op, int pe) {
+                                              uint64_t signal, int sig_op, int pe,
+                                              bool relaxed = false) {
   unsigned long long *target =
       reinterpret_cast<unsigned long long *>(remote_addr(c, sig_addr, pe));
   switch (sig_op) {
     case ROCSHMEM_SIGNAL_SET:
-      amo_set<unsigned long long>(target, signal);
+      amo_set<unsigned long long>(target, signal, relaxed);
       break;
     case ROCSHMEM_SIGNAL_ADD:
-      amo_add<unsigned long long>(target, signal);
+      amo_add<unsigned long long>(target, signal, relaxed);
       break;
     default:
       break;  // unknown op: payload delivered, signal untouched
@@ -90,14 +118,14 @@ __device__ __forceinline__ void putmem_signal_wave(Context *c, void *dest,
   const unsigned long long mask = __ballot(1);
   const unsigned lane = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
   if (lane == static_cast<unsigned>(__ffsll(static_cast<long long>(mask)) - 1))
-    signal_update(c, sig_addr, signal, sig_op, pe);
+    signal_update(c, sig_addr, signal, sig_op, pe, no_store_order(c));
 }
 __device__ __forceinline__ void putmem_signal_wg(Context *c, void *dest,
                                                  const void *source, size_t n,
                                                  uint64_t *sig_addr, uint64_t signal,
                                                  int sig_op, int pe) {
   putmem_wg(c, dest, source, n, pe);
-  if (is_block_leader()) signal_update(c, sig_addr, signal, sig_op, pe);
+  if (is_block_leader()) signal_update(c, sig_addr, signal, sig_op, pe, no_store_order(c));
 }
 
 // signal_fetch: atomic read of the caller's own word (:300-324).

@@ -33,6 +33,14 @@ __device__ __forceinline__ void fence_acquire() {
 __device__ __forceinline__ void fence_full() {
   __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "agent");
 }
+// Wait until every memory operation this wavefront has issued is acknowledged.
+// A write-through (sc1) store is acknowledged once it is visible at agent
+// scope, so after this the wavefront's cooperative-copy stores are complete
+// without an L2 write-back.  Plain stores may still sit dirty in the L2.
+__device__ __forceinline__ void drain_own_stores() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+}
 
 // Integer type of the same width, used to move float/double through atomics.
 template <size_t N> struct BitsOf;
@@ -61,16 +69,23 @@ __device__ __forceinline__ void store_through(T *p, T v) {
 }
 
 // ---- atomic memory operations on an already-translated address -----------
-// Each is one device-wide RMW; the memory order is acquire-release so an AMO
-// can publish or consume data the way the reference's seq_cst ones do.
+// Each is one device-wide RMW.  By default the memory order is
+// acquire-release, so an AMO can publish or consume data the way the
+// reference's seq_cst ones do (src/ipc_policy.hpp:69-99).  With `relaxed`
+// (contexts created with ROCSHMEM_CTX_NOSTORE) only the word itself is
+// atomic, which is all OpenSHMEM asks of an AMO, and the L2 write-back and
+// invalidate that an agent-scope release / acquire costs are left to the
+// caller's quiet / fence / wait_until.
 // One RMW per lane, straight to memory.
 template <typename T>
-__device__ __forceinline__ T amo_fetch_add_each(T *p, T v) {
+__device__ __forceinline__ T amo_fetch_add_each(T *p, T v, bool relaxed = false) {
+  if (relaxed) return __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   return __hip_atomic_fetch_add(p, v, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
 }
 template <typename T>
-__device__ __forceinline__ void amo_add_each(T *p, T v) {
-  (void)__hip_atomic_fetch_add(p, v, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+__device__ __forceinline__ void amo_add_each(T *p, T v, bool relaxed = false) {
+  if (relaxed) (void)__hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  else (void)__hip_atomic_fetch_add(p, v, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 __device__ __forceinline__ unsigned lane_index() {
@@ -129,7 +144,7 @@ __device__ __forceinline__ T from_lane(T v, int lane) {
 // early once kMissBudget lanes in a row turned out to be alone, which keeps
 // the cost flat for address streams without collisions.
 template <typename T, bool kFetch>
-__device__ __forceinline__ T amo_add_wave(T *p, T v) {
+__device__ __forceinline__ T amo_add_wave(T *p, T v, bool relaxed) {
   constexpr int kMissBudget = 6;
   const unsigned lane = lane_index();
   const unsigned long long addr = reinterpret_cast<unsigned long long>(p);
@@ -165,8 +180,8 @@ __device__ __forceinline__ T amo_add_wave(T *p, T v) {
   }
   T base = static_cast<T>(0);
   if (leader == static_cast<int>(lane)) {
-    if constexpr (kFetch) base = amo_fetch_add_each(p, total);
-    else amo_add_each(p, total);
+    if constexpr (kFetch) base = amo_fetch_add_each(p, total, relaxed);
+    else amo_add_each(p, total, relaxed);
   }
   if constexpr (kFetch) {
     base = from_lane(base, leader);
@@ -176,64 +191,78 @@ __device__ __forceinline__ T amo_add_wave(T *p, T v) {
 }
 
 template <typename T>
-__device__ __forceinline__ T amo_fetch_add(T *p, T v) {
-  return amo_add_wave<T, true>(p, v);
+__device__ __forceinline__ T amo_fetch_add(T *p, T v, bool relaxed = false) {
+  return amo_add_wave<T, true>(p, v, relaxed);
 }
 template <typename T>
-__device__ __forceinline__ void amo_add(T *p, T v) {
-  (void)amo_add_wave<T, false>(p, v);
+__device__ __forceinline__ void amo_add(T *p, T v, bool relaxed = false) {
+  (void)amo_add_wave<T, false>(p, v, relaxed);
 }
 template <typename T>
-__device__ __forceinline__ T amo_fetch_cas(T *p, T cond, T v) {
+__device__ __forceinline__ T amo_fetch_cas(T *p, T cond, T v, bool relaxed = false) {
   using B = typename BitsOf<sizeof(T)>::type;
   B expected, desired;
   __builtin_memcpy(&expected, &cond, sizeof(T));
   __builtin_memcpy(&desired, &v, sizeof(T));
-  __hip_atomic_compare_exchange_strong(reinterpret_cast<B *>(p), &expected, desired,
-                                       __ATOMIC_ACQ_REL, __ATOMIC_ACQUIRE,
-                                       __HIP_MEMORY_SCOPE_AGENT);
+  if (relaxed)
+    __hip_atomic_compare_exchange_strong(reinterpret_cast<B *>(p), &expected, desired,
+                                         __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                         __HIP_MEMORY_SCOPE_AGENT);
+  else
+    __hip_atomic_compare_exchange_strong(reinterpret_cast<B *>(p), &expected, desired,
+                                         __ATOMIC_ACQ_REL, __ATOMIC_ACQUIRE,
+                                         __HIP_MEMORY_SCOPE_AGENT);
   T out;
   __builtin_memcpy(&out, &expected, sizeof(T));
   return out;
 }
 template <typename T>
-__device__ __forceinline__ void amo_set(T *p, T v) {
+__device__ __forceinline__ void amo_set(T *p, T v, bool relaxed = false) {
   using B = typename BitsOf<sizeof(T)>::type;
   B b;
   __builtin_memcpy(&b, &v, sizeof(T));
-  __hip_atomic_store(reinterpret_cast<B *>(p), b, __ATOMIC_RELEASE,
-                     __HIP_MEMORY_SCOPE_AGENT);
+  if (relaxed)
+    __hip_atomic_store(reinterpret_cast<B *>(p), b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  else
+    __hip_atomic_store(reinterpret_cast<B *>(p), b, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
 }
 template <typename T>
-__device__ __forceinline__ T amo_fetch(T *p) {
+__device__ __forceinline__ T amo_fetch(T *p, bool relaxed = false) {
   using B = typename BitsOf<sizeof(T)>::type;
-  B b = __hip_atomic_load(reinterpret_cast<const B *>(p), __ATOMIC_ACQUIRE,
-                          __HIP_MEMORY_SCOPE_AGENT);
+  B b = relaxed ? __hip_atomic_load(reinterpret_cast<const B *>(p), __ATOMIC_RELAXED,
+                                    __HIP_MEMORY_SCOPE_AGENT)
+                : __hip_atomic_load(reinterpret_cast<const B *>(p), __ATOMIC_ACQUIRE,
+                                    __HIP_MEMORY_SCOPE_AGENT);
   T out;
   __builtin_memcpy(&out, &b, sizeof(T));
   return out;
 }
 template <typename T>
-__device__ __forceinline__ T amo_swap(T *p, T v) {
+__device__ __forceinline__ T amo_swap(T *p, T v, bool relaxed = false) {
   using B = typename BitsOf<sizeof(T)>::type;
   B b;
   __builtin_memcpy(&b, &v, sizeof(T));
-  B old = __hip_atomic_exchange(reinterpret_cast<B *>(p), b, __ATOMIC_ACQ_REL,
-                                __HIP_MEMORY_SCOPE_AGENT);
+  B old = relaxed ? __hip_atomic_exchange(reinterpret_cast<B *>(p), b, __ATOMIC_RELAXED,
+                                          __HIP_MEMORY_SCOPE_AGENT)
+                  : __hip_atomic_exchange(reinterpret_cast<B *>(p), b, __ATOMIC_ACQ_REL,
+                                          __HIP_MEMORY_SCOPE_AGENT);
   T out;
   __builtin_memcpy(&out, &old, sizeof(T));
   return out;
 }
 template <typename T>
-__device__ __forceinline__ T amo_fetch_and(T *p, T v) {
+__device__ __forceinline__ T amo_fetch_and(T *p, T v, bool relaxed = false) {
+  if (relaxed) return __hip_atomic_fetch_and(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   return __hip_atomic_fetch_and(p, v, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
 }
 template <typename T>
-__device__ __forceinline__ T amo_fetch_or(T *p, T v) {
+__device__ __forceinline__ T amo_fetch_or(T *p, T v, bool relaxed = false) {
+  if (relaxed) return __hip_atomic_fetch_or(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   return __hip_atomic_fetch_or(p, v, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
 }
 template <typename T>
-__device__ __forceinline__ T amo_fetch_xor(T *p, T v) {
+__device__ __forceinline__ T amo_fetch_xor(T *p, T v, bool relaxed = false) {
+  if (relaxed) return __hip_atomic_fetch_xor(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   return __hip_atomic_fetch_xor(p, v, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
 }
 

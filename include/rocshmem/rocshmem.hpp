@@ -121,11 +121,17 @@ __device__ ATTR_NO_INLINE inline void rocshmem_wg_ctx_destroy(rocshmem_ctx_t *ct
 // consistent store per PE).  Every operation of this library has already
 // performed its loads and stores when it returns, so what is left to do is to
 // publish them: a release at agent scope.
-__device__ ATTR_NO_INLINE inline void rocshmem_ctx_fence(rocshmem_ctx_t) { detail::fence_release(); }
+__device__ ATTR_NO_INLINE inline void rocshmem_ctx_fence(rocshmem_ctx_t ctx) {
+  detail::ctx_release(detail::ctx_of(ctx));
+}
 __device__ ATTR_NO_INLINE inline void rocshmem_fence() { detail::fence_release(); }
-__device__ ATTR_NO_INLINE inline void rocshmem_ctx_fence(rocshmem_ctx_t, int) { detail::fence_release(); }
+__device__ ATTR_NO_INLINE inline void rocshmem_ctx_fence(rocshmem_ctx_t ctx, int) {
+  detail::ctx_release(detail::ctx_of(ctx));
+}
 __device__ ATTR_NO_INLINE inline void rocshmem_fence(int) { detail::fence_release(); }
-__device__ ATTR_NO_INLINE inline void rocshmem_ctx_quiet(rocshmem_ctx_t) { detail::fence_release(); }
+__device__ ATTR_NO_INLINE inline void rocshmem_ctx_quiet(rocshmem_ctx_t ctx) {
+  detail::ctx_release(detail::ctx_of(ctx));
+}
 __device__ ATTR_NO_INLINE inline void rocshmem_quiet() { detail::fence_release(); }
 __device__ ATTR_NO_INLINE inline void rocshmem_ctx_threadfence_system(rocshmem_ctx_t) {
   __threadfence_system();

@@ -20,8 +20,9 @@ namespace rocshmem {
 #define ROCSHMEM_AMD_AMO_STANDARD(T, TN)                                                  \
   __device__ ATTR_NO_INLINE inline T rocshmem_ctx_##TN##_atomic_fetch_add(                \
       rocshmem_ctx_t ctx, T *dest, T value, int pe) {                                     \
-    return detail::amo_fetch_add(detail::remote_addr(detail::ctx_of(ctx), dest, pe),      \
-                                 value);                                                  \
+    detail::Context *c = detail::ctx_of(ctx);                                             \
+    return detail::amo_fetch_add(detail::remote_addr(c, dest, pe), value,                 \
+                                 detail::no_store_order(c));                              \
   }                                                                                       \
   __device__ ATTR_NO_INLINE inline T rocshmem_##TN##_atomic_fetch_add(T *dest, T value,   \
                                                                      int pe) {            \
@@ -30,7 +31,8 @@ namespace rocshmem {
   }                                                                                       \
   __device__ ATTR_NO_INLINE inline void rocshmem_ctx_##TN##_atomic_add(                   \
       rocshmem_ctx_t ctx, T *dest, T value, int pe) {                                     \
-    detail::amo_add(detail::remote_addr(detail::ctx_of(ctx), dest, pe), value);           \
+    detail::Context *c = detail::ctx_of(ctx);                                             \
+    detail::amo_add(detail::remote_addr(c, dest, pe), value, detail::no_store_order(c));  \
   }                                                                                       \
   __device__ ATTR_NO_INLINE inline void rocshmem_##TN##_atomic_add(T *dest, T value,      \
                                                                   int pe) {               \
@@ -52,8 +54,9 @@ namespace rocshmem {
   }                                                                                       \
   __device__ ATTR_NO_INLINE inline T rocshmem_ctx_##TN##_atomic_compare_swap(             \
       rocshmem_ctx_t ctx, T *dest, T cond, T value, int pe) {                             \
-    return detail::amo_fetch_cas(detail::remote_addr(detail::ctx_of(ctx), dest, pe), cond,\
-                                 value);                                                  \
+    detail::Context *c = detail::ctx_of(ctx);                                             \
+    return detail::amo_fetch_cas(detail::remote_addr(c, dest, pe), cond, value,           \
+                                 detail::no_store_order(c));                              \
   }                                                                                       \
   __device__ ATTR_NO_INLINE inline T rocshmem_##TN##_atomic_compare_swap(                 \
       T *dest, T cond, T value, int pe) {                                                 \
@@ -64,14 +67,17 @@ namespace rocshmem {
 #define ROCSHMEM_AMD_AMO_EXTENDED(T, TN)                                                  \
   __device__ ATTR_NO_INLINE inline T rocshmem_ctx_##TN##_atomic_fetch(                    \
       rocshmem_ctx_t ctx, T *source, int pe) {                                            \
-    return detail::amo_fetch(detail::remote_addr(detail::ctx_of(ctx), source, pe));       \
+    detail::Context *c = detail::ctx_of(ctx);                                             \
+    return detail::amo_fetch(detail::remote_addr(c, source, pe),                          \
+                             detail::no_store_order(c));                                  \
   }                                                                                       \
   __device__ ATTR_NO_INLINE inline T rocshmem_##TN##_atomic_fetch(T *source, int pe) {    \
     return rocshmem_ctx_##TN##_atomic_fetch(rocshmem_ctx_t{nullptr, nullptr}, source, pe);\
   }                                                                                       \
   __device__ ATTR_NO_INLINE inline void rocshmem_ctx_##TN##_atomic_set(                   \
       rocshmem_ctx_t ctx, T *dest, T value, int pe) {                                     \
-    detail::amo_set(detail::remote_addr(detail::ctx_of(ctx), dest, pe), value);           \
+    detail::Context *c = detail::ctx_of(ctx);                                             \
+    detail::amo_set(detail::remote_addr(c, dest, pe), value, detail::no_store_order(c));  \
   }                                                                                       \
   __device__ ATTR_NO_INLINE inline void rocshmem_##TN##_atomic_set(T *dest, T value,      \
                                                                   int pe) {               \
@@ -79,7 +85,9 @@ namespace rocshmem {
   }                                                                                       \
   __device__ ATTR_NO_INLINE inline T rocshmem_ctx_##TN##_atomic_swap(                     \
       rocshmem_ctx_t ctx, T *dest, T value, int pe) {                                     \
-    return detail::amo_swap(detail::remote_addr(detail::ctx_of(ctx), dest, pe), value);   \
+    detail::Context *c = detail::ctx_of(ctx);                                             \
+    return detail::amo_swap(detail::remote_addr(c, dest, pe), value,                      \
+                            detail::no_store_order(c));                                   \
   }                                                                                       \
   __device__ ATTR_NO_INLINE inline T rocshmem_##TN##_atomic_swap(T *dest, T value,        \
                                                                  int pe) {                \
@@ -90,8 +98,9 @@ namespace rocshmem {
 #define ROCSHMEM_AMD_AMO_BITWISE1(T, TN, OP)                                              \
   __device__ ATTR_NO_INLINE inline T rocshmem_ctx_##TN##_atomic_fetch_##OP(               \
       rocshmem_ctx_t ctx, T *dest, T value, int pe) {                                     \
-    return detail::amo_fetch_##OP(detail::remote_addr(detail::ctx_of(ctx), dest, pe),     \
-                                  value);                                                 \
+    detail::Context *c = detail::ctx_of(ctx);                                             \
+    return detail::amo_fetch_##OP(detail::remote_addr(c, dest, pe), value,                \
+                                  detail::no_store_order(c));                             \
   }                                                                                       \
   __device__ ATTR_NO_INLINE inline T rocshmem_##TN##_atomic_fetch_##OP(T *dest, T value,  \
                                                                       int pe) {           \

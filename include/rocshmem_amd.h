@@ -111,6 +111,17 @@ int rocshmem_amd_my_pe(void);
  * blockIdx.x/y/z mod P). */
 int rocshmem_amd_set_pe(int pe);
 int rocshmem_amd_set_pe_rule(int rule);
+/* Options (ROCSHMEM_CTX_* bits, include/rocshmem/rocshmem_common.hpp:98-102)
+ * of the contexts the RMA, AMO, put_signal, ping-pong and dispatch drivers
+ * below act through, as if each PE had called
+ * rocshmem_ctx_create(options, &ctx) (rocshmem.hpp:144) and used that ctx.
+ * 0 (the start value) is the default context.  With ROCSHMEM_CTX_NOSTORE (1)
+ * quiet / fence, the close of every _wave / _wg put and the signal of
+ * put_signal wait on the wavefront's own write-through stores instead of
+ * writing the L2 back, and AMOs are relaxed (src/fence_policy.hpp:45-63 turns
+ * the reference's flush off for that option).  Returns the previous options,
+ * -1 before init. */
+int64_t rocshmem_amd_set_ctx_options(int64_t options);
 /* rocshmem_malloc / rocshmem_free (rocshmem.hpp:115-123): NULL on size 0 or
  * exhaustion; the object exists at the same offset on every PE. */
 void *rocshmem_amd_malloc(size_t size);
@@ -179,7 +190,6 @@ int rocshmem_amd_timer_destroy(void *timer);
 int rocshmem_amd_rma(int rma_op, int gran, void *dest, const void *source, size_t nbytes,
                      size_t tile_bytes, int my_pe, int pe, int n_wgs, int wg_size,
                      int iters, rocshmem_amd_stream_t stream);
-
 /* Host-initiated bulk copy between PEs over the whole GPU: the host-side
  * rocshmem_putmem / rocshmem_getmem (rocshmem_RMA.hpp; reference forwards them
  * to MPI_Put / MPI_Get, src/host/host_helpers.hpp:52-88). */
@@ -274,6 +284,24 @@ int rocshmem_amd_put_signal(int gran, void *dest, const void *source, size_t nby
  * by PE my_pe from its own word. */
 int rocshmem_amd_signal_fetch(int gran, const uint64_t *sig_addr, int my_pe,
                               uint64_t *value_out);
+
+/* Put, quiet, then raise a flag — the pattern quiet exists for (OpenSHMEM
+ * message passing; rocshmem_ctx_quiet, include/rocshmem/rocshmem.hpp:408;
+ * src/ipc/context_ipc_device.cpp:100-102) — with the receiver checking the
+ * payload inside the same kernel.  `pairs` (<= 128) producer work-groups act
+ * for pe_a, each with a receiver work-group acting for pe_b.  Per round a
+ * producer fills a fresh pattern, calls rocshmem_ctx_putmem_wg of nbytes
+ * (multiple of 4) into its slot of `data` on pe_b, calls rocshmem_ctx_quiet and
+ * then sets its flag on pe_b with a relaxed store — or, with_signal != 0, does
+ * all three with one rocshmem_ctx_putmem_signal_wg (rocshmem_SIG_OP.hpp:128-131);
+ * the receiver waits for the flag, compares every word, and acknowledges.  data: pairs*nbytes symmetric bytes,
+ * flags: 2*pairs symmetric uint64 (addresses on pe_a).  mismatches_out = words
+ * that differed; timed_out_out = 1 if a bounded wait ran out (all work-groups
+ * then leave). */
+int rocshmem_amd_put_flag_check(void *data, uint64_t *flags, size_t nbytes, int pairs, int rounds,
+                                int pe_a, int pe_b, int wg_size, int with_signal,
+                                uint64_t *mismatches_out, int *timed_out_out,
+                                rocshmem_amd_stream_t stream);
 
 /* Ping-pong (tests/functional_tests/ping_pong_tester.cpp:43-61,
  * examples/rocshmem_put_signal_test.cc:31-47): work-group 0 acts for pe_a,

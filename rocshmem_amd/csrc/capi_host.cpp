@@ -31,6 +31,12 @@ int rocshmem_amd_set_pe_rule(int rule) {
   rt().set_pe_rule(rule);
   return 0;
 }
+int64_t rocshmem_amd_set_ctx_options(int64_t options) {
+  if (!rt().live) return -1;
+  const int64_t before = rt().driver_ctx_options;
+  rt().driver_ctx_options = options;
+  return before;
+}
 void *rocshmem_amd_malloc(size_t size) { return rt().sym_malloc(size); }
 int rocshmem_amd_free(void *ptr) {
   rt().sym_free(ptr);

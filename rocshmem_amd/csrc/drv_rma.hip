@@ -150,7 +150,7 @@ int rocshmem_amd_rma(int rma_op, int gran, void *dest, const void *source, size_
   a.source = static_cast<const char *>(source);
   a.nbytes = nbytes;
   a.tile = tile_bytes ? tile_bytes : auto_tile(nbytes, groups);
-  a.ctx = runtime::rt().default_ctx_handle(my_pe);
+  a.ctx = runtime::rt().driver_ctx_handle(my_pe);
   a.pe = pe;
   a.iters = iters;
   hipStream_t s = as_stream(stream);

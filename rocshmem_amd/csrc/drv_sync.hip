@@ -265,6 +265,95 @@ __global__ void pingpong_kernel(PingPongArgs a) {
 }
 
 // ---------------------------------------------------------------------------
+// put + quiet + flag, checked by the receiver inside the same kernel
+// ---------------------------------------------------------------------------
+struct PutFlagArgs {
+  char *data_a;          // [pairs][nbytes], address on pe_a
+  int64_t a_to_b;        // bytes from pe_a's slice to pe_b's
+  uint64_t *flag_b;      // [pairs] on pe_b : round announced by the producer
+  uint64_t *ack_a;       // [pairs] on pe_a : round consumed by the receiver
+  uint32_t *staging;     // [pairs][nbytes/4] producer-side source, plain device memory
+  size_t nbytes;         // per pair, multiple of 4
+  int rounds;
+  int pe_a, pe_b;
+  int with_signal;       // 0: putmem_wg, quiet, relaxed flag store; 1: putmem_signal_wg
+  unsigned spin_limit;
+  rocshmem_ctx_t ctx_a;
+  unsigned long long *mismatches;
+  int *timed_out;
+};
+
+__device__ __forceinline__ uint32_t put_flag_word(int pair, int round, size_t i) {
+  return static_cast<uint32_t>(i) * 2654435761u + static_cast<uint32_t>(round) * 40503u +
+         static_cast<uint32_t>(pair);
+}
+
+// Waits (thread 0, bounded) until *word == round; false when the limit ran out.
+__device__ __forceinline__ bool put_flag_wait(uint64_t *word, uint64_t round, unsigned limit,
+                                              int *timed_out) {
+  __shared__ int ok;
+  if (threadIdx.x == 0) {
+    ok = 0;
+    for (unsigned spin = 0; spin < limit; ++spin) {
+      if (detail::load_through(word) == round) {
+        ok = 1;
+        break;
+      }
+      if (detail::load_through(timed_out)) break;
+      __builtin_amdgcn_s_sleep(2);
+    }
+    if (ok) detail::fence_acquire();
+    else detail::store_through(timed_out, 1);
+  }
+  __syncthreads();
+  const bool r = ok != 0;
+  __syncthreads();
+  return r;
+}
+
+// Even work-groups produce for pe_a, odd ones consume for pe_b.  The flag and
+// the acknowledgement are relaxed write-through stores: the only thing that
+// orders the payload before the flag is the context's quiet.
+__global__ void put_flag_kernel(PutFlagArgs a) {
+  const int pair = blockIdx.x >> 1;
+  const bool producer = (blockIdx.x & 1) == 0;
+  const size_t nwords = a.nbytes / 4;
+  char *data = a.data_a + static_cast<size_t>(pair) * a.nbytes;
+  uint32_t *stage = a.staging + static_cast<size_t>(pair) * nwords;
+  // Own-PE views of the two control words.
+  uint64_t *flag_on_b = a.flag_b + pair;
+  uint64_t *ack_on_a = a.ack_a + pair;
+  for (int r = 1; r <= a.rounds; ++r) {
+    if (producer) {
+      for (size_t i = threadIdx.x; i < nwords; i += blockDim.x) stage[i] = put_flag_word(pair, r, i);
+      __syncthreads();
+      if (a.with_signal) {
+        // flag_on_b is pe_b's address; the call wants pe_a's.
+        uint64_t *flag_sym = reinterpret_cast<uint64_t *>(reinterpret_cast<char *>(flag_on_b) - a.a_to_b);
+        rocshmem_ctx_putmem_signal_wg(a.ctx_a, data, stage, a.nbytes, flag_sym,
+                                      static_cast<uint64_t>(r), ROCSHMEM_SIGNAL_SET, a.pe_b);
+      } else {
+        rocshmem_ctx_putmem_wg(a.ctx_a, data, stage, a.nbytes, a.pe_b);
+        if (threadIdx.x == 0) {
+          rocshmem_ctx_quiet(a.ctx_a);
+          detail::store_through(flag_on_b, static_cast<uint64_t>(r));
+        }
+      }
+      if (!put_flag_wait(ack_on_a, static_cast<uint64_t>(r), a.spin_limit, a.timed_out)) return;
+    } else {
+      if (!put_flag_wait(flag_on_b, static_cast<uint64_t>(r), a.spin_limit, a.timed_out)) return;
+      unsigned bad = 0;
+      const uint32_t *got = reinterpret_cast<const uint32_t *>(data + a.a_to_b);
+      for (size_t i = threadIdx.x; i < nwords; i += blockDim.x)
+        bad += got[i] != put_flag_word(pair, r, i);
+      if (bad) atomicAdd(a.mismatches, static_cast<unsigned long long>(bad));
+      __syncthreads();
+      if (threadIdx.x == 0) detail::store_through(ack_on_a, static_cast<uint64_t>(r));
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // MoE-style dispatch with put_signal
 // ---------------------------------------------------------------------------
 struct DispatchArgs {
@@ -514,7 +603,7 @@ int rocshmem_amd_amo(int amo_op, int dtype, void *counters, uint32_t n_slots,
     a.conds = static_cast<const T *>(conds);
     a.fetched = static_cast<T *>(fetched);
     a.n_ops = n_ops;
-    a.ctx = runtime::rt().default_ctx_handle(my_pe);
+    a.ctx = runtime::rt().driver_ctx_handle(my_pe);
     rc = launch_amo<T>(amo_op, a, n_wgs, wg_size, as_stream(stream));
   });
   return known ? rc : -1;
@@ -539,7 +628,7 @@ int rocshmem_amd_put_signal(int gran, void *dest, const void *source, size_t nby
   a.sig_addr = sig_addr;
   a.signal = signal;
   a.sig_op = sig_op;
-  a.ctx = runtime::rt().default_ctx_handle(my_pe);
+  a.ctx = runtime::rt().driver_ctx_handle(my_pe);
   a.pe = pe;
   a.calls = calls;
   hipStream_t s = as_stream(stream);
@@ -588,7 +677,7 @@ int rocshmem_amd_pingpong(void *buf, uint64_t *sig, size_t nbytes, int iters, in
   a.pe_a = pe_a;
   a.pe_b = pe_b;
   a.pe_stride = r.pe_stride;
-  a.ctx_row = r.d_default_ctx;
+  a.ctx_row = r.driver_ctx_row();
   a.world_row = r.d_teams;
   a.ticks = d_ticks;
   hipStream_t s = as_stream(stream);
@@ -605,6 +694,60 @@ int rocshmem_amd_pingpong(void *buf, uint64_t *sig, size_t nbytes, int iters, in
     DRV_CHECK_HIP(hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev));
     *tick_hz_out = static_cast<double>(khz) * 1e3;
   }
+  return 0;
+}
+
+int rocshmem_amd_put_flag_check(void *data, uint64_t *flags, size_t nbytes, int pairs, int rounds,
+                                int pe_a, int pe_b, int wg_size, int with_signal,
+                                uint64_t *mismatches_out, int *timed_out_out,
+                                rocshmem_amd_stream_t stream) {
+  auto &r = runtime::rt();
+  if (!valid_pe(pe_a) || !valid_pe(pe_b) || pe_a == pe_b || pairs < 1 || pairs > 128 ||
+      !valid_launch(2 * pairs, wg_size) || rounds < 0 || nbytes == 0 || (nbytes & 3))
+    return -1;
+  const size_t total = nbytes * static_cast<size_t>(pairs);
+  if (!sym_ok_on(data, total, pe_a) || !sym_ok_on(flags, 16u * pairs, pe_a)) return -1;
+  if (!mismatches_out || !timed_out_out) return -1;
+  const int64_t a_to_b = static_cast<int64_t>(pe_b - pe_a) * static_cast<int64_t>(r.pe_stride);
+  uint32_t *staging;
+  unsigned long long *d_bad;
+  int *d_timed_out;
+  hipStream_t s = as_stream(stream);
+  DRV_CHECK_HIP(hipMalloc(&staging, total));
+  DRV_CHECK_HIP(hipMalloc(&d_bad, sizeof(unsigned long long)));
+  DRV_CHECK_HIP(hipMalloc(&d_timed_out, sizeof(int)));
+  DRV_CHECK_HIP(hipMemsetAsync(d_bad, 0, sizeof(unsigned long long), s));
+  DRV_CHECK_HIP(hipMemsetAsync(d_timed_out, 0, sizeof(int), s));
+  // Both control arrays start at zero on both PEs.
+  DRV_CHECK_HIP(hipMemsetAsync(flags, 0, 16u * pairs, s));
+  DRV_CHECK_HIP(hipMemsetAsync(reinterpret_cast<char *>(flags) + a_to_b, 0, 16u * pairs, s));
+  PutFlagArgs a;
+  a.data_a = static_cast<char *>(data);
+  a.a_to_b = a_to_b;
+  a.flag_b = reinterpret_cast<uint64_t *>(reinterpret_cast<char *>(flags) + a_to_b);
+  a.ack_a = flags + pairs;
+  a.staging = staging;
+  a.nbytes = nbytes;
+  a.rounds = rounds;
+  a.pe_a = pe_a;
+  a.pe_b = pe_b;
+  a.with_signal = with_signal != 0;
+  a.spin_limit = 1u << 22;
+  a.ctx_a = r.driver_ctx_handle(pe_a);
+  a.mismatches = d_bad;
+  a.timed_out = d_timed_out;
+  hipLaunchKernelGGL(put_flag_kernel, dim3(2 * pairs), dim3(wg_size), 0, s, a);
+  DRV_CHECK_HIP(hipGetLastError());
+  DRV_CHECK_HIP(hipStreamSynchronize(s));
+  unsigned long long bad = 0;
+  int timed_out = 0;
+  DRV_CHECK_HIP(hipMemcpy(&bad, d_bad, sizeof(bad), hipMemcpyDeviceToHost));
+  DRV_CHECK_HIP(hipMemcpy(&timed_out, d_timed_out, sizeof(timed_out), hipMemcpyDeviceToHost));
+  DRV_CHECK_HIP(hipFree(staging));
+  DRV_CHECK_HIP(hipFree(d_bad));
+  DRV_CHECK_HIP(hipFree(d_timed_out));
+  *mismatches_out = bad;
+  *timed_out_out = timed_out;
   return 0;
 }
 
@@ -674,7 +817,7 @@ int rocshmem_amd_dispatch_put_signal(void *recv, const void *send, uint64_t *sig
   a.np = r.npes;
   a.rows_per_call = static_cast<uint32_t>(rows_per_call);
   a.n_calls = t.n_calls;
-  a.ctx_row = r.d_default_ctx;
+  a.ctx_row = r.driver_ctx_row();
   a.world_row = r.d_teams;
   const uint32_t max_senders = 256 * 16;
   const uint32_t senders = a.n_calls < max_senders ? (a.n_calls ? a.n_calls : 1) : max_senders;

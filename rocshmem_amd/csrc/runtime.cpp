@@ -143,6 +143,7 @@ int Runtime::init(int want_npes, size_t want_heap) {
   }
   pe_stride = std::max(min_stride, want / two_mib * two_mib);
   acting_pe = 0;
+  driver_ctx_options = 0;
 
   if (hipMalloc(reinterpret_cast<void **>(&heap_base), pe_stride * npes) != hipSuccess) {
     (void)hipGetLastError();  // not enough room for the spread layout: pack the slices
@@ -178,10 +179,17 @@ int Runtime::init(int want_npes, size_t want_heap) {
     c.options = 0;
     c.pool_slot = slot;
   };
-  std::vector<detail::Context> ctxs(npes);
-  for (int pe = 0; pe < npes; ++pe) fill_ctx(ctxs[pe], pe, -1);
-  RT_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&d_default_ctx), sizeof(detail::Context) * npes));
-  RT_CHECK_HIP(hipMemcpy(d_default_ctx, ctxs.data(), sizeof(detail::Context) * npes,
+  // Rows [0, npes) are the default contexts; rows [npes, 2*npes) are the same
+  // with ROCSHMEM_CTX_NOSTORE set, handed out by rocshmem_ctx_create.
+  std::vector<detail::Context> ctxs(2 * static_cast<size_t>(npes));
+  for (int pe = 0; pe < npes; ++pe) {
+    fill_ctx(ctxs[pe], pe, -1);
+    fill_ctx(ctxs[npes + pe], pe, -1);
+    ctxs[npes + pe].options = static_cast<unsigned>(ROCSHMEM_CTX_NOSTORE);
+  }
+  RT_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&d_default_ctx),
+                         sizeof(detail::Context) * ctxs.size()));
+  RT_CHECK_HIP(hipMemcpy(d_default_ctx, ctxs.data(), sizeof(detail::Context) * ctxs.size(),
                          hipMemcpyHostToDevice));
 
   RT_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&d_ctx_slots),
@@ -410,10 +418,9 @@ __host__ int rocshmem_n_pes() {
   return static_cast<int>(runtime::env_size("ROCSHMEM_EMU_NPES", 1));
 }
 __host__ int rocshmem_my_pe() { return rt().live ? rt().acting_pe : 0; }
-__host__ int rocshmem_ctx_create(int64_t, rocshmem_ctx_t *ctx) {
+__host__ int rocshmem_ctx_create(int64_t options, rocshmem_ctx_t *ctx) {
   rt().require_live("rocshmem_ctx_create");
-  ctx->ctx_opaque = rt().d_default_ctx + rt().acting_pe;
-  ctx->team_opaque = &rt().d_teams[rt().acting_pe].wrt_world;
+  *ctx = rt().ctx_handle(rt().acting_pe, options);
   return 0;
 }
 __host__ void rocshmem_ctx_destroy(rocshmem_ctx_t) {}

@@ -27,7 +27,7 @@ struct Runtime {
   char *heap_base = nullptr;
   char *d_ws = nullptr;
   detail::Team *d_teams = nullptr;         // [max_teams][npes]
-  detail::Context *d_default_ctx = nullptr;  // [npes]
+  detail::Context *d_default_ctx = nullptr;  // [2*npes]: default, then NOSTORE
   detail::Context *d_ctx_slots = nullptr;  // [npes][max_ctxs]
   detail::CtxPool *d_pools = nullptr;      // [npes]
   std::vector<detail::Team> h_teams;       // host mirror of d_teams
@@ -60,6 +60,21 @@ struct Runtime {
   rocshmem_ctx_t default_ctx_handle(int pe, int slot = 0) const {
     return rocshmem_ctx_t{d_default_ctx + pe,
                           &d_teams[static_cast<size_t>(slot) * npes + pe].wrt_world};
+  }
+
+  // Options of the contexts the benchmark/test drivers act through.
+  int64_t driver_ctx_options = 0;
+  detail::Context *driver_ctx_row() const {
+    return d_default_ctx + ((driver_ctx_options & ROCSHMEM_CTX_NOSTORE) ? npes : 0);
+  }
+  rocshmem_ctx_t driver_ctx_handle(int pe) const { return ctx_handle(pe, driver_ctx_options); }
+
+  // Host-created context of PE `pe` on the world team with `options`
+  // (ROCSHMEM_CTX_* bits).  Contexts hold no per-context state here, so all
+  // contexts of one PE with the same ordering option share one object.
+  rocshmem_ctx_t ctx_handle(int pe, int64_t options) const {
+    const bool nostore = (options & ROCSHMEM_CTX_NOSTORE) != 0;
+    return rocshmem_ctx_t{d_default_ctx + (nostore ? npes : 0) + pe, &d_teams[pe].wrt_world};
   }
 
  private:

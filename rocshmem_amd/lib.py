@@ -13,6 +13,7 @@ THREAD, WAVE, WG = range(3)
 PUT, GET = range(2)
 (AMO_FETCH_ADD, AMO_ADD, AMO_FETCH_INC, AMO_INC, AMO_COMPARE_SWAP, AMO_FETCH, AMO_SET,
  AMO_SWAP, AMO_FETCH_AND, AMO_FETCH_OR, AMO_FETCH_XOR) = range(11)
+CTX_NOSTORE = 1  # ROCSHMEM_CTX_NOSTORE
 TEST, WAIT_UNTIL, WAIT_UNTIL_ANY, WAIT_UNTIL_ALL, WAIT_UNTIL_SOME = range(5)
 BARRIER_ALL, SYNC_ALL, TEAM_SYNC = range(3)
 CMP_EQ, CMP_NE, CMP_GT, CMP_GE, CMP_LT, CMP_LE = range(6)
@@ -29,6 +30,7 @@ SIGNATURES = {
     "rocshmem_amd_my_pe": (_i, []),
     "rocshmem_amd_set_pe": (_i, [_i]),
     "rocshmem_amd_set_pe_rule": (_i, [_i]),
+    "rocshmem_amd_set_ctx_options": (C.c_int64, [C.c_int64]),
     "rocshmem_amd_malloc": (_vp, [_sz]),
     "rocshmem_amd_free": (_i, [_vp]),
     "rocshmem_amd_pe_ptr": (_vp, [_vp, _i]),
@@ -63,6 +65,8 @@ SIGNATURES = {
     "rocshmem_amd_timer_elapsed_ms": (C.c_float, [_vp]),
     "rocshmem_amd_timer_destroy": (_i, [_vp]),
     "rocshmem_amd_rma": (_i, [_i, _i, _vp, _vp, _sz, _sz, _i, _i, _i, _i, _i, _vp]),
+    "rocshmem_amd_put_flag_check": (_i, [_vp, _vp, _sz, _i, _i, _i, _i, _i, _i,
+                                         C.POINTER(_u64), C.POINTER(_i), _vp]),
     "rocshmem_amd_putmem": (_i, [_vp, _vp, _sz, _i, _i, _vp]),
     "rocshmem_amd_getmem": (_i, [_vp, _vp, _sz, _i, _i, _vp]),
     "rocshmem_amd_wf_coalesce": (_i, [_vp, _vp, _vp, _vp, _u64, _vp, _vp]),

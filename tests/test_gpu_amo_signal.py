@@ -14,6 +14,17 @@ NP = {"INT": np.int32, "LONG": np.int64, "LONGLONG": np.int64, "UINT": np.uint32
       "SHORT": np.int16}
 
 
+@pytest.fixture(autouse=True, params=[0, 1], ids=["default_ctx", "nostore_ctx"])
+def ctx_options(request, rt):
+    """Every case runs through default contexts and through contexts created
+    with ROCSHMEM_CTX_NOSTORE (relaxed AMOs, no L2 write-back on completion):
+    the values that land must not depend on it."""
+    l = rt.up(P, HEAP)
+    before = l.set_ctx_options(request.param)
+    yield request.param
+    l.set_ctx_options(max(before, 0))
+
+
 class Counters:
     """n_slots symmetric counters per PE, viewed as one PE-major array."""
 

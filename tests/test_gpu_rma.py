@@ -24,7 +24,8 @@ def env(rt, L, orc):
     l.free(dst)
 
 
-def run_case(rt, L, orc, env, op, gran, n, soff, doff, n_wgs, wg_size, my_pe=0, pe=1, tile=0):
+def run_case(rt, L, orc, env, op, gran, n, soff, doff, n_wgs, wg_size, my_pe=0, pe=1, tile=0,
+             ctx_options=0):
     """Copies n bytes from src+soff to dst+doff across PEs and checks the
     destination window including GUARD bytes on both sides."""
     l = env["l"]
@@ -44,7 +45,9 @@ def run_case(rt, L, orc, env, op, gran, n, soff, doff, n_wgs, wg_size, my_pe=0, 
         landing = l.pe_ptr(dst, my_pe) + base + doff
         d_arg, s_arg = landing, remote_mine
     l.fill(landing - GUARD, 0xA5, n + 2 * GUARD)
+    before = l.set_ctx_options(ctx_options)
     rc = l.rma(op, gran, d_arg, s_arg, n, tile, my_pe, pe, n_wgs, wg_size, 1, None)
+    l.set_ctx_options(before)
     assert rc == 0
     l.stream_sync(None)
     got = rt.get_bytes(landing - GUARD, n + 2 * GUARD)
@@ -106,6 +109,49 @@ def test_tiled_multi_group_transfers(rt, L, orc, env, gran):
                                (5000, 4, 64, 17)]:
         run_case(rt, L, orc, env, L.PUT, getattr(L, gran), n, 1, 9, n_wgs, wg, tile=tile)
         run_case(rt, L, orc, env, L.GET, getattr(L, gran), n, 6, 0, n_wgs, wg, tile=tile)
+
+
+@pytest.mark.parametrize("gran", GRANS)
+def test_nostore_context_moves_the_same_bytes(rt, L, orc, env, gran):
+    """A context created with ROCSHMEM_CTX_NOSTORE (src/fence_policy.hpp:45-63)
+    completes its puts without the L2 write-back; the bytes that land are the
+    same for every size class, alignment and tiling."""
+    g = getattr(L, gran)
+    for n in list(range(0, 70)) + [255, 256, 1000, 4099, 65536, 65537, 100001]:
+        run_case(rt, L, orc, env, L.PUT, g, n, 3, 5, 1, 128, ctx_options=L.CTX_NOSTORE)
+    for soff in range(0, 16, 3):
+        for doff in range(16):
+            run_case(rt, L, orc, env, L.PUT, g, 777, soff, doff, 2, 64, ctx_options=L.CTX_NOSTORE)
+    for n, n_wgs, wg, tile in [(1 << 20, 64, 256, 4096), (1 << 22, 128, 1024, 65536), (5000, 4, 64, 17)]:
+        run_case(rt, L, orc, env, L.PUT, g, n, 1, 9, n_wgs, wg, tile=tile, ctx_options=L.CTX_NOSTORE)
+        run_case(rt, L, orc, env, L.GET, g, n, 6, 0, n_wgs, wg, tile=tile, ctx_options=L.CTX_NOSTORE)
+
+
+@pytest.mark.parametrize("with_signal", [0, 1])
+@pytest.mark.parametrize("ctx_options", [0, 1])
+@pytest.mark.parametrize("nbytes,pairs,wg", [(4096, 1, 64), (65536, 16, 256), (1 << 20, 64, 1024),
+                                             (262144 + 4, 128, 256)])
+def test_put_quiet_flag_seen_in_order(rt, L, env, ctx_options, with_signal, nbytes, pairs, wg):
+    """Message passing inside one kernel: the receiver, released by a relaxed
+    flag that follows rocshmem_ctx_quiet (src/ipc/context_ipc_device.cpp:100-102)
+    or by the signal of putmem_signal_wg (:221-247), must find every word of the
+    payload, on a default context and on a ROCSHMEM_CTX_NOSTORE one, over 20
+    rounds with a new pattern each."""
+    import ctypes as C
+    l = env["l"]
+    data = l.malloc(nbytes * pairs)
+    flags = l.malloc(16 * pairs)
+    assert data and flags
+    bad, timed_out = C.c_uint64(99), C.c_int(99)
+    before = l.set_ctx_options(ctx_options)
+    rc = l.put_flag_check(l.pe_ptr(data, 1), l.pe_ptr(flags, 1), nbytes, pairs, 20, 1, 6, wg,
+                          with_signal, C.byref(bad), C.byref(timed_out), None)
+    l.set_ctx_options(before)
+    assert rc == 0
+    assert timed_out.value == 0
+    assert bad.value == 0
+    l.free(data)
+    l.free(flags)
 
 
 def test_every_pe_pair(rt, L, orc, env):
