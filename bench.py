@@ -181,7 +181,7 @@ def zipf_table(K, s):
     return np.cumsum(w / w.sum())
 
 
-def dispatch_config(b, steps):
+def dispatch_config(b, steps, shapes=((64, 1024),)):
     """configs[4] part 2: put_signal dispatch, 4096 tokens/PE, top-8 of 256
     experts by Zipf(1.1), rows of 7168 bf16."""
     l = b.l
@@ -214,19 +214,23 @@ def dispatch_config(b, steps):
         b.fill_random(l.pe_ptr(send, p), rows_out * row, p, 40 + p)
     tabs = [np.ascontiguousarray(a, np.uint32) for a in (counts, send_row, recv_row)]
 
+    shape = [shapes[0]]
+
     def step():
-        for p in range(P):  # signals start from zero each dispatch
-            l.fill(l.pe_ptr(sig, p), 0, 8 * P)
+        assert l.fill_every_pe(sig, 0, 8 * P, None) == 0  # signals start from zero each dispatch
         assert l.dispatch_put_signal(recv, send, sig, tabs[0].ctypes.data, tabs[1].ctypes.data,
-                                     tabs[2].ctypes.data, row, 128, 1024, None) == 0
+                                     tabs[2].ctypes.data, row, shape[0][0], shape[0][1], None) == 0
 
     alg = 2 * int(counts.sum()) * row
     res = {"rows": int(counts.sum())}
     for name, opt in CTX_KINDS:
         l.set_ctx_options(opt)
-        ms = b.time_ms(step, max(5, steps // 10), 2)
-        res[name] = {"ms": round(ms, 4), "gbs": round(alg / ms / 1e6, 1),
-                     "frac": round(alg / ms / 1e6 / HBM_PEAK_GBS, 4)}
+        for sh in shapes:
+            shape[0] = sh
+            ms = b.time_ms(step, max(5, steps // 10), 2)
+            key = name if len(shapes) == 1 else "%s_rows%d_wg%d" % (name, sh[0], sh[1])
+            res[key] = {"ms": round(ms, 4), "gbs": round(alg / ms / 1e6, 1),
+                        "frac": round(alg / ms / 1e6 / HBM_PEAK_GBS, 4)}
     l.set_ctx_options(0)
     for x in (send, recv, sig):
         l.free(x)

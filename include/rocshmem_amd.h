@@ -166,6 +166,9 @@ int rocshmem_amd_dev_free(void *ptr);
 int rocshmem_amd_copy_in(void *dst_dev, const void *src_host, size_t n);
 int rocshmem_amd_copy_out(void *dst_host, const void *src_dev, size_t n);
 int rocshmem_amd_fill(void *dst_dev, int byte, size_t n);
+/* The symmetric object `sym` (address on PE 0) set to `byte` on every PE with
+ * one launch on `stream` — e.g. signal words cleared between dispatches. */
+int rocshmem_amd_fill_every_pe(void *sym, int byte, size_t n, rocshmem_amd_stream_t stream);
 /* hipMemcpy device-to-device by the HIP runtime's own copy kernel: a plain copy
  * of known size to calibrate hardware byte counters against. */
 int rocshmem_amd_copy_dev(void *dst_dev, const void *src_dev, size_t n);

@@ -108,6 +108,14 @@ void launch_bulk(char *dst, const char *src, size_t nbytes, hipStream_t stream) 
   DRV_CHECK_HIP(hipGetLastError());
 }
 
+// The same byte range of every PE's slice set to one value: blockIdx.y is the PE.
+__global__ void fill_every_pe_kernel(char *base, uint64_t pe_stride, size_t nbytes, int byte) {
+  char *p = base + static_cast<uint64_t>(blockIdx.y) * pe_stride;
+  const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nbytes; i += stride)
+    p[i] = static_cast<char>(byte);
+}
+
 __global__ void coalesce_kernel(const int *pe, const uint64_t *src, const uint64_t *dst,
                                 const uint64_t *size, uint64_t active_mask, int *sends,
                                 uint64_t *size_out) {
@@ -164,6 +172,18 @@ int rocshmem_amd_rma(int rma_op, int gran, void *dest, const void *source, size_
   RMA_CASE(ROCSHMEM_AMD_GET, ROCSHMEM_AMD_WAVE)
   RMA_CASE(ROCSHMEM_AMD_GET, ROCSHMEM_AMD_WG)
 #undef RMA_CASE
+  DRV_CHECK_HIP(hipGetLastError());
+  return 0;
+}
+
+int rocshmem_amd_fill_every_pe(void *sym, int byte, size_t nbytes, rocshmem_amd_stream_t stream) {
+  auto &r = runtime::rt();
+  if (!r.live || !sym_ok_on(sym, nbytes, 0)) return -1;
+  if (!nbytes) return 0;
+  const size_t want = (nbytes + 255) / 256;
+  const dim3 grid(static_cast<unsigned>(want < 1024 ? want : 1024), r.npes);
+  hipLaunchKernelGGL(fill_every_pe_kernel, grid, dim3(256), 0, as_stream(stream),
+                     static_cast<char *>(sym), r.pe_stride, nbytes, byte);
   DRV_CHECK_HIP(hipGetLastError());
   return 0;
 }

@@ -361,7 +361,7 @@ struct DispatchArgs {
   const char *send0;
   uint64_t *sig0;
   const uint32_t *count, *send_row, *recv_row;
-  const uint32_t *call_start;  // [P*P+1] first call number of every pair
+  const uint2 *calls;   // [n_calls] {pair, first row of the call within the pair}
   size_t row_bytes;
   uint64_t pe_stride;
   int np;
@@ -379,14 +379,9 @@ __global__ void dispatch_kernel(DispatchArgs a) {
   const unsigned senders = gridDim.x - P;
   if (blockIdx.x < senders) {
     for (uint32_t c = blockIdx.x; c < a.n_calls; c += senders) {
-      // pair whose call range holds c: P*P+1 sorted entries, binary search
-      int lo = 0, hi = P * P;
-      while (hi - lo > 1) {
-        const int mid = (lo + hi) >> 1;
-        if (a.call_start[mid] <= c) lo = mid; else hi = mid;
-      }
-      const int pair = lo, s = pair / P, d = pair % P;
-      const uint32_t first = (c - a.call_start[pair]) * a.rows_per_call;
+      const uint2 call = a.calls[c];
+      const int pair = static_cast<int>(call.x), s = pair / P, d = pair % P;
+      const uint32_t first = call.y;
       const uint32_t cnt = a.count[pair];
       const uint32_t rows = cnt - first < a.rows_per_call ? cnt - first : a.rows_per_call;
       rocshmem_ctx_t ctx{a.ctx_row + s, &a.world_row[s].wrt_world};
@@ -755,7 +750,7 @@ int rocshmem_amd_put_flag_check(void *data, uint64_t *flags, size_t nbytes, int 
 // with the same tables only launches.
 namespace {
 struct DispatchTables {
-  std::vector<uint32_t> host;  // count | send_row | recv_row | call_start
+  std::vector<uint32_t> host;  // count | send_row | recv_row | calls {pair, first row}
   uint32_t *dev = nullptr;
   size_t pp = 0;
   uint32_t rows_per_call = 0;
@@ -775,7 +770,7 @@ int rocshmem_amd_dispatch_put_signal(void *recv, const void *send, uint64_t *sig
   if (!count || !send_row || !recv_row) return -1;
   const size_t pp = static_cast<size_t>(r.npes) * r.npes;
   DispatchTables &t = g_tables;
-  std::vector<uint32_t> h(4 * pp + 1);
+  std::vector<uint32_t> h(3 * pp);
   std::copy(count, count + pp, h.begin());
   std::copy(send_row, send_row + pp, h.begin() + pp);
   std::copy(recv_row, recv_row + pp, h.begin() + 2 * pp);
@@ -788,10 +783,12 @@ int rocshmem_amd_dispatch_put_signal(void *recv, const void *send, uint64_t *sig
     for (size_t i = 0; i < pp; ++i) {
       t.max_send = std::max<size_t>(t.max_send, static_cast<size_t>(h[pp + i]) + h[i]);
       t.max_recv = std::max<size_t>(t.max_recv, static_cast<size_t>(h[2 * pp + i]) + h[i]);
-      h[3 * pp + i] = calls;
-      calls += (h[i] + rows_per_call - 1) / rows_per_call;
+      for (uint32_t first = 0; first < h[i]; first += static_cast<uint32_t>(rows_per_call)) {
+        h.push_back(static_cast<uint32_t>(i));
+        h.push_back(first);
+        ++calls;
+      }
     }
-    h[4 * pp] = calls;
     DRV_CHECK_HIP(hipDeviceSynchronize());  // nobody is reading the old tables any more
     if (t.dev) DRV_CHECK_HIP(hipFree(t.dev));
     DRV_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&t.dev), h.size() * 4));
@@ -811,7 +808,7 @@ int rocshmem_amd_dispatch_put_signal(void *recv, const void *send, uint64_t *sig
   a.count = t.dev;
   a.send_row = t.dev + pp;
   a.recv_row = t.dev + 2 * pp;
-  a.call_start = t.dev + 3 * pp;
+  a.calls = reinterpret_cast<const uint2 *>(t.dev + 3 * pp);
   a.row_bytes = row_bytes;
   a.pe_stride = r.pe_stride;
   a.np = r.npes;
@@ -819,7 +816,7 @@ int rocshmem_amd_dispatch_put_signal(void *recv, const void *send, uint64_t *sig
   a.n_calls = t.n_calls;
   a.ctx_row = r.driver_ctx_row();
   a.world_row = r.d_teams;
-  const uint32_t max_senders = 256 * 16;
+  const uint32_t max_senders = 256 * 64;
   const uint32_t senders = a.n_calls < max_senders ? (a.n_calls ? a.n_calls : 1) : max_senders;
   hipLaunchKernelGGL(dispatch_kernel, dim3(senders + r.npes), dim3(wg_size), 0, as_stream(stream), a);
   DRV_CHECK_HIP(hipGetLastError());

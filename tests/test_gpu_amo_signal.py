@@ -340,7 +340,8 @@ def test_dispatch_put_signal(rt, L, orc, rows_per_call):
         packed.append(rows)
         rt.put_bytes(l.pe_ptr(send, s), rows)
         l.fill(l.pe_ptr(recv, s), 0, max_rows * row)
-        l.fill(l.pe_ptr(sig, s), 0, 8 * P)
+        l.fill(l.pe_ptr(sig, s), 0xFF, 8 * P)
+    assert l.fill_every_pe(sig, 0, 8 * P, None) == 0
     counts, send_row, recv_row = (np.ascontiguousarray(a, np.uint32) for a in (counts, send_row, recv_row))
     assert l.dispatch_put_signal(recv, send, sig, counts.ctypes.data, send_row.ctypes.data,
                                  recv_row.ctypes.data, row, rows_per_call, 256, None) == 0

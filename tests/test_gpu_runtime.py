@@ -63,6 +63,23 @@ def test_same_offset_on_every_pe_and_slices_do_not_overlap(rt, L):
     l.free(a)
 
 
+def test_fill_every_pe_touches_exactly_the_object(rt, L):
+    l = rt.up(4, 1 << 26)
+    for n in (1, 64, 1000, 300001):
+        obj = l.malloc(n + 128)
+        for pe in range(4):
+            l.fill(l.pe_ptr(obj, pe), 0x11, n + 128)
+        assert l.fill_every_pe(obj + 64, 0xC3, n, None) == 0
+        l.stream_sync(None)
+        for pe in range(4):
+            got = rt.get_bytes(l.pe_ptr(obj, pe), n + 128)
+            assert (got[:64] == 0x11).all() and (got[64 + n:] == 0x11).all(), (n, pe)
+            assert (got[64:64 + n] == 0xC3).all(), (n, pe)
+        l.free(obj)
+    assert l.fill_every_pe(None, 0, 8, None) == -1
+    assert l.fill_every_pe(l.pe_ptr(l.malloc(128), 1), 0, 8, None) == -1  # not PE 0's address
+
+
 def test_teams(rt, L, orc):
     """src/rocshmem.cpp:193-319 and tests/sos_tests/shmem_team_translate.cpp."""
     l = rt.up(8, 1 << 24)
