@@ -68,13 +68,18 @@ class Bench:
         l.timer_stop(self.timer, None)
         return l.timer_elapsed_ms(self.timer) / steps
 
-    def fill_random(self, ptr, nbytes, pe, seed):
+    def fill_random(self, ptr, nbytes, pe, seed, kind="u8"):
         """Random payload resident on the device: a seeded 4 MiB tile uploaded
-        once and doubled in place by on-device copies."""
+        once and doubled in place by on-device copies.  kind: "u8" uniform
+        bytes, "f32" / "bf16" N(0,1) values (bf16 by truncating the fp32)."""
         l = self.l
         tile = min(nbytes, 4 * MiB)
         rng = np.random.default_rng(seed)
-        host = rng.integers(0, 256, tile, dtype=np.uint8)
+        if kind == "u8":
+            host = rng.integers(0, 256, tile, dtype=np.uint8)
+        else:
+            f = rng.standard_normal(tile // (4 if kind == "f32" else 2), dtype=np.float32)
+            host = f if kind == "f32" else (f.view(np.uint32) >> 16).astype(np.uint16)
         l.copy_in(ptr, host.ctypes.data, tile)
         done = tile
         while done < nbytes:
@@ -108,18 +113,29 @@ def headline(b, steps, warmup):
 
     ms = b.time_ms(rotating(lambda me, pe: l.putmem(dsts[me], srcs[me], n, me, pe, None)), steps, warmup)
     out = {"bytes_per_step": 2 * n, "ms": ms, "gbs": 2 * n / ms / 1e6}
-    # the rest of the bandwidth curve (device API, one work-group and all CUs)
+    # The bandwidth curve, 8 B .. 256 MiB (26 sizes).  One work-group of 64, 256
+    # and 1024 threads issuing rocshmem_putmem_wg / getmem_wg: the call is
+    # repeated inside the kernel (as the reference's testers loop inside theirs)
+    # so the launch does not count; small messages are then re-read from cache.
+    # All CUs: the host-initiated copy, one launch per message, launch included.
     curve = {}
-    for e in (3, 6, 10, 13, 16, 20, 24, 28):
+    reps = max(3, min(steps, 10))
+    for e in range(3, 29):
         m = 1 << e
-        reps = max(3, min(steps, 20))
-        t1 = b.time_ms(rotating(lambda me, pe: l.rma(b.L.PUT, b.L.WG, dsts[me], srcs[me], m, 0, me, pe,
-                                                     1, 1024, 1, None)), reps if e < 24 else 3, 2)
+        inner = 200 if e <= 16 else (20 if e <= 24 else 2)
+        point = {}
+        for threads in (64, 256, 1024):
+            t = b.time_ms(rotating(lambda me, pe: l.rma(b.L.PUT, b.L.WG, dsts[me], srcs[me], m, 0, me, pe,
+                                                        1, threads, inner, None)), 3, 1) / inner
+            point["putmem_wg_1wg_%dthr_gbs" % threads] = round(2 * m / t / 1e6, 3)
+        t = b.time_ms(rotating(lambda me, pe: l.rma(b.L.GET, b.L.WG, dsts[me], srcs[me], m, 0, me, pe,
+                                                    1, 1024, inner, None)), 3, 1) / inner
+        point["getmem_wg_1wg_1024thr_gbs"] = round(2 * m / t / 1e6, 3)
         tg = b.time_ms(rotating(lambda me, pe: l.putmem(dsts[me], srcs[me], m, me, pe, None)), reps, 2)
         tget = b.time_ms(rotating(lambda me, pe: l.getmem(dsts[me], srcs[me], m, me, pe, None)), reps, 2)
-        curve[str(m)] = {"putmem_wg_1wg_gbs": round(2 * m / t1 / 1e6, 3),
-                         "putmem_all_cus_gbs": round(2 * m / tg / 1e6, 3),
-                         "getmem_all_cus_gbs": round(2 * m / tget / 1e6, 3)}
+        point["putmem_all_cus_gbs"] = round(2 * m / tg / 1e6, 3)
+        point["getmem_all_cus_gbs"] = round(2 * m / tget / 1e6, 3)
+        curve[str(m)] = point
     out["curve"] = curve
     # Device API from every CU: rocshmem_ctx_putmem_wg on 64 KiB tiles, one
     # quiet per work-group, through a default and a NOSTORE context.
@@ -147,10 +163,9 @@ def to_all_configs(b, steps, warmup):
                              ("fp32_max", L.FLOAT, L.MAX, 4), ("bf16_sum", L.BF16, L.SUM, 2)):
         src, dst = l.malloc(n * es), l.malloc(n * es)
         assert src and dst, name
+        kind = {L.FLOAT: "f32", L.BF16: "bf16"}.get(dt, "u8")
         for p in range(P):
-            b.fill_random(l.pe_ptr(src, p), n * es, p, 10 + p)
-            if dt in (L.FLOAT, L.BF16):
-                pass  # random bit patterns: NaNs cost the same as numbers here
+            b.fill_random(l.pe_ptr(src, p), n * es, p, 10 + p, kind)
         ms = b.time_ms(lambda: l.to_all(dt, op, dst, src, n, 0, 0, P, None), max(5, steps // 5), 3)
         alg = 2 * P * n * es
         res[name] = {"ms": round(ms, 4), "gbs": round(alg / ms / 1e6, 1),
@@ -269,24 +284,33 @@ def amo_config(b, steps):
 
 
 def pingpong_config(b):
-    """configs[5] part 2: put_signal / wait_until ping-pong between two
-    work-groups acting as two PEs."""
+    """configs[5] part 2: put_signal / wait_until ping-pong between work-groups
+    acting as two PEs: one pair over 14 payload sizes, and 8 and 32 pairs at
+    once at 8 B and 4 KiB (aggregate message rate)."""
     l = b.l
-    buf, sig = l.malloc(65536), l.malloc(8)
+    max_pairs = 32
+    buf, sig = l.malloc(65536 * max_pairs), l.malloc(8 * max_pairs)
     res = {}
     iters = 2000
-    for k in range(3, 17):
-        n = 1 << k
-        res[str(n)] = {}
+
+    def run(n, pairs):
+        out = {}
         for name, opt in CTX_KINDS:
             l.set_ctx_options(opt)
-            for p in (0, 1):
-                l.fill(l.pe_ptr(sig, p), 0, 8)
+            assert l.fill_every_pe(sig, 0, 8 * max_pairs, None) == 0
             ticks, hz = C.c_uint64(), C.c_double()
-            assert l.pingpong(buf, sig, n, iters, 0, 1, 256, C.byref(ticks), C.byref(hz), None) == 0
+            assert l.pingpong(buf, sig, n, iters, pairs, 0, 1, 256, C.byref(ticks), C.byref(hz),
+                              None) == 0
             one_way_us = ticks.value / hz.value / iters / 2 * 1e6
-            res[str(n)][name] = {"latency_us": round(one_way_us, 3),
-                                 "msg_per_s": round(1e6 / one_way_us, 1)}
+            out[name] = {"latency_us": round(one_way_us, 3),
+                         "msg_per_s": round(pairs * 1e6 / one_way_us, 1)}
+        return out
+
+    for k in range(3, 17):
+        res[str(1 << k)] = run(1 << k, 1)
+    for pairs in (8, 32):
+        for n in (8, 4096):
+            res["%d_x%dpairs" % (n, pairs)] = run(n, pairs)
     l.set_ctx_options(0)
     l.free(buf)
     l.free(sig)

@@ -307,15 +307,19 @@ int rocshmem_amd_put_flag_check(void *data, uint64_t *flags, size_t nbytes, int 
                                 rocshmem_amd_stream_t stream);
 
 /* Ping-pong (tests/functional_tests/ping_pong_tester.cpp:43-61,
- * examples/rocshmem_put_signal_test.cc:31-47): work-group 0 acts for pe_a,
- * work-group 1 for pe_b; `iters` round trips of putmem_signal_wg (payload
- * nbytes from `buf` to the peer's `buf`, signal word `sig` set to the round
- * number) answered after rocshmem_ulong_wait_until.  buf/sig: addresses on
- * pe_a.  ticks_out (host, optional) receives the wall_clock64 ticks pe_a
+ * examples/rocshmem_put_signal_test.cc:31-47; the reference runs it with 1, 8
+ * and 32 work-groups, scripts/functional_tests/driver.sh:313-315): `pairs`
+ * (<= 128) pairs of work-groups at once, the even one of a pair acting for
+ * pe_a, the odd one for pe_b; `iters` round trips of putmem_signal_wg (payload
+ * nbytes from the pair's slot of `buf` to the same slot on the peer, the
+ * pair's word of `sig` set to the round number) answered after
+ * rocshmem_ulong_wait_until.  Slots are nbytes rounded up to 256 bytes apart;
+ * sig holds `pairs` words.  buf/sig: addresses on pe_a.  ticks_out (host,
+ * optional) receives the wall_clock64 ticks the slowest pair's pe_a side
  * spent; tick_hz_out the tick rate. */
-int rocshmem_amd_pingpong(void *buf, uint64_t *sig, size_t nbytes, int iters, int pe_a,
-                          int pe_b, int wg_size, uint64_t *ticks_out, double *tick_hz_out,
-                          rocshmem_amd_stream_t stream);
+int rocshmem_amd_pingpong(void *buf, uint64_t *sig, size_t nbytes, int iters, int pairs,
+                          int pe_a, int pe_b, int wg_size, uint64_t *ticks_out,
+                          double *tick_hz_out, rocshmem_amd_stream_t stream);
 
 /* MoE-style dispatch with put_signal.  For every ordered pair (s, d) of the P
  * world PEs, rows [send_row[s*P+d], +count[s*P+d]) of s's `send` buffer go to

@@ -226,21 +226,24 @@ struct PingPongArgs {
   char *buf_a;      // address on pe_a
   uint64_t *sig_a;  // address on pe_a
   size_t nbytes;
+  size_t slot_bytes;  // distance between the buffers of consecutive pairs
   int iters;
   int pe_a, pe_b;
   uint64_t pe_stride;
   detail::Context *ctx_row;
   detail::Team *world_row;
-  unsigned long long *ticks;
+  unsigned long long *ticks;  // [pairs]
 };
 
 __global__ void pingpong_kernel(PingPongArgs a) {
-  const bool is_a = blockIdx.x == 0;
+  // Work-groups 2k and 2k+1 are the two ends of pair k.
+  const bool is_a = (blockIdx.x & 1) == 0;
+  const size_t pair = blockIdx.x >> 1;
   const int me = is_a ? a.pe_a : a.pe_b;
   const int peer = is_a ? a.pe_b : a.pe_a;
   const int64_t shift = static_cast<int64_t>(me - a.pe_a) * static_cast<int64_t>(a.pe_stride);
-  char *buf = a.buf_a + shift;
-  uint64_t *sig = reinterpret_cast<uint64_t *>(reinterpret_cast<char *>(a.sig_a) + shift);
+  char *buf = a.buf_a + shift + pair * a.slot_bytes;
+  uint64_t *sig = reinterpret_cast<uint64_t *>(reinterpret_cast<char *>(a.sig_a) + shift) + pair;
   rocshmem_ctx_t ctx{a.ctx_row + me, &a.world_row[me].wrt_world};
   const unsigned long long t0 = wall_clock64();
   for (int r = 1; r <= a.iters; ++r) {
@@ -261,7 +264,7 @@ __global__ void pingpong_kernel(PingPongArgs a) {
     }
   }
   const unsigned long long t1 = wall_clock64();
-  if (is_a && threadIdx.x == 0) *a.ticks = t1 - t0;
+  if (is_a && threadIdx.x == 0) a.ticks[pair] = t1 - t0;
 }
 
 // ---------------------------------------------------------------------------
@@ -653,21 +656,24 @@ int rocshmem_amd_signal_fetch(int gran, const uint64_t *sig_addr, int my_pe, uin
   return out[1] == 0 ? 0 : -2;
 }
 
-int rocshmem_amd_pingpong(void *buf, uint64_t *sig, size_t nbytes, int iters, int pe_a, int pe_b,
-                          int wg_size, uint64_t *ticks_out, double *tick_hz_out,
-                          rocshmem_amd_stream_t stream) {
-  if (!valid_pe(pe_a) || !valid_pe(pe_b) || pe_a == pe_b || !valid_launch(2, wg_size) ||
-      iters < 0 || nbytes == 0)
+int rocshmem_amd_pingpong(void *buf, uint64_t *sig, size_t nbytes, int iters, int pairs,
+                          int pe_a, int pe_b, int wg_size, uint64_t *ticks_out,
+                          double *tick_hz_out, rocshmem_amd_stream_t stream) {
+  if (!valid_pe(pe_a) || !valid_pe(pe_b) || pe_a == pe_b || pairs < 1 || pairs > 128 ||
+      !valid_launch(2 * pairs, wg_size) || iters < 0 || nbytes == 0)
     return -1;
-  if (!sym_ok_on(buf, nbytes, pe_a) || !sym_ok_on(sig, 8, pe_a)) return -1;
+  const size_t slot = (nbytes + 255) / 256 * 256;
+  if (!sym_ok_on(buf, slot * (pairs - 1) + nbytes, pe_a) || !sym_ok_on(sig, 8u * pairs, pe_a))
+    return -1;
   auto &r = runtime::rt();
   unsigned long long *d_ticks;
-  DRV_CHECK_HIP(hipMalloc(&d_ticks, sizeof(unsigned long long)));
-  DRV_CHECK_HIP(hipMemset(d_ticks, 0, sizeof(unsigned long long)));
+  DRV_CHECK_HIP(hipMalloc(&d_ticks, sizeof(unsigned long long) * pairs));
+  DRV_CHECK_HIP(hipMemset(d_ticks, 0, sizeof(unsigned long long) * pairs));
   PingPongArgs a;
   a.buf_a = static_cast<char *>(buf);
   a.sig_a = sig;
   a.nbytes = nbytes;
+  a.slot_bytes = slot;
   a.iters = iters;
   a.pe_a = pe_a;
   a.pe_b = pe_b;
@@ -676,13 +682,15 @@ int rocshmem_amd_pingpong(void *buf, uint64_t *sig, size_t nbytes, int iters, in
   a.world_row = r.d_teams;
   a.ticks = d_ticks;
   hipStream_t s = as_stream(stream);
-  hipLaunchKernelGGL(pingpong_kernel, dim3(2), dim3(wg_size), 0, s, a);
+  hipLaunchKernelGGL(pingpong_kernel, dim3(2 * pairs), dim3(wg_size), 0, s, a);
   DRV_CHECK_HIP(hipGetLastError());
   DRV_CHECK_HIP(hipStreamSynchronize(s));
-  unsigned long long ticks = 0;
-  DRV_CHECK_HIP(hipMemcpy(&ticks, d_ticks, sizeof(ticks), hipMemcpyDeviceToHost));
+  std::vector<unsigned long long> ticks(pairs);
+  DRV_CHECK_HIP(hipMemcpy(ticks.data(), d_ticks, sizeof(unsigned long long) * pairs,
+                          hipMemcpyDeviceToHost));
   DRV_CHECK_HIP(hipFree(d_ticks));
-  if (ticks_out) *ticks_out = ticks;
+  // The slowest pair: all pairs run the same number of round trips at once.
+  if (ticks_out) *ticks_out = *std::max_element(ticks.begin(), ticks.end());
   if (tick_hz_out) {
     int khz = 0, dev = 0;
     DRV_CHECK_HIP(hipGetDevice(&dev));

@@ -84,7 +84,7 @@ SIGNATURES = {
     "rocshmem_amd_amo": (_i, [_i, _i, _vp, _u32, _vp, _vp, _vp, _vp, _sz, _i, _i, _i, _vp]),
     "rocshmem_amd_put_signal": (_i, [_i, _vp, _vp, _sz, _vp, _u64, _i, _i, _i, _i, _i, _i, _vp]),
     "rocshmem_amd_signal_fetch": (_i, [_i, _vp, _i, C.POINTER(_u64)]),
-    "rocshmem_amd_pingpong": (_i, [_vp, _vp, _sz, _i, _i, _i, _i, C.POINTER(_u64),
+    "rocshmem_amd_pingpong": (_i, [_vp, _vp, _sz, _i, _i, _i, _i, _i, C.POINTER(_u64),
                                    C.POINTER(C.c_double), _vp]),
     "rocshmem_amd_dispatch_put_signal": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _vp]),
     "rocshmem_amd_wait_test": (_i, [_i, _i, _vp, _sz, _vp, _i, _vp, C.POINTER(_sz), _vp]),

@@ -267,25 +267,33 @@ def test_signal_fetch(rt, L, gran):
     l.free(sig)
 
 
+@pytest.mark.parametrize("pairs", [1, 8, 32])
 @pytest.mark.parametrize("nbytes", [8, 64, 1024, 65536])
-def test_pingpong(rt, L, orc, nbytes):
-    """ping_pong_tester.cpp:43-61: after `iters` round trips both signal words
-    hold `iters` and both buffers hold the payload that bounced."""
+def test_pingpong(rt, L, orc, nbytes, pairs):
+    """ping_pong_tester.cpp:43-61, run with 1, 8 and 32 work-groups as
+    scripts/functional_tests/driver.sh:313-315 does: after `iters` round trips
+    both signal words of every pair hold `iters` and both buffers hold the
+    payload that bounced."""
     l = rt.up(P, HEAP)
-    buf, sig = l.malloc(nbytes), l.malloc(8)
-    host = orc.fill_u8(nbytes, 2, 3)
+    slot = (nbytes + 255) // 256 * 256
+    buf, sig = l.malloc(slot * pairs), l.malloc(8 * pairs)
+    host = orc.fill_u8(slot * pairs, 2, 3)
     rt.put_bytes(l.pe_ptr(buf, 2), host)
-    l.fill(l.pe_ptr(buf, 6), 0, nbytes)
+    l.fill(l.pe_ptr(buf, 6), 0, slot * pairs)
     for p in (2, 6):
-        l.fill(l.pe_ptr(sig, p), 0, 8)
+        l.fill(l.pe_ptr(sig, p), 0, 8 * pairs)
     ticks, hz = ctypes.c_uint64(), ctypes.c_double()
-    iters = 500
-    assert l.pingpong(l.pe_ptr(buf, 2), l.pe_ptr(sig, 2), nbytes, iters, 2, 6, 256,
+    iters = 300
+    assert l.pingpong(l.pe_ptr(buf, 2), l.pe_ptr(sig, 2), nbytes, iters, pairs, 2, 6, 256,
                       ctypes.byref(ticks), ctypes.byref(hz), None) == 0
-    for p in (2, 6):
-        assert int(rt.get_bytes(l.pe_ptr(sig, p), 8, np.uint64)[0]) == iters
-        assert np.array_equal(rt.get_bytes(l.pe_ptr(buf, p), nbytes), host)
+    want = host.copy().reshape(pairs, slot)
+    want_b = np.zeros_like(want)
+    want_b[:, :nbytes] = want[:, :nbytes]  # only the payload crosses; slot padding stays
+    for p, w in ((2, want), (6, want_b)):
+        assert (rt.get_bytes(l.pe_ptr(sig, p), 8 * pairs, np.uint64) == iters).all()
+        assert np.array_equal(rt.get_bytes(l.pe_ptr(buf, p), slot * pairs).reshape(pairs, slot), w)
     assert ticks.value > 0 and hz.value > 1e6
+    assert l.pingpong(l.pe_ptr(buf, 2), l.pe_ptr(sig, 2), nbytes, 1, 129, 2, 6, 256, None, None, None) == -1
     l.free(buf)
     l.free(sig)
 
