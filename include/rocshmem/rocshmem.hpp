@@ -47,6 +47,7 @@ static inline int MPI_Abort(MPI_Comm, int errorcode) {
 #include "rocshmem_P2P_SYNC.hpp"
 #include "rocshmem_RMA_X.hpp"
 #include "rocshmem_emu.hpp"
+#include "rocshmem_HOST.hpp"
 
 namespace rocshmem {
 

@@ -45,7 +45,12 @@ enum rocshmem_amd_dtype {
   ROCSHMEM_AMD_BF16 = 6,
   ROCSHMEM_AMD_UINT = 7,
   ROCSHMEM_AMD_ULONG = 8,
-  ROCSHMEM_AMD_ULONGLONG = 9
+  ROCSHMEM_AMD_ULONGLONG = 9,
+  /* host-side waits only */
+  ROCSHMEM_AMD_CHAR = 10,
+  ROCSHMEM_AMD_SCHAR = 11,
+  ROCSHMEM_AMD_UCHAR = 12,
+  ROCSHMEM_AMD_USHORT = 13
 };
 
 /* Reduction operators: values of ROCSHMEM_OP (rocshmem_common.hpp:40-49). */
@@ -258,6 +263,54 @@ int rocshmem_amd_broadcastmem(rocshmem_amd_team_t team, void *dest, const void *
                               size_t nbytes, int pe_root, rocshmem_amd_stream_t stream);
 int rocshmem_amd_fcollectmem(rocshmem_amd_team_t team, void *dest, const void *source,
                              size_t nbytes, rocshmem_amd_stream_t stream);
+
+/* ========================= host-side operations =========================== */
+
+/* The __host__ halves of rocshmem_RMA.hpp / rocshmem_AMO.hpp /
+ * rocshmem_P2P_SYNC.hpp, which the reference forwards to MPI one-sided calls
+ * on a window over the heap (src/host/host.cpp:162-249).  The typed C++ names
+ * (include/rocshmem/rocshmem_HOST.hpp) are inline wrappers over these.  All of
+ * them are complete when they return. */
+
+/* PE a context handle belongs to (rocshmem_ctx_t::ctx_opaque, as filled in by
+ * rocshmem_ctx_create or a driver); the acting PE for NULL; -1 if the pointer
+ * is not a context of this runtime. */
+int rocshmem_amd_ctx_pe(const void *ctx_opaque);
+/* rocshmem_ctx_putmem / rocshmem_ctx_getmem called from the host
+ * (rocshmem_RMA.hpp:237-242,618-623; src/host/host_helpers.hpp:52-88:
+ * MPI_Put / MPI_Get + flush).  The symmetric side is given as my_pe's address
+ * and resolved on `pe`; the local side may be host memory (pageable or pinned)
+ * or device memory. */
+int rocshmem_amd_host_putmem(void *dest, const void *source, size_t nbytes, int my_pe, int pe);
+int rocshmem_amd_host_getmem(void *dest, const void *source, size_t nbytes, int my_pe, int pe);
+/* One rocshmem_ctx_<T>_atomic_<op> called from the host (rocshmem_AMO.hpp;
+ * src/host/host_templates.hpp:254-330: MPI_Fetch_and_op /
+ * MPI_Compare_and_swap).  value / cond / fetched point at one element of
+ * `dtype` in host memory (cond is read for compare_swap only; fetched may be
+ * NULL). */
+int rocshmem_amd_host_amo(int amo_op, int dtype, void *dest, const void *value, const void *cond,
+                          int my_pe, int pe, void *fetched);
+/* nbytes of device memory as they are now, read on a stream of the library's
+ * own so that a kernel running on another stream does not hold the read back
+ * (the reference reads its own window with MPI_Fetch_and_op(MPI_NO_OP),
+ * src/host/host_templates.hpp:426-446). */
+int rocshmem_amd_host_peek(void *dst_host, const void *src_dev, size_t nbytes);
+/* rocshmem_<T>_test / _wait_until / _wait_until_any / _all / _some called from
+ * the host (rocshmem_P2P_SYNC.hpp; src/host/host_templates.hpp:448-641).
+ * ivars: device memory; status (may be NULL), value, indices_out, ret_out:
+ * host memory.  ret_out: test -> 0/1, any -> index or SIZE_MAX, some -> count,
+ * others -> 0.  timeout_ms < 0 waits for ever; otherwise the call gives up
+ * after that long and returns 1. */
+int rocshmem_amd_host_wait_test(int wait_fn, int dtype, const void *ivars, size_t nelems,
+                                const int *status, int cmp, const void *value, long timeout_ms,
+                                size_t *ret_out, size_t *indices_out);
+/* Host rocshmem_ctx_<T>_broadcast over an active set (rocshmem_COLL.hpp:122-125;
+ * src/host/host_templates.hpp:160-175): nbytes from the root's source to the
+ * dest of every other member.  pe_root counts within the set.  dest/source:
+ * addresses on PE_start. */
+int rocshmem_amd_broadcast_active_set(void *dest, const void *source, size_t nbytes, int pe_root,
+                                      int PE_start, int logPE_stride, int PE_size,
+                                      rocshmem_amd_stream_t stream);
 
 /* ====================== atomics, signals, waits ============================ */
 

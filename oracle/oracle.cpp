@@ -48,7 +48,7 @@ namespace {
 // dtype / op codes (same numbering as include/rocshmem_amd.h)
 // ----------------------------------------------------------------------------
 enum { DT_SHORT, DT_INT, DT_LONG, DT_LONGLONG, DT_FLOAT, DT_DOUBLE, DT_BF16, DT_UINT, DT_ULONG,
-       DT_ULONGLONG };
+       DT_ULONGLONG, DT_CHAR, DT_SCHAR, DT_UCHAR, DT_USHORT };
 enum { OP_SUM, OP_MAX, OP_MIN, OP_PROD, OP_AND, OP_OR, OP_XOR };
 
 inline float bf16_to_f32(uint16_t b) {
@@ -632,7 +632,8 @@ int cmp_typed(int cmp, const void *x, const void *v) {
 }
 size_t dtype_size(int dtype) {
   switch (dtype) {
-    case DT_SHORT: case DT_BF16: return 2;
+    case DT_CHAR: case DT_SCHAR: case DT_UCHAR: return 1;
+    case DT_SHORT: case DT_BF16: case DT_USHORT: return 2;
     case DT_INT: case DT_FLOAT: case DT_UINT: return 4;
     default: return 8;
   }
@@ -649,6 +650,11 @@ ORC_API int orc_test(int dtype, int cmp, const void *x, const void *val) {
     case DT_DOUBLE: return cmp_typed<double>(cmp, x, val);
     case DT_UINT: return cmp_typed<uint32_t>(cmp, x, val);
     case DT_ULONG: case DT_ULONGLONG: return cmp_typed<uint64_t>(cmp, x, val);
+    // The wait types only the host side has (include/rocshmem/rocshmem_P2P_SYNC.hpp:
+    // char, schar, uchar, ushort); plain char is signed on this platform.
+    case DT_CHAR: case DT_SCHAR: return cmp_typed<int8_t>(cmp, x, val);
+    case DT_UCHAR: return cmp_typed<uint8_t>(cmp, x, val);
+    case DT_USHORT: return cmp_typed<uint16_t>(cmp, x, val);
     default: return 0;
   }
 }

@@ -14,14 +14,16 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 ORACLE_PATH = os.path.join(_HERE, "liboracle.so")
 REF_ALLOCATOR_PATH = os.path.join(_HERE, "_ref", "libref_allocator.so")
 
-SHORT, INT, LONG, LONGLONG, FLOAT, DOUBLE, BF16, UINT, ULONG, ULONGLONG = range(10)
+(SHORT, INT, LONG, LONGLONG, FLOAT, DOUBLE, BF16, UINT, ULONG, ULONGLONG, CHAR, SCHAR, UCHAR,
+ USHORT) = range(14)
 SUM, MAX, MIN, PROD, AND, OR, XOR = range(7)
 SIZE_MAX = (1 << 64) - 1
 WOULD_BLOCK = SIZE_MAX - 1
 
 NP_DTYPE = {SHORT: np.int16, INT: np.int32, LONG: np.int64, LONGLONG: np.int64,
             FLOAT: np.float32, DOUBLE: np.float64, BF16: np.uint16, UINT: np.uint32,
-            ULONG: np.uint64, ULONGLONG: np.uint64}
+            ULONG: np.uint64, ULONGLONG: np.uint64, CHAR: np.int8, SCHAR: np.int8,
+            UCHAR: np.uint8, USHORT: np.uint16}
 
 _vp, _sz, _i, _u32, _u64, _d = C.c_void_p, C.c_size_t, C.c_int, C.c_uint32, C.c_uint64, C.c_double
 

@@ -553,6 +553,20 @@ int rocshmem_amd_broadcastmem(rocshmem_amd_team_t team, void *dest, const void *
                               size_t nbytes, int pe_root, rocshmem_amd_stream_t stream) {
   return grid_move_common<MOVE_BROADCAST>(team, dest, source, nbytes, pe_root, as_stream(stream));
 }
+int rocshmem_amd_broadcast_active_set(void *dest, const void *source, size_t nbytes, int pe_root,
+                                      int PE_start, int logPE_stride, int PE_size,
+                                      rocshmem_amd_stream_t stream) {
+  auto &r = runtime::rt();
+  if (!r.live || PE_start < 0 || logPE_stride < 0 || logPE_stride > 30 || PE_size < 1) return -1;
+  const int stride = 1 << logPE_stride;
+  if (PE_start + static_cast<long>(stride) * (PE_size - 1) >= r.npes) return -1;
+  if (pe_root < 0 || pe_root >= PE_size) return -1;
+  if (!sym_ok_on(dest, nbytes, PE_start) || !sym_ok_on(source, nbytes, PE_start)) return -1;
+  launch_grid_move<MOVE_BROADCAST>(static_cast<char *>(dest), static_cast<const char *>(source),
+                                   static_cast<int64_t>(stride) * r.pe_stride, PE_size, pe_root,
+                                   nbytes, as_stream(stream));
+  return 0;
+}
 int rocshmem_amd_fcollectmem(rocshmem_amd_team_t team, void *dest, const void *source,
                              size_t nbytes, rocshmem_amd_stream_t stream) {
   return grid_move_common<MOVE_FCOLLECT>(team, dest, source, nbytes, 0, as_stream(stream));

@@ -7,7 +7,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "librocshmem_amd.so")
 
 # Enumerations of include/rocshmem_amd.h.
-SHORT, INT, LONG, LONGLONG, FLOAT, DOUBLE, BF16, UINT, ULONG, ULONGLONG = range(10)
+(SHORT, INT, LONG, LONGLONG, FLOAT, DOUBLE, BF16, UINT, ULONG, ULONGLONG, CHAR, SCHAR, UCHAR,
+ USHORT) = range(14)
 SUM, MAX, MIN, PROD, AND, OR, XOR = range(7)
 THREAD, WAVE, WG = range(3)
 PUT, GET = range(2)
@@ -66,6 +67,14 @@ SIGNATURES = {
     "rocshmem_amd_timer_elapsed_ms": (C.c_float, [_vp]),
     "rocshmem_amd_timer_destroy": (_i, [_vp]),
     "rocshmem_amd_rma": (_i, [_i, _i, _vp, _vp, _sz, _sz, _i, _i, _i, _i, _i, _vp]),
+    "rocshmem_amd_ctx_pe": (_i, [_vp]),
+    "rocshmem_amd_host_putmem": (_i, [_vp, _vp, _sz, _i, _i]),
+    "rocshmem_amd_host_getmem": (_i, [_vp, _vp, _sz, _i, _i]),
+    "rocshmem_amd_host_amo": (_i, [_i, _i, _vp, _vp, _vp, _i, _i, _vp]),
+    "rocshmem_amd_host_peek": (_i, [_vp, _vp, _sz]),
+    "rocshmem_amd_host_wait_test": (_i, [_i, _i, _vp, _sz, _vp, _i, _vp, C.c_long,
+                                         C.POINTER(_sz), _vp]),
+    "rocshmem_amd_broadcast_active_set": (_i, [_vp, _vp, _sz, _i, _i, _i, _i, _vp]),
     "rocshmem_amd_put_flag_check": (_i, [_vp, _vp, _sz, _i, _i, _i, _i, _i, _i,
                                          C.POINTER(_u64), C.POINTER(_i), _vp]),
     "rocshmem_amd_putmem": (_i, [_vp, _vp, _sz, _i, _i, _vp]),
