@@ -14,8 +14,10 @@
 //
 // Which PE the host acts as: the PE of the context passed in (contexts made
 // by rocshmem_ctx_create belong to the PE that was acting then); calls
-// without a context act as the current acting PE (rocshmem_emu_set_pe).  A
-// collective is ONE call for the whole team, not one per member.
+// without a context act as the current acting PE (rocshmem_emu_set_pe), or,
+// in a PE thread (rocshmem_emu_run_pes), as that thread's PE.  Outside PE
+// threads a collective is ONE call for the whole team, not one per member; PE
+// threads call it once each, as the processes of the reference do.
 #ifndef ROCSHMEM_AMD_HOST_HPP_
 #define ROCSHMEM_AMD_HOST_HPP_
 
@@ -48,9 +50,23 @@ inline void host_require(int rc, const char *what) {
 
 // Host collectives return when the data is in place (the reference's
 // MPI_Bcast / MPI_Allreduce block): launch, then wait for the null stream.
-inline void host_collective(int rc, const char *what) {
+// The callers are the PEs start, start + stride, ... (size of them, world
+// numbering).  Outside PE threads there is one caller and it does the work;
+// in PE threads (rocshmem_emu_run_pes) every member calls and the last one to
+// arrive does the work for all while the others wait.
+template <typename Launch>
+inline void host_collective(int start, int stride, int size, Launch &&launch, const char *what) {
+  if (!rocshmem_amd_pe_threads_enter(start, stride, size)) return;
+  int rc = launch();
+  if (rc == 0) rc = rocshmem_amd_stream_sync(nullptr);
+  rocshmem_amd_pe_threads_leave(start, stride, size);
   host_require(rc, what);
-  host_require(rocshmem_amd_stream_sync(nullptr), what);
+}
+template <typename Launch>
+inline void host_team_collective(rocshmem_team_t team, Launch &&launch, const char *what) {
+  int start = 0, stride = 1, size = 1;
+  host_require(rocshmem_amd_team_active_set(team, &start, &stride, &size), what);
+  host_collective(start, stride, size, launch, what);
 }
 
 inline int host_pe_of(rocshmem_ctx_t ctx) { return rocshmem_amd_ctx_pe(ctx.ctx_opaque); }
@@ -219,8 +235,9 @@ template <typename T>
 inline T host_amo(int amo_op, rocshmem_ctx_t ctx, T *dest, T value, T cond, int pe,
                   const char *what) {
   T out = T();
-  host_require(rocshmem_amd_host_amo(amo_op, host_dtype<T>(), dest, &value, &cond,
-                                     host_pe_of(ctx), pe, &out),
+  const int me = host_pe_of(ctx);
+  host_require(rocshmem_amd_host_amo(amo_op, host_dtype<T>(), rocshmem_amd_pe_ptr(dest, me), &value,
+                                     &cond, me, pe, &out),
                what);
   return out;
 }
@@ -245,9 +262,13 @@ constexpr rocshmem_ctx_t ROCSHMEM_AMD_HOST_DEFAULT_CTX{nullptr, nullptr};
 // complete on return as well (permitted: they may complete at any time up to
 // the next quiet).
 // ---------------------------------------------------------------------------
+// The symmetric side may be given as any PE's address of the object; it is
+// taken as the calling PE's.
 __host__ inline void rocshmem_ctx_putmem(rocshmem_ctx_t ctx, void *dest, const void *source,
                                          size_t nelems, int pe) {
-  detail::host_require(rocshmem_amd_host_putmem(dest, source, nelems, detail::host_pe_of(ctx), pe),
+  const int me = detail::host_pe_of(ctx);
+  detail::host_require(rocshmem_amd_host_putmem(nelems ? rocshmem_amd_pe_ptr(dest, me) : dest,
+                                                source, nelems, me, pe),
                        "putmem");
 }
 __host__ inline void rocshmem_putmem(void *dest, const void *source, size_t nelems, int pe) {
@@ -255,8 +276,11 @@ __host__ inline void rocshmem_putmem(void *dest, const void *source, size_t nele
 }
 __host__ inline void rocshmem_ctx_getmem(rocshmem_ctx_t ctx, void *dest, const void *source,
                                          size_t nelems, int pe) {
-  detail::host_require(rocshmem_amd_host_getmem(dest, source, nelems, detail::host_pe_of(ctx), pe),
-                       "getmem");
+  const int me = detail::host_pe_of(ctx);
+  detail::host_require(
+      rocshmem_amd_host_getmem(dest, nelems ? rocshmem_amd_pe_ptr(source, me) : source, nelems, me,
+                               pe),
+      "getmem");
 }
 __host__ inline void rocshmem_getmem(void *dest, const void *source, size_t nelems, int pe) {
   rocshmem_ctx_getmem(ROCSHMEM_AMD_HOST_DEFAULT_CTX, dest, source, nelems, pe);
@@ -470,21 +494,28 @@ ROCSHMEM_AMD_WAIT_TYPES(ROCSHMEM_AMD_HOST_WAIT)
                                                      int nelems, int pe_root, int pe_start,       \
                                                      int log_pe_stride, int pe_size, long *) {    \
     detail::host_collective(                                                                      \
-        nelems < 0 ? -1                                                                           \
-                   : rocshmem_amd_broadcast_active_set(dest, source,                              \
-                                                       static_cast<size_t>(nelems) * sizeof(T),   \
-                                                       pe_root, pe_start, log_pe_stride, pe_size, \
-                                                       nullptr),                                  \
+        pe_start, 1 << log_pe_stride, pe_size,                                                    \
+        [&] {                                                                                     \
+          return nelems < 0 ? -1                                                                  \
+                            : rocshmem_amd_broadcast_active_set(                                  \
+                                  rocshmem_amd_pe_ptr(dest, pe_start),                            \
+                                  rocshmem_amd_pe_ptr(source, pe_start),                          \
+                                  static_cast<size_t>(nelems) * sizeof(T), pe_root, pe_start,     \
+                                  log_pe_stride, pe_size, nullptr);                               \
+        },                                                                                        \
         "broadcast");                                                                             \
   }                                                                                               \
   __host__ inline void rocshmem_ctx_##TN##_broadcast(rocshmem_ctx_t, rocshmem_team_t team,        \
                                                      T *dest, const T *source, int nelems,        \
                                                      int pe_root) {                               \
-    detail::host_collective(                                                                      \
-        nelems < 0 ? -1                                                                           \
-                   : rocshmem_amd_broadcastmem(team, dest, source,                                \
-                                               static_cast<size_t>(nelems) * sizeof(T), pe_root,  \
-                                               nullptr),                                          \
+    detail::host_team_collective(                                                                 \
+        team,                                                                                     \
+        [&] {                                                                                     \
+          return nelems < 0 ? -1                                                                  \
+                            : rocshmem_amd_broadcastmem(team, dest, source,                       \
+                                                        static_cast<size_t>(nelems) * sizeof(T),  \
+                                                        pe_root, nullptr);                        \
+        },                                                                                        \
         "broadcast");                                                                             \
   }
 ROCSHMEM_AMD_COLL_TYPES(ROCSHMEM_AMD_HOST_BROADCAST)
@@ -493,36 +524,47 @@ ROCSHMEM_AMD_COLL_TYPES(ROCSHMEM_AMD_HOST_BROADCAST)
 // The active-set form rocshmem_ctx_<T>_<op>_to_all is defined by the reference
 // library (src/rocshmem.cpp:974-980) and used by its tests
 // (tests/sos_tests/to_all.cpp) although its public headers do not declare it.
+// The team form under the to_all name is what two more of its tests call
+// (tests/sos_tests/shmem_team_reduce.cpp:128) though the library has no such
+// overload; it is the same as _reduce.
 #define ROCSHMEM_AMD_HOST_REDUCE1(T, TN, OPN, OPCODE)                                             \
   __host__ inline void rocshmem_ctx_##TN##_##OPN##_to_all(rocshmem_ctx_t, T *dest,                \
                                                           const T *source, int nreduce,           \
                                                           int PE_start, int logPE_stride,         \
                                                           int PE_size, T *, long *) {             \
-    detail::host_collective(rocshmem_amd_to_all(detail::host_dtype<T>(), OPCODE, dest, source,    \
-                                             nreduce, PE_start, logPE_stride, PE_size, nullptr),  \
-                         #OPN "_to_all");                                                         \
+    detail::host_collective(                                                                      \
+        PE_start, 1 << logPE_stride, PE_size,                                                     \
+        [&] {                                                                                     \
+          return rocshmem_amd_to_all(detail::host_dtype<T>(), OPCODE,                             \
+                                     rocshmem_amd_pe_ptr(dest, PE_start),                         \
+                                     rocshmem_amd_pe_ptr(source, PE_start), nreduce, PE_start,    \
+                                     logPE_stride, PE_size, nullptr);                             \
+        },                                                                                        \
+        #OPN "_to_all");                                                                          \
   }                                                                                               \
   __host__ inline int rocshmem_ctx_##TN##_##OPN##_reduce(rocshmem_ctx_t, rocshmem_team_t team,    \
                                                          T *dest, const T *source, int nreduce) { \
-    detail::host_collective(rocshmem_amd_reduce(detail::host_dtype<T>(), OPCODE, team, dest,      \
-                                                source, nreduce, nullptr),                        \
-                            #OPN "_reduce");                                                      \
+    detail::host_team_collective(                                                                 \
+        team,                                                                                     \
+        [&] {                                                                                     \
+          return rocshmem_amd_reduce(detail::host_dtype<T>(), OPCODE, team, dest, source,         \
+                                     nreduce, nullptr);                                           \
+        },                                                                                        \
+        #OPN "_reduce");                                                                          \
     return ROCSHMEM_SUCCESS;                                                                      \
   }                                                                                               \
-  /* Team form under the to_all name, which two of the reference's tests call                     \
-     (tests/sos_tests/shmem_team_reduce.cpp:128) though the library has no such overload. */      \
   __host__ inline int rocshmem_ctx_##TN##_##OPN##_to_all(rocshmem_ctx_t ctx, rocshmem_team_t team, \
                                                          T *dest, const T *source, int nreduce) { \
     return rocshmem_ctx_##TN##_##OPN##_reduce(ctx, team, dest, source, nreduce);                  \
   }
-#define ROCSHMEM_AMD_HOST_REDUCE_ARITH(T, TN)                                                     \
-  ROCSHMEM_AMD_HOST_REDUCE1(T, TN, sum, ROCSHMEM_AMD_SUM)                                         \
-  ROCSHMEM_AMD_HOST_REDUCE1(T, TN, min, ROCSHMEM_AMD_MIN)                                         \
-  ROCSHMEM_AMD_HOST_REDUCE1(T, TN, max, ROCSHMEM_AMD_MAX)                                         \
+#define ROCSHMEM_AMD_HOST_REDUCE_ARITH(T, TN)                   \
+  ROCSHMEM_AMD_HOST_REDUCE1(T, TN, sum, ROCSHMEM_AMD_SUM)       \
+  ROCSHMEM_AMD_HOST_REDUCE1(T, TN, min, ROCSHMEM_AMD_MIN)       \
+  ROCSHMEM_AMD_HOST_REDUCE1(T, TN, max, ROCSHMEM_AMD_MAX)       \
   ROCSHMEM_AMD_HOST_REDUCE1(T, TN, prod, ROCSHMEM_AMD_PROD)
-#define ROCSHMEM_AMD_HOST_REDUCE_BITWISE(T, TN)                                                   \
-  ROCSHMEM_AMD_HOST_REDUCE1(T, TN, or, ROCSHMEM_AMD_OR)                                           \
-  ROCSHMEM_AMD_HOST_REDUCE1(T, TN, and, ROCSHMEM_AMD_AND)                                         \
+#define ROCSHMEM_AMD_HOST_REDUCE_BITWISE(T, TN)                 \
+  ROCSHMEM_AMD_HOST_REDUCE1(T, TN, or, ROCSHMEM_AMD_OR)         \
+  ROCSHMEM_AMD_HOST_REDUCE1(T, TN, and, ROCSHMEM_AMD_AND)       \
   ROCSHMEM_AMD_HOST_REDUCE1(T, TN, xor, ROCSHMEM_AMD_XOR)
 ROCSHMEM_AMD_INT_REDUCE_TYPES(ROCSHMEM_AMD_HOST_REDUCE_ARITH)
 ROCSHMEM_AMD_INT_REDUCE_TYPES(ROCSHMEM_AMD_HOST_REDUCE_BITWISE)

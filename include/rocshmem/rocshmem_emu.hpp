@@ -8,6 +8,16 @@
 //     rocshmem_my_pe(), rocshmem_malloc() and team handles are reported for
 //     that PE.  rocshmem_malloc() allocates the object on every PE at once
 //     and returns the acting PE's address.
+//   * Or every PE gets a host thread of its own: rocshmem_emu_run_pes(P, fn,
+//     argc, argv) runs fn once per PE, each in its own thread, and inside them
+//     the host API behaves as it does in the reference's one-process-per-PE
+//     programs: rocshmem_my_pe() is the thread's PE, rocshmem_init / malloc /
+//     free / barrier_all / team_split_strided / broadcast / reduce are
+//     collective calls that every member makes.  A program written for the
+//     reference runs that way unchanged when it is compiled with
+//     -DROCSHMEM_EMU_PE_THREADS_MAIN: its main() becomes the per-PE function
+//     (single translation unit; P from ROCSHMEM_EMU_NPES).  File-scope
+//     variables of such a program are shared by all PEs.
 //   * A work-group learns its PE from its context.  Contexts made by
 //     rocshmem_wg_team_create_ctx take the PE of the team object; the default
 //     context and rocshmem_wg_ctx_create use the rule chosen with
@@ -28,6 +38,9 @@ enum rocshmem_emu_pe_rule {
   ROCSHMEM_EMU_PE_BLOCK_Z = 3
 };
 
+// Runs pe_main(argc, argv) in npes threads (npes <= 0: ROCSHMEM_EMU_NPES), one
+// per PE, before the runtime is up; returns the first non-zero result.
+int rocshmem_emu_run_pes(int npes, int (*pe_main)(int, char **), int argc, char **argv);
 void rocshmem_emu_set_npes(int npes);
 void rocshmem_emu_set_pe(int pe);
 void rocshmem_emu_set_pe_rule(int rule);
@@ -40,5 +53,27 @@ rocshmem_team_t rocshmem_emu_team_on(rocshmem_team_t team, int pe);
 size_t rocshmem_emu_pe_stride();
 
 }  // namespace rocshmem
+
+#if defined(ROCSHMEM_EMU_PE_THREADS_MAIN)
+// The program's own main, under another name, in whichever of the usual
+// forms it was written.
+int rocshmem_emu_pe_main(int argc, char **argv, char **envp) __attribute__((weak));
+int rocshmem_emu_pe_main(int argc, char **argv) __attribute__((weak));
+int rocshmem_emu_pe_main() __attribute__((weak));
+extern char **environ;
+int main(int argc, char **argv) {
+  return rocshmem::rocshmem_emu_run_pes(
+      0,
+      [](int c, char **v) -> int {
+        int (*with_env)(int, char **, char **) = rocshmem_emu_pe_main;
+        int (*with_args)(int, char **) = rocshmem_emu_pe_main;
+        int (*without_args)() = rocshmem_emu_pe_main;
+        if (with_env) return with_env(c, v, environ);
+        return with_args ? with_args(c, v) : without_args();
+      },
+      argc, argv);
+}
+#define main rocshmem_emu_pe_main
+#endif
 
 #endif  // ROCSHMEM_AMD_EMU_HPP_

@@ -165,6 +165,19 @@ int rocshmem_amd_team_translate_pe(rocshmem_amd_team_t src_team, int src_pe,
 /* The same team as seen by another PE (NULL if that PE is not a member). */
 rocshmem_amd_team_t rocshmem_amd_team_on(rocshmem_amd_team_t team, int pe);
 
+/* World PEs of a team: PE_start, PE_start + PE_stride, ... (PE_size of them). */
+int rocshmem_amd_team_active_set(rocshmem_amd_team_t team, int *PE_start, int *PE_stride,
+                                 int *PE_size);
+/* Meeting point of the host collectives when every PE is a thread of this
+ * process (rocshmem_emu_run_pes, include/rocshmem/rocshmem_emu.hpp; the
+ * reference's PEs are processes that meet inside MPI).  Each member of the
+ * strided set calls enter: it returns 1 in the last one to arrive, which then
+ * performs the operation for the whole set and calls leave; in the others it
+ * returns 0 once that has happened.  Outside PE threads enter returns 1 at
+ * once and leave does nothing. */
+int rocshmem_amd_pe_threads_enter(int PE_start, int PE_stride, int PE_size);
+void rocshmem_amd_pe_threads_leave(int PE_start, int PE_stride, int PE_size);
+
 /* Plain device memory and staging for callers without a HIP binding. */
 void *rocshmem_amd_dev_alloc(size_t size);
 int rocshmem_amd_dev_free(void *ptr);

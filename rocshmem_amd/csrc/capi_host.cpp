@@ -37,6 +37,23 @@ int64_t rocshmem_amd_set_ctx_options(int64_t options) {
   rt().driver_ctx_options = options;
   return before;
 }
+int rocshmem_amd_pe_threads_enter(int PE_start, int PE_stride, int PE_size) {
+  return rocshmem::runtime::pe_threads_enter(PE_start, PE_stride, PE_size, nullptr) ? 1 : 0;
+}
+void rocshmem_amd_pe_threads_leave(int PE_start, int PE_stride, int PE_size) {
+  rocshmem::runtime::pe_threads_leave(PE_start, PE_stride, PE_size, 0);
+}
+int rocshmem_amd_team_active_set(rocshmem_amd_team_t team, int *PE_start, int *PE_stride,
+                                 int *PE_size) {
+  if (!rt().live || !PE_start || !PE_stride || !PE_size) return -1;
+  const rocshmem::detail::Team *t =
+      rt().host_team(rt().my_view(static_cast<rocshmem::rocshmem_team_t>(team)));
+  if (!t) return -1;
+  *PE_start = t->wrt_world.pe_start;
+  *PE_stride = t->wrt_world.stride;
+  *PE_size = t->wrt_world.size;
+  return 0;
+}
 void *rocshmem_amd_malloc(size_t size) { return rt().sym_malloc(size); }
 int rocshmem_amd_free(void *ptr) {
   rt().sym_free(ptr);

@@ -276,7 +276,7 @@ struct TeamView {
 };
 inline bool view_team(rocshmem_amd_team_t team, TeamView *v) {
   auto &r = runtime::rt();
-  v->host = r.host_team(static_cast<rocshmem_team_t>(team));
+  v->host = r.host_team(r.my_view(static_cast<rocshmem_team_t>(team)));
   if (!v->host || v->host->my_pe < 0) return false;
   v->row = r.d_teams + static_cast<size_t>(v->host->pool_index) * r.npes;
   return true;
@@ -285,7 +285,7 @@ inline bool view_team(rocshmem_amd_team_t team, TeamView *v) {
 inline char *on_pe0(const void *p) {
   auto &r = runtime::rt();
   return const_cast<char *>(static_cast<const char *>(p)) -
-         static_cast<size_t>(r.acting_pe) * r.pe_stride;
+         static_cast<size_t>(r.me()) * r.pe_stride;
 }
 inline bool in_heap(const void *p) {
   return runtime::rt().offset_of(p) != runtime::Pow2Allocator::kNoBlock;
@@ -393,7 +393,7 @@ int wg_move_common(int elem_size, rocshmem_amd_team_t team, void *dest, const vo
   {
     const size_t blk = static_cast<size_t>(nelems) * elem_size;
     const size_t all = blk * v.host->num_pes;
-    const int me = runtime::rt().acting_pe;
+    const int me = runtime::rt().me();
     if (!sym_ok_on(dest, kMove == MOVE_BROADCAST ? blk : all, me)) return -1;
     if (!sym_ok_on(source, kMove == MOVE_ALLTOALL ? all : blk, me)) return -1;
   }
@@ -418,7 +418,7 @@ int grid_move_common(rocshmem_amd_team_t team, void *dest, const void *source, s
   if (!view_team(team, &v)) return -1;
   {
     const size_t all = nbytes * v.host->num_pes;
-    const int me = runtime::rt().acting_pe;
+    const int me = runtime::rt().me();
     if (!sym_ok_on(dest, kMove == MOVE_BROADCAST ? nbytes : all, me)) return -1;
     if (!sym_ok_on(source, kMove == MOVE_ALLTOALL ? all : nbytes, me)) return -1;
   }
@@ -442,7 +442,7 @@ int rocshmem_amd_wg_reduce(int dtype, int op, rocshmem_amd_team_t team, void *de
   if (!view_team(team, &v) || !valid_launch(1, wg_size) || nreduce < 0) return -1;
   {
     const size_t bytes = static_cast<size_t>(nreduce) * dtype_size(dtype);
-    const int me = runtime::rt().acting_pe;
+    const int me = runtime::rt().me();
     if (!sym_ok_on(dest, bytes, me) || !sym_ok_on(source, bytes, me)) return -1;
   }
   int *d_status;
@@ -486,13 +486,13 @@ int rocshmem_amd_wg_fcollect(int elem_size, rocshmem_amd_team_t team, void *dest
 int rocshmem_amd_wg_sync(int sync_fn, rocshmem_amd_team_t team, uint64_t *scratch, int rounds,
                          int wg_size, rocshmem_amd_stream_t stream) {
   auto &r = runtime::rt();
-  if (!r.live || rounds < 0 || !valid_launch(1, wg_size) || !sym_ok_on(scratch, 8, r.acting_pe)) return -1;
+  if (!r.live || rounds < 0 || !valid_launch(1, wg_size) || !sym_ok_on(scratch, 8, r.me())) return -1;
   if (sync_fn < ROCSHMEM_AMD_BARRIER_ALL || sync_fn > ROCSHMEM_AMD_TEAM_SYNC) return -1;
   TeamView v;
   if (sync_fn == ROCSHMEM_AMD_TEAM_SYNC) {
     if (!view_team(team, &v)) return -1;
   } else {
-    if (!view_team(r.team_handle(0, r.acting_pe), &v)) return -1;
+    if (!view_team(r.team_handle(0, r.me()), &v)) return -1;
   }
   int *d_err;
   DRV_CHECK_HIP(hipMalloc(&d_err, sizeof(int)));
@@ -538,7 +538,7 @@ int rocshmem_amd_reduce(int dtype, int op, rocshmem_amd_team_t team, void *dest,
   if (!view_team(team, &v) || nreduce < 0) return -1;
   auto &r = runtime::rt();
   const size_t bytes = static_cast<size_t>(nreduce) * dtype_size(dtype);
-  if (!sym_ok_on(dest, bytes, r.acting_pe) || !sym_ok_on(source, bytes, r.acting_pe)) return -1;
+  if (!sym_ok_on(dest, bytes, r.me()) || !sym_ok_on(source, bytes, r.me())) return -1;
   const int64_t first = static_cast<int64_t>(v.host->wrt_world.pe_start) * r.pe_stride;
   const int64_t hop = static_cast<int64_t>(v.host->wrt_world.stride) * r.pe_stride;
   return grid_reduce_common(dtype, op, on_pe0(dest) + first, on_pe0(source) + first, hop,

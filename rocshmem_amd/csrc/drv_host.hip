@@ -99,7 +99,7 @@ extern "C" {
 int rocshmem_amd_ctx_pe(const void *ctx_opaque) {
   auto &r = runtime::rt();
   if (!r.live) return -1;
-  if (!ctx_opaque) return r.acting_pe;
+  if (!ctx_opaque) return r.me();
   const auto *c = static_cast<const detail::Context *>(ctx_opaque);
   if (c >= r.d_default_ctx && c < r.d_default_ctx + 2 * r.npes)
     return static_cast<int>((c - r.d_default_ctx) % r.npes);

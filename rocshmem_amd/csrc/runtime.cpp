@@ -10,10 +10,13 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <condition_variable>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <map>
 #include <mutex>
+#include <thread>
 #include <vector>
 
 #include "rocshmem/rocshmem.hpp"
@@ -23,6 +26,8 @@ namespace rocshmem {
 rocshmem_team_t ROCSHMEM_TEAM_WORLD = ROCSHMEM_TEAM_INVALID;
 
 namespace runtime {
+
+thread_local int tl_pe = -1;
 
 #define RT_CHECK_HIP(expr)                                                        \
   do {                                                                            \
@@ -64,6 +69,53 @@ int ilog2(int x) {
 }  // namespace
 
 Runtime &rt() { return g_rt; }
+
+// ---- one thread per PE -------------------------------------------------------
+namespace {
+struct MeetingPoint {
+  std::mutex m;
+  std::condition_variable cv;
+  int arrived = 0;
+  uint64_t round = 0;
+  uint64_t result = 0;
+};
+struct PeThreads {
+  int npes = 0;
+  std::mutex m;
+  std::map<uint64_t, MeetingPoint> points;  // node-based: references stay valid
+  MeetingPoint &at(int start, int stride, int size) {
+    const uint64_t key = (static_cast<uint64_t>(start) << 42) |
+                         (static_cast<uint64_t>(stride) << 21) | static_cast<uint64_t>(size);
+    std::lock_guard<std::mutex> g(m);
+    return points[key];
+  }
+};
+PeThreads g_threads;
+}  // namespace
+
+int pe_threads_count() { return g_threads.npes; }
+void pe_threads_start(int npes) { g_threads.npes = npes; }
+
+bool pe_threads_enter(int start, int stride, int size, uint64_t *result) {
+  if (tl_pe < 0 || g_threads.npes == 0 || size <= 1) return true;
+  MeetingPoint &p = g_threads.at(start, stride, size);
+  std::unique_lock<std::mutex> lk(p.m);
+  if (++p.arrived == size) return true;  // the last to arrive does the work (lock released here)
+  const uint64_t round = p.round;
+  p.cv.wait(lk, [&] { return p.round != round; });
+  if (result) *result = p.result;
+  return false;
+}
+
+void pe_threads_leave(int start, int stride, int size, uint64_t result) {
+  if (tl_pe < 0 || g_threads.npes == 0 || size <= 1) return;
+  MeetingPoint &p = g_threads.at(start, stride, size);
+  std::lock_guard<std::mutex> lk(p.m);
+  p.arrived = 0;
+  p.result = result;
+  ++p.round;
+  p.cv.notify_all();
+}
 
 void Runtime::push_state() {
   for (auto fn : uploaders()) fn(&state);
@@ -272,7 +324,7 @@ void *Runtime::sym_malloc(size_t size) {
   require_live("rocshmem_malloc");
   const uint64_t off = allocator.alloc(size);
   if (off == Pow2Allocator::kNoBlock) return nullptr;
-  return heap_base + static_cast<size_t>(acting_pe) * pe_stride + off;
+  return heap_base + static_cast<size_t>(me()) * pe_stride + off;
 }
 
 void Runtime::sym_free(void *ptr) {
@@ -341,8 +393,8 @@ int Runtime::team_split_strided(rocshmem_team_t parent, int start, int stride, i
     write_team(slot, pe, world, wrt_parent, mine);
   }
   RT_CHECK_HIP(hipDeviceSynchronize());
-  if (h_teams[static_cast<size_t>(slot) * npes + acting_pe].my_pe >= 0)
-    *new_team = team_handle(slot, acting_pe);
+  if (h_teams[static_cast<size_t>(slot) * npes + me()].my_pe >= 0)
+    *new_team = team_handle(slot, me());
   last_created_slot = slot;
   return 0;
 }
@@ -400,27 +452,73 @@ void register_state_uploader(StateUploader fn) {
 // ============================ public host API ===============================
 using runtime::rt;
 
-__host__ void rocshmem_init(MPI_Comm) { rt().init(0, 0); }
-__host__ void rocshmem_init_thread(int, int *provided, MPI_Comm) {
-  rt().init(0, 0);
+// In PE threads every thread calls the collective host functions; the last
+// caller of each does the work for all (pe_threads_enter / _leave).
+namespace {
+struct WorldMeeting {
+  uint64_t result = 0;
+  bool mine;
+  WorldMeeting() : mine(runtime::pe_threads_enter(0, 1, runtime::pe_threads_count(), &result)) {}
+  void done(uint64_t r = 0) {
+    result = r;
+    runtime::pe_threads_leave(0, 1, runtime::pe_threads_count(), r);
+  }
+};
+}  // namespace
+
+__host__ void rocshmem_init(MPI_Comm) {
+  WorldMeeting w;
+  if (w.mine) {
+    rt().init(runtime::pe_threads_count(), 0);
+    w.done();
+  }
+}
+__host__ void rocshmem_init_thread(int, int *provided, MPI_Comm comm) {
+  rocshmem_init(comm);
   rocshmem_query_thread(provided);
 }
 __host__ void rocshmem_query_thread(int *provided) { *provided = ROCSHMEM_THREAD_MULTIPLE; }
 __host__ void rocshmem_dump_stats() {}
 __host__ void rocshmem_reset_stats() {}
-__host__ void rocshmem_finalize() { rt().finalize(); }
-__host__ void *rocshmem_malloc(size_t size) { return rt().sym_malloc(size); }
-__host__ void rocshmem_free(void *ptr) { rt().sym_free(ptr); }
+__host__ void rocshmem_finalize() {
+  WorldMeeting w;
+  if (w.mine) {
+    rt().finalize();
+    w.done();
+  }
+}
+// Collective (include/rocshmem/rocshmem.hpp:115-123): one allocation serves
+// every PE; each caller gets the address in its own slice.
+__host__ void *rocshmem_malloc(size_t size) {
+  WorldMeeting w;
+  if (w.mine) {
+    void *mine = rt().sym_malloc(size);
+    w.done(mine ? rt().offset_of(mine) + 1 : 0);
+  }
+  if (!w.result) return nullptr;
+  return rt().heap_base + static_cast<size_t>(rt().me()) * rt().pe_stride + (w.result - 1);
+}
+__host__ void rocshmem_free(void *ptr) {
+  WorldMeeting w;
+  if (w.mine) {
+    rt().sym_free(ptr);
+    w.done();
+  }
+}
 // Usable before rocshmem_init, as in the reference (src/rocshmem.cpp:113-121).
 __host__ int rocshmem_n_pes() {
   if (rt().live) return rt().npes;
+  if (runtime::pe_threads_count() > 0) return runtime::pe_threads_count();
   if (runtime::g_requested_npes > 0) return runtime::g_requested_npes;
   return static_cast<int>(runtime::env_size("ROCSHMEM_EMU_NPES", 1));
 }
-__host__ int rocshmem_my_pe() { return rt().live ? rt().acting_pe : 0; }
+__host__ int rocshmem_my_pe() {
+  if (runtime::tl_pe >= 0) return runtime::tl_pe;
+  return rt().live ? rt().acting_pe : 0;
+}
 __host__ int rocshmem_ctx_create(int64_t options, rocshmem_ctx_t *ctx) {
   rt().require_live("rocshmem_ctx_create");
-  *ctx = rt().ctx_handle(rt().acting_pe, options);
+  *ctx = rt().ctx_handle(rt().me(), options);
   return 0;
 }
 __host__ void rocshmem_ctx_destroy(rocshmem_ctx_t) {}
@@ -428,8 +526,8 @@ __host__ void rocshmem_ctx_destroy(rocshmem_ctx_t) {}
 // src/team.cpp:51-111
 __host__ int rocshmem_team_translate_pe(rocshmem_team_t src_team, int src_pe,
                                         rocshmem_team_t dest_team) {
-  const detail::Team *s = rt().host_team(src_team);
-  const detail::Team *d = rt().host_team(dest_team);
+  const detail::Team *s = rt().host_team(rt().my_view(src_team));
+  const detail::Team *d = rt().host_team(rt().my_view(dest_team));
   if (!s || !d) return -1;
   const int world = s->wrt_world.pe_start + s->wrt_world.stride * src_pe;
   const int off = world - d->wrt_world.pe_start;
@@ -438,21 +536,48 @@ __host__ int rocshmem_team_translate_pe(rocshmem_team_t src_team, int src_pe,
   return rel >= d->num_pes ? -1 : rel;
 }
 __host__ int rocshmem_team_n_pes(rocshmem_team_t team) {
-  const detail::Team *t = rt().host_team(team);
+  const detail::Team *t = rt().host_team(rt().my_view(team));
   return t ? t->num_pes : -1;
 }
 __host__ int rocshmem_team_my_pe(rocshmem_team_t team) {
-  const detail::Team *t = rt().host_team(team);
+  const detail::Team *t = rt().host_team(rt().my_view(team));
   return t ? t->my_pe : -1;
 }
+// Collective over the parent team (src/rocshmem.cpp:221-303).  In PE threads
+// the last member to arrive creates the team objects of all PEs; every caller
+// then takes the handle of its own PE.
 __host__ int rocshmem_team_split_strided(rocshmem_team_t parent_team, int start, int stride,
                                          int size, const rocshmem_team_config_t *, long,
                                          rocshmem_team_t *new_team) {
-  return rt().team_split_strided(parent_team, start, stride, size, new_team);
+  parent_team = rt().my_view(parent_team);
+  const detail::Team *pt = rt().host_team(parent_team);
+  if (!pt || runtime::tl_pe < 0)
+    return rt().team_split_strided(parent_team, start, stride, size, new_team);
+  const detail::TeamInfo w = pt->wrt_world;
+  uint64_t packed = 0;  // (return code + 1) << 32 | (slot + 1)
+  if (runtime::pe_threads_enter(w.pe_start, w.stride, w.size, &packed)) {
+    rocshmem_team_t unused;
+    const int rc = rt().team_split_strided(parent_team, start, stride, size, &unused);
+    packed = (static_cast<uint64_t>(rc + 1) << 32) |
+             static_cast<uint64_t>(rc == 0 ? rt().last_created_slot + 1 : 0);
+    runtime::pe_threads_leave(w.pe_start, w.stride, w.size, packed);
+  }
+  const int rc = static_cast<int>(packed >> 32) - 1;
+  const int slot = static_cast<int>(packed & 0xffffffffu) - 1;
+  *new_team = ROCSHMEM_TEAM_INVALID;
+  if (rc == 0 && slot >= 0) *new_team = rt().team_on(rt().team_handle(slot, w.pe_start), rt().me());
+  return rc;
 }
 __host__ void rocshmem_team_destroy(rocshmem_team_t team) {
-  if (team == ROCSHMEM_TEAM_WORLD) return;
-  rt().team_destroy(team);
+  if (team == ROCSHMEM_TEAM_WORLD || team == ROCSHMEM_TEAM_INVALID) return;
+  team = rt().my_view(team);
+  const detail::Team *t = rt().host_team(team);
+  if (!t || t->pool_index == 0) return;
+  const detail::TeamInfo w = t->wrt_world;
+  if (runtime::pe_threads_enter(w.pe_start, w.stride, w.size, nullptr)) {
+    rt().team_destroy(team);
+    runtime::pe_threads_leave(w.pe_start, w.stride, w.size, 0);
+  }
 }
 // With every PE in this process, host-side ordering and barriers reduce to
 // draining the device.
@@ -460,9 +585,42 @@ __host__ void rocshmem_ctx_fence(rocshmem_ctx_t) { RT_CHECK_HIP(hipDeviceSynchro
 __host__ void rocshmem_fence() { RT_CHECK_HIP(hipDeviceSynchronize()); }
 __host__ void rocshmem_ctx_quiet(rocshmem_ctx_t) { RT_CHECK_HIP(hipDeviceSynchronize()); }
 __host__ void rocshmem_quiet() { RT_CHECK_HIP(hipDeviceSynchronize()); }
-__host__ void rocshmem_barrier_all() { RT_CHECK_HIP(hipDeviceSynchronize()); }
-__host__ void rocshmem_sync_all() { RT_CHECK_HIP(hipDeviceSynchronize()); }
-__host__ void rocshmem_global_exit(int status) { exit(status); }
+__host__ void rocshmem_barrier_all() {
+  WorldMeeting w;
+  if (w.mine) {
+    RT_CHECK_HIP(hipDeviceSynchronize());
+    w.done();
+  }
+}
+__host__ void rocshmem_sync_all() { rocshmem_barrier_all(); }
+// Ends the whole job at once, as the reference's MPI_Abort does
+// (src/rocshmem.cpp): other PE threads may be asleep inside a collective, so
+// no destructors run.
+__host__ void rocshmem_global_exit(int status) {
+  fflush(nullptr);
+  _Exit(status);
+}
+
+int rocshmem_emu_run_pes(int npes, int (*pe_main)(int, char **), int argc, char **argv) {
+  if (npes <= 0) npes = rocshmem_n_pes();
+  if (runtime::pe_threads_count() != 0 || rt().live) {
+    fprintf(stderr, "rocshmem: rocshmem_emu_run_pes needs a runtime that is not yet up\n");
+    abort();
+  }
+  runtime::pe_threads_start(npes);
+  std::vector<int> rc(npes, 0);
+  std::vector<std::thread> threads;
+  for (int pe = 0; pe < npes; ++pe)
+    threads.emplace_back([&rc, pe, pe_main, argc, argv] {
+      runtime::tl_pe = pe;
+      rc[pe] = pe_main(argc, argv);
+    });
+  for (auto &t : threads) t.join();
+  runtime::pe_threads_start(0);
+  for (int r : rc)
+    if (r) return r;
+  return 0;
+}
 
 void rocshmem_emu_set_npes(int npes) { runtime::g_requested_npes = npes; }
 void rocshmem_emu_set_pe(int pe) { rt().set_pe(pe); }

@@ -13,10 +13,16 @@
 namespace rocshmem {
 namespace runtime {
 
+// PE this thread runs as while rocshmem_emu_run_pes hosts one thread per PE;
+// -1 for every other thread.
+extern thread_local int tl_pe;
+
 struct Runtime {
   bool live = false;
   int npes = 0;
-  int acting_pe = 0;
+  int acting_pe = 0;  // PE the host acts as outside PE threads (rocshmem_emu_set_pe)
+  // PE the calling thread acts as.
+  int me() const { return tl_pe >= 0 ? tl_pe : acting_pe; }
   int max_ctxs = 0;
   int max_teams = 0;
   int num_user_teams = 0;
@@ -51,6 +57,12 @@ struct Runtime {
   void team_destroy(rocshmem_team_t team);
   rocshmem_team_t team_handle(int pool_index, int pe) const;
   rocshmem_team_t team_on(rocshmem_team_t team, int pe) const;
+  // The handle a PE thread should use for `team`: its own PE's view of it
+  // (ROCSHMEM_TEAM_WORLD is one global and names PE 0's view).  Unchanged
+  // outside PE threads.
+  rocshmem_team_t my_view(rocshmem_team_t team) const {
+    return tl_pe < 0 ? team : team_on(team, tl_pe);
+  }
   const detail::Team *host_team(rocshmem_team_t team) const;
 
   void set_pe(int pe);
@@ -85,6 +97,18 @@ struct Runtime {
 };
 
 Runtime &rt();
+
+// ---- one thread per PE (rocshmem_emu_run_pes) --------------------------------
+// Collective host calls made by PE threads meet here.  The callers are the
+// members of the strided set (start, stride, size) of world PEs.  enter()
+// returns true in exactly one of them, the last to arrive, which performs the
+// operation for the whole set and then calls leave(result); the others sleep
+// in enter() until then and return false with *result filled in.  Outside PE
+// threads enter() returns true at once and leave() does nothing.
+bool pe_threads_enter(int start, int stride, int size, uint64_t *result);
+void pe_threads_leave(int start, int stride, int size, uint64_t result);
+int pe_threads_count();  // P while PE threads run, else 0
+void pe_threads_start(int npes);
 
 }  // namespace runtime
 }  // namespace rocshmem

@@ -53,6 +53,9 @@ SIGNATURES = {
     "rocshmem_amd_team_my_pe": (_i, [_vp]),
     "rocshmem_amd_team_translate_pe": (_i, [_vp, _i, _vp]),
     "rocshmem_amd_team_on": (_vp, [_vp, _i]),
+    "rocshmem_amd_team_active_set": (_i, [_vp, C.POINTER(_i), C.POINTER(_i), C.POINTER(_i)]),
+    "rocshmem_amd_pe_threads_enter": (_i, [_i, _i, _i]),
+    "rocshmem_amd_pe_threads_leave": (None, [_i, _i, _i]),
     "rocshmem_amd_dev_alloc": (_vp, [_sz]),
     "rocshmem_amd_dev_free": (_i, [_vp]),
     "rocshmem_amd_copy_in": (_i, [_vp, _vp, _sz]),

@@ -17,6 +17,7 @@ P, HEAP = 8, 1 << 30
 GUARD = 64
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 SOS_DIR = os.path.join(ROOT, "oracle", "_ref", "sos")
+SOS_THREADS_DIR = os.path.join(ROOT, "oracle", "_ref", "sos_threads")
 
 NP = {"INT": np.int32, "LONG": np.int64, "LONGLONG": np.int64, "UINT": np.uint32,
       "ULONG": np.uint64, "ULONGLONG": np.uint64, "FLOAT": np.float32, "DOUBLE": np.float64,
@@ -350,3 +351,44 @@ def test_reference_host_programs_run_against_this_library(rt, name):
         assert r.returncode != 0, "now passes: drop it from the exceptions"
         return
     assert r.returncode == 0, (name, r.stdout[-800:], r.stderr[-800:])
+
+
+# Run with one thread per PE (rocshmem_emu_run_pes), all PEs share the
+# program's file-scope variables and only the PE threads themselves carry a PE
+# identity; programs that cannot live with that, or that race by construction,
+# are left out:
+SOS_NOT_AS_PE_THREADS = {
+    "to_all": "keeps its symmetric pointers in file-scope variables",
+    "micro_unit_shmem": "keeps its symmetric pointers in file-scope variables",
+    "bigput": "hands addresses of static variables to a reduction",
+    "put_ctx_mbw_mr": "needs exactly two processes and carries on after finalize otherwise",
+    "query_thread": "branches on a variable it never initialises",
+    "mt_a2a": "starts threads of its own inside each PE",
+    "threading": "starts threads of its own inside each PE",
+    "cxx_test_shmem_test": "zeroes its own word with no barrier before the neighbour's put to it",
+    "cxx_test_shmem_wait_until": "zeroes its own word with no barrier before the neighbour's put to it",
+    "shmem_test": "zeroes its own word with no barrier before the neighbour's put to it",
+    "sping": "zeroes its own word with no barrier before the neighbour's put to it",
+}
+
+
+def sos_thread_programs():
+    if not os.path.isdir(SOS_THREADS_DIR):
+        return []
+    return sorted(f for f in os.listdir(SOS_THREADS_DIR)
+                  if os.access(os.path.join(SOS_THREADS_DIR, f), os.X_OK) and f not in SOS_NOT_AS_PE_THREADS)
+
+
+@pytest.mark.skipif(not sos_thread_programs(), reason="oracle/_ref/sos_threads is built where the reference tree exists")
+@pytest.mark.parametrize("npes", [2, 8])
+@pytest.mark.parametrize("name", sos_thread_programs())
+def test_reference_host_programs_run_with_a_thread_per_pe(rt, name, npes):
+    """The same programs with their main() run once per PE, every PE a host
+    thread of one process (-DROCSHMEM_EMU_PE_THREADS_MAIN): puts, gets,
+    atomics, waits, barriers, team splits, broadcasts and reductions between 2
+    and 8 PEs, checked by the programs themselves."""
+    rt.down()
+    env = dict(os.environ, ROCSHMEM_EMU_NPES=str(npes), ROCSHMEM_HEAP_SIZE=str(1 << 30))
+    r = subprocess.run([os.path.join(SOS_THREADS_DIR, name)], env=env, capture_output=True, text=True,
+                       timeout=100)
+    assert r.returncode == 0, (name, npes, r.stdout[-800:], r.stderr[-800:])
