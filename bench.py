@@ -416,6 +416,9 @@ def main():
                      # HIP runtime's own copy kernel (profiles/bulk_copy_256MiB_hbm_traffic.txt)
                      "traffic": 536896658, "kernel": "bulk_copy_kernel<true>",
                      "algorithmic_bytes_per_launch": head["bytes_per_step"]},
+        # the reference's own convention (tests/functional_tests/tester.cpp:505-508):
+        # payload bytes per second in GiB/s, counting each byte once
+        "reference_convention_payload_gib_s": round(256 * MiB / (head["ms"] * 1e-3) / 2**30, 1),
         "cpu_baseline": cpu,
         "all_configs": allc,
     }
