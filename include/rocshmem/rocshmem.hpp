@@ -14,28 +14,16 @@
 
 #include <hip/hip_runtime.h>
 
+#include <cassert>
 #include <cstdlib>
 
+// No MPI is used by this library; MPI_Comm only keeps rocshmem_init's
+// signature source-compatible.  Without a real mpi.h the names come from
+// compat/mpi.h.
 #if __has_include(<mpi.h>) && !defined(ROCSHMEM_AMD_NO_MPI_HEADER)
 #include <mpi.h>
 #else
-// No MPI is used by this library; the type only keeps rocshmem_init's
-// signature source-compatible.
-#ifndef ROCSHMEM_AMD_MPI_STANDIN
-#define ROCSHMEM_AMD_MPI_STANDIN 1
-typedef int MPI_Comm;
-#ifndef MPI_COMM_WORLD
-#define MPI_COMM_WORLD 0
-#endif
-#ifndef MPI_COMM_NULL
-#define MPI_COMM_NULL (-1)
-#endif
-// Programs written for the reference end a failed run with MPI_Abort.
-static inline int MPI_Abort(MPI_Comm, int errorcode) {
-  exit(errorcode);
-  return 0;
-}
-#endif
+#include "compat/mpi.h"
 #endif
 
 #include "rocshmem_config.h"

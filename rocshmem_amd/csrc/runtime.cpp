@@ -96,10 +96,19 @@ PeThreads g_threads;
 int pe_threads_count() { return g_threads.npes; }
 void pe_threads_start(int npes) { g_threads.npes = npes; }
 
+// ROCSHMEM_EMU_TRACE=1: one line on stderr per arrival at a meeting point.
+bool tracing() {
+  static const bool on = getenv("ROCSHMEM_EMU_TRACE") && atoi(getenv("ROCSHMEM_EMU_TRACE")) != 0;
+  return on;
+}
+
 bool pe_threads_enter(int start, int stride, int size, uint64_t *result) {
   if (tl_pe < 0 || g_threads.npes == 0 || size <= 1) return true;
   MeetingPoint &p = g_threads.at(start, stride, size);
   std::unique_lock<std::mutex> lk(p.m);
+  if (tracing())
+    fprintf(stderr, "rocshmem: PE %d arrives at (%d,%d,%d) round %llu as %d of %d\n", tl_pe, start,
+            stride, size, static_cast<unsigned long long>(p.round), p.arrived + 1, size);
   if (++p.arrived == size) return true;  // the last to arrive does the work (lock released here)
   const uint64_t round = p.round;
   p.cv.wait(lk, [&] { return p.round != round; });

@@ -392,3 +392,97 @@ def test_reference_host_programs_run_with_a_thread_per_pe(rt, name, npes):
     r = subprocess.run([os.path.join(SOS_THREADS_DIR, name)], env=env, capture_output=True, text=True,
                        timeout=100)
     assert r.returncode == 0, (name, npes, r.stdout[-800:], r.stderr[-800:])
+
+
+# ------------------------------------- the reference's device-API functional tests
+# The test matrix of scripts/functional_tests/driver.sh:142-320 (all of it runs
+# with 2 ranks): (test name, number of the TestType enum in
+# tests/functional_tests/tester.hpp, work-groups, threads per work-group,
+# largest message size or None).
+FUNCTIONAL_MATRIX = [
+    ("put", 2, 1, 1, 1048576), ("put", 2, 1, 1024, 512), ("put", 2, 8, 1, 1048576),
+    ("put", 2, 16, 128, 8), ("put", 2, 32, 256, 512), ("put", 2, 64, 1024, 8),
+    ("wgput", 27, 1, 64, 1048576), ("wgput", 27, 2, 64, 1048576), ("wgput", 27, 16, 64, 8),
+    ("waveput", 31, 1, 64, 1048576), ("waveput", 31, 2, 64, 1048576),
+    ("waveput", 31, 2, 128, 1048576), ("waveput", 31, 16, 128, 8),
+    ("teamctxput", 37, 1, 1, 1048576), ("get", 0, 1, 1, 1048576), ("get", 0, 1, 1024, 512),
+    ("get", 0, 8, 1, 1048576), ("get", 0, 16, 128, 8), ("get", 0, 32, 256, 512),
+    ("get", 0, 64, 1024, 8), ("wgget", 25, 1, 64, 1048576), ("wgget", 25, 2, 64, 1048576),
+    ("wgget", 25, 16, 64, 8), ("waveget", 29, 1, 64, 1048576), ("waveget", 29, 2, 64, 1048576),
+    ("waveget", 29, 2, 128, 1048576), ("waveget", 29, 16, 128, 8),
+    ("teamctxget", 35, 1, 1, 1048576), ("putnbi", 3, 1, 1, 1048576), ("putnbi", 3, 1, 1024, 512),
+    ("putnbi", 3, 8, 1, 1048576), ("putnbi", 3, 16, 128, 8), ("putnbi", 3, 32, 256, 512),
+    ("putnbi", 3, 64, 1024, 8), ("wgputnbi", 28, 1, 64, 1048576), ("wgputnbi", 28, 2, 64, 1048576),
+    ("wgputnbi", 28, 16, 64, 8), ("waveputnbi", 32, 1, 64, 1048576),
+    ("waveputnbi", 32, 2, 64, 1048576), ("waveputnbi", 32, 2, 128, 1048576),
+    ("waveputnbi", 32, 16, 128, 8), ("teamctxputnbi", 38, 1, 1, 1048576),
+    ("getnbi", 1, 1, 1, 1048576), ("getnbi", 1, 1, 1024, 512), ("getnbi", 1, 8, 1, 1048576),
+    ("getnbi", 1, 16, 128, 8), ("getnbi", 1, 32, 256, 512), ("getnbi", 1, 64, 1024, 8),
+    ("wggetnbi", 26, 1, 64, 1048576), ("wggetnbi", 26, 2, 64, 1048576),
+    ("wggetnbi", 26, 16, 64, 8), ("wavegetnbi", 30, 1, 64, 1048576),
+    ("wavegetnbi", 30, 2, 64, 1048576), ("wavegetnbi", 30, 2, 128, 1048576),
+    ("wavegetnbi", 30, 16, 128, 8), ("teamctxgetnbi", 36, 1, 1, 1048576),
+    ("amo_fetch", 7, 1, 1, None), ("amo_fetch", 7, 1, 1024, None), ("amo_fetch", 7, 8, 1, None),
+    ("amo_fetch", 7, 32, 128, None), ("amo_set", 41, 1, 1, None), ("amo_set", 41, 8, 1, None),
+    ("amo_set", 41, 32, 1, None), ("amo_fcswap", 8, 1, 1, None), ("amo_fcswap", 8, 32, 1, None),
+    ("amo_fcswap", 8, 8, 1, None), ("amo_finc", 6, 1, 1, None), ("amo_finc", 6, 1, 1024, None),
+    ("amo_finc", 6, 8, 1, None), ("amo_finc", 6, 32, 128, None), ("amo_inc", 10, 1, 1, None),
+    ("amo_inc", 10, 1, 1024, None), ("amo_inc", 10, 8, 1, None), ("amo_inc", 10, 32, 128, None),
+    ("amo_fadd", 5, 1, 1, None), ("amo_fadd", 5, 1, 1024, None), ("amo_fadd", 5, 8, 1, None),
+    ("amo_fadd", 5, 32, 128, None), ("amo_add", 9, 1, 1, None), ("amo_add", 9, 1, 1024, None),
+    ("amo_add", 9, 8, 1, None), ("amo_add", 9, 32, 128, None), ("amo_fetchand", 43, 1, 1, None),
+    ("amo_and", 46, 1, 1, None), ("amo_xor", 48, 1, 1, None), ("putsignal", 50, 1, 1, 1048576),
+    ("putsignal", 50, 2, 32, 1048576), ("wgputsignal", 51, 2, 32, 1048576),
+    ("waveputsignal", 52, 1, 32, 1048576), ("waveputsignal", 52, 2, 64, 1048576),
+    ("putsignalnbi", 53, 1, 1, 1048576), ("putsignalnbi", 53, 2, 32, 1048576),
+    ("wgputsignalnbi", 54, 2, 32, 1048576), ("waveputsignalnbi", 55, 1, 32, 1048576),
+    ("waveputsignalnbi", 55, 2, 64, 1048576), ("signalfetch", 56, 1, 1, None),
+    ("wgsignalfetch", 57, 2, 32, None), ("wavesignalfetch", 58, 1, 32, None),
+    ("wavesignalfetch", 58, 1, 64, None), ("barrierall", 15, 1, 1, None), ("sync", 17, 1, 1, None),
+    ("syncall", 16, 1, 1, None), ("alltoall", 20, 1, 1, 512), ("teambroadcast", 33, 1, 1, 32768),
+    ("fcollect", 19, 1, 1, 512), ("fcollect", 19, 1, 1, 32768), ("teamreduction", 34, 1, 1, 32768),
+    ("init", 12, 1, 1, None), ("pingpong", 13, 1, 1, None), ("pingpong", 13, 8, 1, None),
+    ("pingpong", 13, 32, 1, None), ("teamctxinfra", 39, 1, 1, None),
+]
+FUNCTIONAL_DRIVER = os.path.join(ROOT, "oracle", "_ref", "functional", "rocshmem_example_driver")
+# Tests in which BOTH ranks launch a kernel that finds its PE through the
+# default context or rocshmem_wg_ctx_create.  One process hosts both PEs here,
+# and such a kernel cannot tell which PE's thread launched it, so these stay
+# out.  So do the testers that keep a team handle in a file-scope variable,
+# which the two PE threads share and overwrite (team_reduction_tester.cpp:71,
+# team_ctx_primitive_tester.cpp).  Kernels that take their PE from a team
+# handle held per tester object (alltoall, broadcast, fcollect) or that only
+# PE 0 launches through the default context (all RMA, AMO and signalling
+# tests) run.
+FUNCTIONAL_NEEDS_ONE_PROCESS_PER_PE = {"pingpong", "barrierall", "sync", "syncall", "teamreduction",
+                                       "teamctxput", "teamctxget", "teamctxputnbi", "teamctxgetnbi"}
+
+
+def functional_cases():
+    if not os.path.exists(FUNCTIONAL_DRIVER):
+        return []
+    return [c for c in FUNCTIONAL_MATRIX if c[0] not in FUNCTIONAL_NEEDS_ONE_PROCESS_PER_PE]
+
+
+@pytest.mark.skipif(not functional_cases(),
+                    reason="oracle/_ref/functional is built where the reference tree exists")
+@pytest.mark.parametrize("name,number,wgs,threads,max_size", functional_cases(),
+                         ids=["%s-w%d-z%d-%s" % (c[0], c[2], c[3], c[4]) for c in functional_cases()])
+def test_reference_functional_driver(rt, name, number, wgs, threads, max_size):
+    """The reference's own functional test driver (tests/functional_tests: the
+    testers' kernels call rocshmem_putmem/getmem/_wg/_wave, the atomics,
+    put_signal, signal_fetch, team alltoall/broadcast/fcollect ... and each
+    tester verifies the data itself), compiled unchanged against these headers
+    by oracle/Makefile, run with 2 PEs as two host threads, with the arguments
+    of the reference's driver script.  Exit status 0 = the tester's own
+    verification passed for every message size.  Work-groups of different PEs
+    wait for each other inside kernels, so each PE thread's stream needs a
+    hardware queue of its own: 16 queues instead of HIP's default 4."""
+    rt.down()
+    env = dict(os.environ, ROCSHMEM_EMU_NPES="2", GPU_MAX_HW_QUEUES="16",
+               ROCSHMEM_MAX_NUM_CONTEXTS="1024" if name == "teamctxinfra" else str(wgs))
+    cmd = [FUNCTIONAL_DRIVER, "-a", str(number), "-w", str(wgs), "-z", str(threads)]
+    if max_size is not None:
+        cmd += ["-s", str(max_size)]
+    r = subprocess.run(cmd, env=env, capture_output=True, text=True, timeout=100)
+    assert r.returncode == 0, (name, r.stdout[-600:], r.stderr[-600:])
