@@ -34,8 +34,20 @@ enum PeRule : int {
   PE_RULE_FIXED = 0,    // DeviceState::fixed_pe
   PE_RULE_BLOCK_X = 1,  // blockIdx.x % n_pes
   PE_RULE_BLOCK_Y = 2,  // blockIdx.y % n_pes
-  PE_RULE_BLOCK_Z = 3   // blockIdx.z % n_pes
+  PE_RULE_BLOCK_Z = 3,  // blockIdx.z % n_pes
+  PE_RULE_QUEUE = 4     // the PE whose host thread bound the hardware queue the
+                        // kernel was dispatched on (DeviceState::queue_table)
 };
+
+// One entry of the queue -> PE table used when every PE is a host thread: the
+// thread binds each stream it launches on by running a one-thread kernel on
+// it, which records the id of the hardware queue it finds itself on.
+struct QueueBinding {
+  unsigned long long queue_id;
+  int pe;
+  int pad_;
+};
+constexpr int kQueueTableSize = 64;
 
 // (pe_start, stride, size) of a team with respect to the world team; the
 // object rocshmem_ctx_t::team_opaque points at.  Mirrors what the reference
@@ -119,6 +131,7 @@ struct DeviceState {
   CtxPool *ctx_pool;      // [n_pes] one pool per PE
   char *ws_base;          // work/sync area of PE 0
   uint64_t nt_bytes;      // copies at least this large use non-temporal accesses
+  QueueBinding *queue_table;  // [kQueueTableSize], indexed by queue id modulo the size
 };
 
 #if defined(__HIPCC__)
@@ -126,12 +139,25 @@ struct DeviceState {
 // This translation unit's copy of the runtime state.
 __attribute__((used)) static __constant__ DeviceState g_state;
 
+// Id of the hardware (HSA) queue this kernel was dispatched on: the `id`
+// field of hsa_queue_t, 32 bytes into the structure the queue pointer names.
+__device__ __forceinline__ unsigned long long dispatch_queue_id() {
+  typedef __attribute__((address_space(4))) unsigned long long constant_u64;
+  const constant_u64 *q = (const constant_u64 *)__builtin_amdgcn_queue_ptr();  // NOLINT
+  return q[4];
+}
+
 __device__ __forceinline__ int acting_pe() {
   const int n = g_state.n_pes;
   switch (g_state.pe_rule) {
     case PE_RULE_BLOCK_X: return static_cast<int>(blockIdx.x % n);
     case PE_RULE_BLOCK_Y: return static_cast<int>(blockIdx.y % n);
     case PE_RULE_BLOCK_Z: return static_cast<int>(blockIdx.z % n);
+    case PE_RULE_QUEUE: {
+      const unsigned long long id = dispatch_queue_id();
+      const QueueBinding b = g_state.queue_table[id % kQueueTableSize];
+      return b.queue_id == id ? b.pe : g_state.fixed_pe;
+    }
     default: return g_state.fixed_pe;
   }
 }
@@ -142,8 +168,15 @@ __device__ __forceinline__ Context *ctx_of(rocshmem_ctx_t ctx) {
   return c ? c : g_state.default_ctx + acting_pe();
 }
 
+// A team handle names one PE's object of the team.  When kernels take their PE
+// from the queue they were dispatched on (one host thread per PE), a handle
+// may come from a variable that the PE threads share, so it is re-read as
+// "this team" and resolved to the acting PE's object: the objects of one team
+// are consecutive, indexed by world PE.
 __device__ __forceinline__ Team *team_of(rocshmem_team_t team) {
-  return reinterpret_cast<Team *>(team);
+  Team *t = reinterpret_cast<Team *>(team);
+  if (t && g_state.pe_rule == PE_RULE_QUEUE) t = t - t->my_pe_in_world + acting_pe();
+  return t;
 }
 
 // Address of the same symmetric object on PE `pe`.

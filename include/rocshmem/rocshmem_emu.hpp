@@ -25,6 +25,8 @@
 #ifndef ROCSHMEM_AMD_EMU_HPP_
 #define ROCSHMEM_AMD_EMU_HPP_
 
+#include <hip/hip_runtime.h>
+
 #include <cstddef>
 
 #include "rocshmem_common.hpp"
@@ -35,12 +37,20 @@ enum rocshmem_emu_pe_rule {
   ROCSHMEM_EMU_PE_FIXED = 0,
   ROCSHMEM_EMU_PE_BLOCK_X = 1,
   ROCSHMEM_EMU_PE_BLOCK_Y = 2,
-  ROCSHMEM_EMU_PE_BLOCK_Z = 3
+  ROCSHMEM_EMU_PE_BLOCK_Z = 3,
+  ROCSHMEM_EMU_PE_QUEUE = 4  // the PE thread that bound the kernel's queue (the rule in PE threads)
 };
 
 // Runs pe_main(argc, argv) in npes threads (npes <= 0: ROCSHMEM_EMU_NPES), one
 // per PE, before the runtime is up; returns the first non-zero result.
 int rocshmem_emu_run_pes(int npes, int (*pe_main)(int, char **), int argc, char **argv);
+// In a PE thread: makes kernels launched on `stream` from now on act as this
+// thread's PE when they use the default context or rocshmem_wg_ctx_create
+// (a one-thread kernel on the stream records the hardware queue it runs on).
+// Each PE thread needs streams, and hardware queues, of its own
+// (GPU_MAX_HW_QUEUES at least the number of streams in use).  Compiling with
+// -DROCSHMEM_EMU_PE_THREADS makes hipLaunchKernelGGL call this by itself.
+void rocshmem_emu_bind_stream(hipStream_t stream);
 void rocshmem_emu_set_npes(int npes);
 void rocshmem_emu_set_pe(int pe);
 void rocshmem_emu_set_pe_rule(int rule);
@@ -53,6 +63,16 @@ rocshmem_team_t rocshmem_emu_team_on(rocshmem_team_t team, int pe);
 size_t rocshmem_emu_pe_stride();
 
 }  // namespace rocshmem
+
+#if defined(ROCSHMEM_EMU_PE_THREADS) || defined(ROCSHMEM_EMU_PE_THREADS_MAIN)
+// Every hipLaunchKernelGGL first binds its stream to the launching PE thread.
+#undef hipLaunchKernelGGLInternal
+#define hipLaunchKernelGGLInternal(kernelName, numBlocks, numThreads, memPerBlock, streamId, ...) \
+  do {                                                                                            \
+    ::rocshmem::rocshmem_emu_bind_stream(streamId);                                               \
+    kernelName<<<(numBlocks), (numThreads), (memPerBlock), (streamId)>>>(__VA_ARGS__);            \
+  } while (0)
+#endif
 
 #if defined(ROCSHMEM_EMU_PE_THREADS_MAIN)
 // The program's own main, under another name, in whichever of the usual

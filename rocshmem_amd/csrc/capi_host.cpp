@@ -27,7 +27,7 @@ int rocshmem_amd_set_pe(int pe) {
   return 0;
 }
 int rocshmem_amd_set_pe_rule(int rule) {
-  if (!rt().live || rule < 0 || rule > 3) return -1;
+  if (!rt().live || rule < 0 || rule > 4) return -1;
   rt().set_pe_rule(rule);
   return 0;
 }

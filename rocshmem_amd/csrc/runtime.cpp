@@ -271,12 +271,24 @@ int Runtime::init(int want_npes, size_t want_heap) {
   RT_CHECK_HIP(hipMemcpy(d_pools, pools.data(), sizeof(detail::CtxPool) * npes,
                          hipMemcpyHostToDevice));
 
+  // Queue -> PE table; no queue is bound yet (an id no queue has).
+  {
+    std::vector<detail::QueueBinding> none(detail::kQueueTableSize,
+                                           detail::QueueBinding{~0ull, 0, 0});
+    RT_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&d_queue_table),
+                           sizeof(detail::QueueBinding) * none.size()));
+    RT_CHECK_HIP(hipMemcpy(d_queue_table, none.data(), sizeof(detail::QueueBinding) * none.size(),
+                           hipMemcpyHostToDevice));
+  }
+  state.queue_table = d_queue_table;
   state.heap_base = heap_base;
   state.pe_stride = pe_stride;
   state.heap_size = heap_size;
   state.ws_stride = ws_stride;
   state.n_pes = npes;
-  state.pe_rule = detail::PE_RULE_FIXED;
+  // With a host thread per PE, kernels learn their PE from the queue their
+  // launching thread bound (rocshmem_emu_bind_stream).
+  state.pe_rule = pe_threads_count() > 0 ? detail::PE_RULE_QUEUE : detail::PE_RULE_FIXED;
   state.fixed_pe = 0;
   state.max_teams = max_teams;
   state.default_ctx = d_default_ctx;
@@ -293,6 +305,8 @@ int Runtime::init(int want_npes, size_t want_heap) {
 void Runtime::finalize() {
   if (!live) return;
   RT_CHECK_HIP(hipDeviceSynchronize());
+  RT_CHECK_HIP(hipFree(d_queue_table));
+  d_queue_table = nullptr;
   RT_CHECK_HIP(hipFree(d_pools));
   RT_CHECK_HIP(hipFree(d_ctx_slots));
   RT_CHECK_HIP(hipFree(d_default_ctx));
@@ -439,7 +453,7 @@ void Runtime::set_pe(int pe) {
 
 void Runtime::set_pe_rule(int rule) {
   require_live("rocshmem_emu_set_pe_rule");
-  if (rule < detail::PE_RULE_FIXED || rule > detail::PE_RULE_BLOCK_Z) {
+  if (rule < detail::PE_RULE_FIXED || rule > detail::PE_RULE_QUEUE) {
     fprintf(stderr, "rocshmem: unknown PE rule %d\n", rule);
     abort();
   }
@@ -573,8 +587,18 @@ __host__ int rocshmem_team_split_strided(rocshmem_team_t parent_team, int start,
   }
   const int rc = static_cast<int>(packed >> 32) - 1;
   const int slot = static_cast<int>(packed & 0xffffffffu) - 1;
+  // Every member receives the same handle (the first member's object), so a
+  // program that keeps it in a variable its PE threads share still works; the
+  // host calls and, under the queue rule, the device calls resolve it to the
+  // caller's own object.
   *new_team = ROCSHMEM_TEAM_INVALID;
-  if (rc == 0 && slot >= 0) *new_team = rt().team_on(rt().team_handle(slot, w.pe_start), rt().me());
+  if (rc == 0 && slot >= 0) {
+    const rocshmem_team_t mine = rt().team_on(rt().team_handle(slot, w.pe_start), rt().me());
+    if (mine != ROCSHMEM_TEAM_INVALID) {
+      const detail::Team *t = rt().host_team(mine);
+      *new_team = rt().team_handle(slot, t->wrt_world.pe_start);
+    }
+  }
   return rc;
 }
 __host__ void rocshmem_team_destroy(rocshmem_team_t team) {
@@ -608,6 +632,29 @@ __host__ void rocshmem_sync_all() { rocshmem_barrier_all(); }
 __host__ void rocshmem_global_exit(int status) {
   fflush(nullptr);
   _Exit(status);
+}
+
+namespace {
+__global__ void bind_queue_kernel(detail::QueueBinding *table, int pe) {
+  const unsigned long long id = detail::dispatch_queue_id();
+  table[id % detail::kQueueTableSize] = detail::QueueBinding{id, pe, 0};
+}
+}  // namespace
+
+void rocshmem_emu_bind_stream(hipStream_t stream) {
+  if (runtime::tl_pe < 0 || !rt().live) return;
+  // Streams this thread has bound since the runtime came up.
+  static thread_local std::vector<hipStream_t> bound;
+  static thread_local const void *bound_for = nullptr;
+  if (bound_for != rt().d_queue_table) {
+    bound.clear();
+    bound_for = rt().d_queue_table;
+  }
+  if (std::find(bound.begin(), bound.end(), stream) != bound.end()) return;
+  hipLaunchKernelGGL(bind_queue_kernel, dim3(1), dim3(1), 0, stream, rt().d_queue_table,
+                     runtime::tl_pe);
+  RT_CHECK_HIP(hipGetLastError());
+  bound.push_back(stream);
 }
 
 int rocshmem_emu_run_pes(int npes, int (*pe_main)(int, char **), int argc, char **argv) {

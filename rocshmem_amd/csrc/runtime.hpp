@@ -36,6 +36,7 @@ struct Runtime {
   detail::Context *d_default_ctx = nullptr;  // [2*npes]: default, then NOSTORE
   detail::Context *d_ctx_slots = nullptr;  // [npes][max_ctxs]
   detail::CtxPool *d_pools = nullptr;      // [npes]
+  detail::QueueBinding *d_queue_table = nullptr;  // [kQueueTableSize]
   std::vector<detail::Team> h_teams;       // host mirror of d_teams
   std::vector<bool> team_slot_used;
   Pow2Allocator allocator;

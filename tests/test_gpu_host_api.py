@@ -445,17 +445,11 @@ FUNCTIONAL_MATRIX = [
     ("pingpong", 13, 32, 1, None), ("teamctxinfra", 39, 1, 1, None),
 ]
 FUNCTIONAL_DRIVER = os.path.join(ROOT, "oracle", "_ref", "functional", "rocshmem_example_driver")
-# Tests in which BOTH ranks launch a kernel that finds its PE through the
-# default context or rocshmem_wg_ctx_create.  One process hosts both PEs here,
-# and such a kernel cannot tell which PE's thread launched it, so these stay
-# out.  So do the testers that keep a team handle in a file-scope variable,
-# which the two PE threads share and overwrite (team_reduction_tester.cpp:71,
-# team_ctx_primitive_tester.cpp).  Kernels that take their PE from a team
-# handle held per tester object (alltoall, broadcast, fcollect) or that only
-# PE 0 launches through the default context (all RMA, AMO and signalling
-# tests) run.
-FUNCTIONAL_NEEDS_ONE_PROCESS_PER_PE = {"pingpong", "barrierall", "sync", "syncall", "teamreduction",
-                                       "teamctxput", "teamctxget", "teamctxputnbi", "teamctxgetnbi"}
+# Nothing is left out: kernels that both ranks launch find their PE through the
+# hardware queue their PE thread bound, and team handles kept in file-scope
+# variables (team_reduction_tester.cpp:71, team_ctx_primitive_tester.cpp:29)
+# are the same value in every PE thread.
+FUNCTIONAL_NEEDS_ONE_PROCESS_PER_PE = set()
 
 
 def functional_cases():
