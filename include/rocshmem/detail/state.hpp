@@ -218,8 +218,10 @@ void register_state_uploader(StateUploader fn);
 
 #if defined(__HIPCC__)
 static void upload_state_to_this_tu(const DeviceState *s) {
-  hipError_t e = hipMemcpyToSymbol(HIP_SYMBOL(g_state), s, sizeof(DeviceState),
-                                   0, hipMemcpyHostToDevice);
+  // The address form of the symbol: the only one every HIP build mode offers
+  // (a per-thread default stream leaves out the reference-taking overload).
+  hipError_t e = hipMemcpyToSymbol(static_cast<const void *>(&g_state), s, sizeof(DeviceState), 0,
+                                   hipMemcpyHostToDevice);
   if (e != hipSuccess) {
     fprintf(stderr, "rocshmem: state upload failed: %s\n", hipGetErrorString(e));
     abort();

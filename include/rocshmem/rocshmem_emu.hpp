@@ -51,6 +51,10 @@ int rocshmem_emu_run_pes(int npes, int (*pe_main)(int, char **), int argc, char 
 // (GPU_MAX_HW_QUEUES at least the number of streams in use).  Compiling with
 // -DROCSHMEM_EMU_PE_THREADS makes hipLaunchKernelGGL call this by itself.
 void rocshmem_emu_bind_stream(hipStream_t stream);
+// In a PE thread: waits for the streams this thread has bound, i.e. for this
+// PE's own device work, as hipDeviceSynchronize does in a process that is one
+// PE.  -DROCSHMEM_EMU_PE_THREADS makes hipDeviceSynchronize() mean this.
+hipError_t rocshmem_emu_device_synchronize();
 void rocshmem_emu_set_npes(int npes);
 void rocshmem_emu_set_pe(int pe);
 void rocshmem_emu_set_pe_rule(int rule);
@@ -65,7 +69,10 @@ size_t rocshmem_emu_pe_stride();
 }  // namespace rocshmem
 
 #if defined(ROCSHMEM_EMU_PE_THREADS) || defined(ROCSHMEM_EMU_PE_THREADS_MAIN)
-// Every hipLaunchKernelGGL first binds its stream to the launching PE thread.
+// hipDeviceSynchronize() covers the calling PE's work only (the other PEs'
+// kernels may be waiting for one this thread has yet to launch), and every
+// hipLaunchKernelGGL first binds its stream to the launching PE thread.
+#define hipDeviceSynchronize() ::rocshmem::rocshmem_emu_device_synchronize()
 #undef hipLaunchKernelGGLInternal
 #define hipLaunchKernelGGLInternal(kernelName, numBlocks, numThreads, memPerBlock, streamId, ...) \
   do {                                                                                            \

@@ -495,6 +495,10 @@ __host__ void rocshmem_init(MPI_Comm) {
     rt().init(runtime::pe_threads_count(), 0);
     w.done();
   }
+  // A program built with -fgpu-default-stream=per-thread launches its
+  // kernel<<<grid, block>>> on this thread's own default stream: bind it now,
+  // since such launches do not pass through hipLaunchKernelGGL.
+  if (runtime::tl_pe >= 0) rocshmem_emu_bind_stream(hipStreamPerThread);
 }
 __host__ void rocshmem_init_thread(int, int *provided, MPI_Comm comm) {
   rocshmem_init(comm);
@@ -619,9 +623,13 @@ __host__ void rocshmem_fence() { RT_CHECK_HIP(hipDeviceSynchronize()); }
 __host__ void rocshmem_ctx_quiet(rocshmem_ctx_t) { RT_CHECK_HIP(hipDeviceSynchronize()); }
 __host__ void rocshmem_quiet() { RT_CHECK_HIP(hipDeviceSynchronize()); }
 __host__ void rocshmem_barrier_all() {
+  // A PE thread drains its own streams and then meets the others; draining the
+  // whole device from here could wait on a kernel of another PE that in turn
+  // waits for work this PE launches after the barrier.
+  if (runtime::tl_pe >= 0) RT_CHECK_HIP(rocshmem_emu_device_synchronize());
   WorldMeeting w;
   if (w.mine) {
-    RT_CHECK_HIP(hipDeviceSynchronize());
+    if (runtime::tl_pe < 0) RT_CHECK_HIP(hipDeviceSynchronize());
     w.done();
   }
 }
@@ -641,20 +649,40 @@ __global__ void bind_queue_kernel(detail::QueueBinding *table, int pe) {
 }
 }  // namespace
 
-void rocshmem_emu_bind_stream(hipStream_t stream) {
-  if (runtime::tl_pe < 0 || !rt().live) return;
-  // Streams this thread has bound since the runtime came up.
+namespace {
+// Streams the calling PE thread has bound since the runtime came up.
+std::vector<hipStream_t> &bound_streams() {
   static thread_local std::vector<hipStream_t> bound;
   static thread_local const void *bound_for = nullptr;
   if (bound_for != rt().d_queue_table) {
     bound.clear();
     bound_for = rt().d_queue_table;
   }
+  return bound;
+}
+}  // namespace
+
+void rocshmem_emu_bind_stream(hipStream_t stream) {
+  if (runtime::tl_pe < 0 || !rt().live) return;
+  std::vector<hipStream_t> &bound = bound_streams();
   if (std::find(bound.begin(), bound.end(), stream) != bound.end()) return;
   hipLaunchKernelGGL(bind_queue_kernel, dim3(1), dim3(1), 0, stream, rt().d_queue_table,
                      runtime::tl_pe);
   RT_CHECK_HIP(hipGetLastError());
   bound.push_back(stream);
+}
+
+// What hipDeviceSynchronize means to a process that is one PE: wait for this
+// PE's own work.  The device-wide call would also wait for the kernels of the
+// other PE threads, which may be waiting for a kernel this thread has yet to
+// launch.
+hipError_t rocshmem_emu_device_synchronize() {
+  if (runtime::tl_pe < 0 || !rt().live) return hipDeviceSynchronize();
+  for (hipStream_t s : bound_streams()) {
+    const hipError_t e = hipStreamSynchronize(s);
+    if (e != hipSuccess) return e;
+  }
+  return hipSuccess;
 }
 
 int rocshmem_emu_run_pes(int npes, int (*pe_main)(int, char **), int argc, char **argv) {

@@ -480,3 +480,32 @@ def test_reference_functional_driver(rt, name, number, wgs, threads, max_size):
         cmd += ["-s", str(max_size)]
     r = subprocess.run(cmd, env=env, capture_output=True, text=True, timeout=100)
     assert r.returncode == 0, (name, r.stdout[-600:], r.stderr[-600:])
+
+
+# ------------------------------------------------- the reference's example programs
+EXAMPLES_DIR = os.path.join(ROOT, "oracle", "_ref", "examples")
+
+
+def example_programs():
+    if not os.path.isdir(EXAMPLES_DIR):
+        return []
+    return sorted(f for f in os.listdir(EXAMPLES_DIR) if os.access(os.path.join(EXAMPLES_DIR, f), os.X_OK))
+
+
+@pytest.mark.skipif(not example_programs(), reason="oracle/_ref/examples is built where the reference tree exists")
+@pytest.mark.parametrize("npes", [2, 8])
+@pytest.mark.parametrize("name", example_programs())
+def test_reference_examples_run_with_a_thread_per_pe(rt, name, npes):
+    """examples/*.cc of the reference (all-reduce, alltoall, broadcast, getmem,
+    put_signal + wait_until inside kernels that every PE launches with
+    kernel<<<...>>> on its default stream), built unchanged by oracle/Makefile
+    with a per-thread default stream, one host thread per PE.  Each PE checks
+    its own result and prints [PASS] or [FAIL] (the broadcast root checks
+    nothing)."""
+    rt.down()
+    env = dict(os.environ, ROCSHMEM_EMU_NPES=str(npes), GPU_MAX_HW_QUEUES="16")
+    r = subprocess.run([os.path.join(EXAMPLES_DIR, name)], env=env, capture_output=True, text=True,
+                       timeout=100)
+    assert r.returncode == 0, (name, npes, r.stdout[-600:], r.stderr[-600:])
+    assert r.stdout.count("[FAIL]") == 0, r.stdout[-600:]
+    assert r.stdout.count("[PASS]") >= npes - 1, r.stdout[-600:]
