@@ -135,18 +135,34 @@ __device__ __forceinline__ void copy_lanes(void *dst, const void *src, size_t n,
                                            size_t nt_bytes = kNonTemporalBytes) {
   char *d = static_cast<char *>(dst);
   const char *s = static_cast<const char *>(src);
-  if (n >= nt_bytes) {
+  // Few lanes (one or two wavefronts) cannot cover the memory latency with 4
+  // loads each; they keep 16 in flight.  A full work-group saturates its CU
+  // with 4.
+  if (nlanes <= 128 && n >= nlanes * 256) {
+    if (n >= nt_bytes) copy_lanes_impl<16, true>(d, s, n, lane, nlanes);
+    else copy_lanes_impl<16, false>(d, s, n, lane, nlanes);
+  } else if (n >= nt_bytes) {
     copy_lanes_impl<4, true>(d, s, n, lane, nlanes);
   } else {
     copy_lanes_impl<4, false>(d, s, n, lane, nlanes);
   }
 }
 
-// One lane copies n bytes on its own: 16-byte moves, then 8/4/2/1.
+// One lane copies n bytes on its own: 16-byte moves, then 8/4/2/1.  A lone
+// lane is bound by memory latency, so large messages keep eight loads in
+// flight (measured: 1 MiB from one thread in 7 ms with one load at a time).
 __device__ __forceinline__ void copy_thread(void *dst, const void *src,
                                             size_t n) {
   char *d = static_cast<char *>(dst);
   const char *s = static_cast<const char *>(src);
+  while (n >= 128) {
+    u32x4 v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const u32x4_any *>(s + 16 * u);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) *reinterpret_cast<u32x4_any *>(d + 16 * u) = v[u];
+    d += 128; s += 128; n -= 128;
+  }
   while (n >= 16) {
     *reinterpret_cast<u32x4_any *>(d) = *reinterpret_cast<const u32x4_any *>(s);
     d += 16; s += 16; n -= 16;
