@@ -55,6 +55,10 @@ void rocshmem_emu_bind_stream(hipStream_t stream);
 // PE's own device work, as hipDeviceSynchronize does in a process that is one
 // PE.  -DROCSHMEM_EMU_PE_THREADS makes hipDeviceSynchronize() mean this.
 hipError_t rocshmem_emu_device_synchronize();
+// Tells the library that the program was built with
+// -fgpu-default-stream=per-thread, so that rocshmem_init binds each PE
+// thread's own default stream.  Called by itself in such builds (below).
+void rocshmem_emu_per_thread_default_stream();
 void rocshmem_emu_set_npes(int npes);
 void rocshmem_emu_set_pe(int pe);
 void rocshmem_emu_set_pe_rule(int rule);
@@ -67,6 +71,16 @@ rocshmem_team_t rocshmem_emu_team_on(rocshmem_team_t team, int pe);
 size_t rocshmem_emu_pe_stride();
 
 }  // namespace rocshmem
+
+#if (defined(ROCSHMEM_EMU_PE_THREADS) || defined(ROCSHMEM_EMU_PE_THREADS_MAIN)) && \
+    defined(HIP_API_PER_THREAD_DEFAULT_STREAM)
+namespace rocshmem {
+namespace detail {
+__attribute__((used)) static const int per_thread_default_stream_announced_ =
+    (rocshmem_emu_per_thread_default_stream(), 0);
+}  // namespace detail
+}  // namespace rocshmem
+#endif
 
 #if defined(ROCSHMEM_EMU_PE_THREADS) || defined(ROCSHMEM_EMU_PE_THREADS_MAIN)
 // hipDeviceSynchronize() covers the calling PE's work only (the other PEs'

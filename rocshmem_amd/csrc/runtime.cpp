@@ -48,6 +48,7 @@ std::vector<detail::StateUploader> &uploaders() {
 
 Runtime g_rt;
 int g_requested_npes = 0;
+bool g_per_thread_default_stream = false;
 
 size_t env_size(const char *name, size_t fallback) {
   const char *v = getenv(name);
@@ -497,8 +498,10 @@ __host__ void rocshmem_init(MPI_Comm) {
   }
   // A program built with -fgpu-default-stream=per-thread launches its
   // kernel<<<grid, block>>> on this thread's own default stream: bind it now,
-  // since such launches do not pass through hipLaunchKernelGGL.
-  if (runtime::tl_pe >= 0) rocshmem_emu_bind_stream(hipStreamPerThread);
+  // since such launches do not pass through hipLaunchKernelGGL.  (Not for
+  // other programs: the stream would take a hardware queue for nothing.)
+  if (runtime::tl_pe >= 0 && runtime::g_per_thread_default_stream)
+    rocshmem_emu_bind_stream(hipStreamPerThread);
 }
 __host__ void rocshmem_init_thread(int, int *provided, MPI_Comm comm) {
   rocshmem_init(comm);
@@ -707,6 +710,7 @@ int rocshmem_emu_run_pes(int npes, int (*pe_main)(int, char **), int argc, char 
 }
 
 void rocshmem_emu_set_npes(int npes) { runtime::g_requested_npes = npes; }
+void rocshmem_emu_per_thread_default_stream() { runtime::g_per_thread_default_stream = true; }
 void rocshmem_emu_set_pe(int pe) { rt().set_pe(pe); }
 void rocshmem_emu_set_pe_rule(int rule) { rt().set_pe_rule(rule); }
 void *rocshmem_emu_pe_ptr(const void *ptr, int pe) { return rt().pe_ptr(ptr, pe); }
