@@ -414,7 +414,7 @@ def main():
                      "unit": "GB/s", "frac": round(head["gbs"] / HBM_PEAK_GBS, 4),
                      # FETCH_SIZE + WRITE_SIZE per launch under rocprofv3 --pmc, scaled by the
                      # HIP runtime's own copy kernel (profiles/bulk_copy_256MiB_hbm_traffic.txt)
-                     "traffic": 536896658, "kernel": "bulk_copy_kernel<true>",
+                     "traffic": 536896718, "kernel": "bulk_copy_kernel<true>",
                      "algorithmic_bytes_per_launch": head["bytes_per_step"]},
         # the reference's own convention (tests/functional_tests/tester.cpp:505-508):
         # payload bytes per second in GiB/s, counting each byte once

@@ -130,21 +130,22 @@ __device__ __forceinline__ void copy_lanes_impl(char *dst, const char *src, size
   copy_window<kUnroll, kNonTemporal>(dst, src, n, lane, nlanes);
 }
 
+// kLoads: 16-byte loads each lane keeps in flight.  4 saturates a CU when a
+// full work-group copies; a lone wavefront needs more to cover the memory
+// latency.  The register count of a kernel is that of its widest path, so the
+// deeper variant is chosen per call site, not at run time: with 8 in a
+// work-group path the tiled whole-GPU put lost a quarter of its bandwidth to
+// halved occupancy.
+template <int kLoads = 4>
 __device__ __forceinline__ void copy_lanes(void *dst, const void *src, size_t n, size_t lane,
                                            size_t nlanes,
                                            size_t nt_bytes = kNonTemporalBytes) {
   char *d = static_cast<char *>(dst);
   const char *s = static_cast<const char *>(src);
-  // Few lanes (one or two wavefronts) cannot cover the memory latency with 4
-  // loads each; they keep 16 in flight.  A full work-group saturates its CU
-  // with 4.
-  if (nlanes <= 128 && n >= nlanes * 256) {
-    if (n >= nt_bytes) copy_lanes_impl<16, true>(d, s, n, lane, nlanes);
-    else copy_lanes_impl<16, false>(d, s, n, lane, nlanes);
-  } else if (n >= nt_bytes) {
-    copy_lanes_impl<4, true>(d, s, n, lane, nlanes);
+  if (n >= nt_bytes) {
+    copy_lanes_impl<kLoads, true>(d, s, n, lane, nlanes);
   } else {
-    copy_lanes_impl<4, false>(d, s, n, lane, nlanes);
+    copy_lanes_impl<kLoads, false>(d, s, n, lane, nlanes);
   }
 }
 
@@ -199,7 +200,7 @@ __device__ __forceinline__ void copy_wave(void *dst, const void *src, size_t n,
                                           size_t nt_bytes = kNonTemporalBytes) {
   unsigned count;
   const unsigned rank = active_lane_rank(&count);
-  copy_lanes(dst, src, n, rank, count, nt_bytes);
+  copy_lanes<8>(dst, src, n, rank, count, nt_bytes);
 }
 
 }  // namespace detail
