@@ -170,6 +170,25 @@ def to_all_configs(b, steps, warmup):
         alg = 2 * P * n * es
         res[name] = {"ms": round(ms, 4), "gbs": round(alg / ms / 1e6, 1),
                      "frac": round(alg / ms / 1e6 / HBM_PEAK_GBS, 4)}
+        if name == "fp32_sum":
+            # The device call rocshmem_ctx_float_sum_wg_reduce: by its contract ONE
+            # work-group per PE takes part, so 8 of the 256 CUs do all the work.
+            ms = b.time_ms(lambda: l.wg_reduce(dt, op, l.team_world(), dst, src, n, 1024, None), 3, 1)
+            res["fp32_sum_wg_reduce_one_wg_per_pe"] = {"ms": round(ms, 4),
+                                                       "gbs": round(alg / ms / 1e6, 1)}
+            # ... and the way the reference's testers scale it: one team per
+            # work-group, 64 teams x 8 PEs at once (two work-groups per CU).
+            NT = 64
+            teams = (C.c_void_p * NT)()
+            for t in range(NT):
+                h = C.c_void_p()
+                assert l.team_split_strided(l.team_world(), 0, 1, P, C.byref(h)) == 0 and h.value
+                teams[t] = h.value
+            ms = b.time_ms(lambda: l.wg_reduce_teams(dt, op, teams, NT, dst, src, n, 1024, None), 3, 1)
+            res["fp32_sum_wg_reduce_64_teams"] = {"ms": round(ms, 4), "gbs": round(alg / ms / 1e6, 1),
+                                                  "frac": round(alg / ms / 1e6 / HBM_PEAK_GBS, 4)}
+            for t in range(NT):
+                l.team_destroy(teams[t])
         l.free(src)
         l.free(dst)
     return res
@@ -373,6 +392,7 @@ def main():
     # 8 slices of 8 GiB: with Zipf(1.1) routing the busiest PE receives 2.3 GiB
     # of rows, a 4 GiB block of the power-of-two allocator.  That request goes
     # first because the allocator never merges freed blocks.
+    os.environ.setdefault("ROCSHMEM_MAX_NUM_TEAMS", "72")  # the many-teams all-reduce uses 64
     assert b.l.init(P, 8 << 30) == 0
     allc = {}
     if not a.quick:

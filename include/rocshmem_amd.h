@@ -236,6 +236,15 @@ int rocshmem_amd_wf_coalesce(const int *pe, const uint64_t *src, const uint64_t 
 int rocshmem_amd_wg_reduce(int dtype, int op, rocshmem_amd_team_t team, void *dest,
                            const void *source, int nreduce, int wg_size,
                            rocshmem_amd_stream_t stream);
+/* The same call made by n_teams (<= 64) work-groups per PE at once, each with a
+ * team of its own over the same PEs — how the reference's testers spread a
+ * device collective over the GPU (one team per work-group,
+ * tests/functional_tests/team_reduction_tester.cpp:60-110).  Team t reduces
+ * the t-th slice of the arrays (equal slices, whole 16-byte vectors).  teams:
+ * host array of handles of distinct teams with the same members. */
+int rocshmem_amd_wg_reduce_teams(int dtype, int op, const rocshmem_amd_team_t *teams, int n_teams,
+                                 void *dest, const void *source, int nreduce, int wg_size,
+                                 rocshmem_amd_stream_t stream);
 /* rocshmem_ctx_<T>_wg_alltoall / _wg_broadcast / _wg_fcollect
  * (rocshmem_COLL.hpp:44-258; context_ipc_tmpl_device.hpp:420-531).
  * elem_size in {1,2,4,8} selects the typed entry point (char/short/int/long). */

@@ -83,6 +83,40 @@ __global__ void wg_reduce_kernel(WgCollArgs a) {
   if (threadIdx.x == 0 && rc != ROCSHMEM_SUCCESS) atomicMax(a.status, rc);
 }
 
+// Several teams over the same PEs at once, the way the reference's testers
+// scale a device collective (one team per work-group,
+// tests/functional_tests/team_reduction_tester.cpp): work-group (x, y) acts
+// for member x of team y and reduces the y-th slice of the arrays.
+constexpr int kMaxTeamsPerLaunch = 64;
+struct WgTeamsArgs {
+  detail::Team *rows[kMaxTeamsPerLaunch];  // team objects of each team, indexed by world PE
+  detail::Context *ctx_row;
+  char *dest0;
+  const char *src0;
+  uint64_t pe_stride;
+  int pe_start;
+  int stride;
+  int nelems;       // all slices together
+  int slice_elems;  // per team
+  int *status;
+};
+
+template <typename T, ROCSHMEM_OP Op>
+__global__ void wg_reduce_teams_kernel(WgTeamsArgs a) {
+  const int pe = a.pe_start + static_cast<int>(blockIdx.x) * a.stride;
+  detail::Team *row = a.rows[blockIdx.y];
+  const rocshmem_ctx_t ctx{a.ctx_row + pe, &row[pe].wrt_world};
+  const rocshmem_team_t team = reinterpret_cast<rocshmem_team_t>(row + pe);
+  const long lo = static_cast<long>(blockIdx.y) * a.slice_elems;
+  long cnt = a.nelems - lo;
+  if (cnt > a.slice_elems) cnt = a.slice_elems;
+  if (cnt < 0) cnt = 0;
+  T *dest = reinterpret_cast<T *>(a.dest0 + static_cast<uint64_t>(pe) * a.pe_stride) + lo;
+  const T *source = reinterpret_cast<const T *>(a.src0 + static_cast<uint64_t>(pe) * a.pe_stride) + lo;
+  const int rc = PublicReduce<T, Op>::call(ctx, team, dest, source, static_cast<int>(cnt));
+  if (threadIdx.x == 0 && rc != ROCSHMEM_SUCCESS) atomicMax(a.status, rc);
+}
+
 enum WgMove { MOVE_ALLTOALL, MOVE_BROADCAST, MOVE_FCOLLECT };
 
 template <typename T, int kMove>
@@ -453,6 +487,63 @@ int rocshmem_amd_wg_reduce(int dtype, int op, rocshmem_amd_team_t team, void *de
   const bool ok = for_dtype_op(dtype, op, [&](auto *tag, auto opc) {
     using T = typename std::remove_pointer<decltype(tag)>::type;
     launch_wg_reduce<T, decltype(opc)::value>(a, v.host->num_pes, wg_size, s);
+  });
+  int status = -1;
+  if (ok) {
+    DRV_CHECK_HIP(hipGetLastError());
+    DRV_CHECK_HIP(hipStreamSynchronize(s));
+    DRV_CHECK_HIP(hipMemcpy(&status, d_status, sizeof(int), hipMemcpyDeviceToHost));
+  }
+  DRV_CHECK_HIP(hipFree(d_status));
+  return status;
+}
+
+int rocshmem_amd_wg_reduce_teams(int dtype, int op, const rocshmem_amd_team_t *teams, int n_teams,
+                                 void *dest, const void *source, int nreduce, int wg_size,
+                                 rocshmem_amd_stream_t stream) {
+  if (!teams || n_teams < 1 || n_teams > kMaxTeamsPerLaunch || !valid_launch(1, wg_size) ||
+      nreduce < 0)
+    return -1;
+  TeamView first;
+  if (!view_team(teams[0], &first)) return -1;
+  WgTeamsArgs a;
+  for (int t = 0; t < n_teams; ++t) {
+    TeamView v;
+    if (!view_team(teams[t], &v)) return -1;
+    const detail::TeamInfo &x = v.host->wrt_world, &y = first.host->wrt_world;
+    if (x.pe_start != y.pe_start || x.stride != y.stride || x.size != y.size) return -1;
+    for (int u = 0; u < t; ++u)
+      if (a.rows[u] == v.row) return -1;  // one work-group per team member
+    a.rows[t] = v.row;
+  }
+  const size_t es = dtype_size(dtype);
+  {
+    const size_t bytes = static_cast<size_t>(nreduce) * es;
+    const int me = runtime::rt().me();
+    if (!es || !sym_ok_on(dest, bytes, me) || !sym_ok_on(source, bytes, me)) return -1;
+  }
+  auto &r = runtime::rt();
+  int *d_status;
+  DRV_CHECK_HIP(hipMalloc(&d_status, sizeof(int)));
+  DRV_CHECK_HIP(hipMemset(d_status, 0, sizeof(int)));
+  a.ctx_row = r.d_default_ctx;
+  a.dest0 = on_pe0(dest);
+  a.src0 = on_pe0(source);
+  a.pe_stride = r.pe_stride;
+  a.pe_start = first.host->wrt_world.pe_start;
+  a.stride = first.host->wrt_world.stride;
+  a.nelems = nreduce;
+  // Equal slices, a whole number of 16-byte vectors each.
+  const int per_vec = static_cast<int>(16 / es);
+  int slice = (nreduce + n_teams - 1) / n_teams;
+  slice = (slice + per_vec - 1) / per_vec * per_vec;
+  a.slice_elems = slice > 0 ? slice : per_vec;
+  a.status = d_status;
+  hipStream_t s = as_stream(stream);
+  const dim3 grid(first.host->num_pes, n_teams), block(wg_size);
+  const bool ok = for_dtype_op(dtype, op, [&](auto *tag, auto opc) {
+    using T = typename std::remove_pointer<decltype(tag)>::type;
+    hipLaunchKernelGGL((wg_reduce_teams_kernel<T, decltype(opc)::value>), grid, block, 0, s, a);
   });
   int status = -1;
   if (ok) {

@@ -164,6 +164,53 @@ def test_active_sets_and_teams(rt, L, orc):
     l.set_pe(0)
 
 
+@pytest.mark.parametrize("n_teams", [1, 3, 16, 39])
+def test_many_teams_reduce_their_slices_at_once(rt, L, orc, n_teams):
+    """tests/functional_tests/team_reduction_tester.cpp: one team per
+    work-group.  n_teams duplicates of a team each reduce their slice of one
+    array in the same launch; the whole array must equal the oracle's fold,
+    for the world team and for a strided one, with ragged sizes."""
+    import ctypes
+    l = rt.up(8, HEAP)
+    for start, stride, size in [(0, 1, 8), (1, 2, 3)]:
+        pes = [start + stride * k for k in range(size)]
+        l.set_pe(pes[0])
+        teams = (ctypes.c_void_p * n_teams)()
+        for t in range(n_teams):
+            h = ctypes.c_void_p()
+            assert l.team_split_strided(l.team_world(), start, stride, size, ctypes.byref(h)) == 0 and h.value
+            teams[t] = h.value
+        for dtype_name, op_name, n in [("FLOAT", "SUM", 100003), ("INT", "XOR", 7), ("BF16", "SUM", 4099),
+                                       ("DOUBLE", "MAX", 1 << 16)]:
+            np_t = orc.NP_DTYPE[getattr(orc, dtype_name)]
+            es = np.dtype(np_t).itemsize
+            b = Buffers(rt, l, (n + 8) * es)
+            srcs = make_inputs(orc, dtype_name, size, n, n_teams)
+            for p in range(8):
+                l.fill(l.pe_ptr(b.dst, p), 0x5A, (n + 8) * es)
+            for k, p in enumerate(pes):
+                rt.put_bytes(l.pe_ptr(b.src, p), srcs[k])
+            assert l.wg_reduce_teams(getattr(L, dtype_name), getattr(L, op_name), teams, n_teams,
+                                     l.pe_ptr(b.dst, pes[0]), l.pe_ptr(b.src, pes[0]), n, 256, None) == 0
+            want = orc.to_all(getattr(orc, dtype_name), getattr(orc, op_name), srcs)
+            for p in range(8):
+                got = rt.get_bytes(l.pe_ptr(b.dst, p), (n + 8) * es, np_t)
+                if p in pes:
+                    assert np.array_equal(got[:n].view(np.uint8), want.view(np.uint8)), (dtype_name, n, p)
+                    assert (got[n:].view(np.uint8) == 0x5A).all()
+                else:
+                    assert (got.view(np.uint8) == 0x5A).all()
+            b.free()
+        # the same team twice, or teams over different PEs, are refused
+        if n_teams >= 2:
+            twice = (ctypes.c_void_p * 2)(teams[0], teams[0])
+            assert l.wg_reduce_teams(L.INT, L.SUM, twice, 2, l.pe_ptr(b.src, pes[0]), l.pe_ptr(b.src, pes[0]),
+                                     0, 64, None) == -1
+        for t in range(n_teams):
+            l.team_destroy(teams[t])
+    l.set_pe(0)
+
+
 def test_closed_forms_of_the_reference_tests(rt, L, orc):
     """examples/rocshmem_allreduce_test.cc:49-70 (src[i] = pe + i%9) and
     tests/functional_tests/tester.cpp:147-159 (all ones -> P)."""
