@@ -292,7 +292,11 @@ int rocshmem_amd_fcollectmem(rocshmem_amd_team_t team, void *dest, const void *s
  * rocshmem_P2P_SYNC.hpp, which the reference forwards to MPI one-sided calls
  * on a window over the heap (src/host/host.cpp:162-249).  The typed C++ names
  * (include/rocshmem/rocshmem_HOST.hpp) are inline wrappers over these.  All of
- * them are complete when they return. */
+ * them are complete when they return.  They run on streams of the library's
+ * own and are ordered with each other only — not with work the caller has
+ * queued on HIP streams, which a host call therefore neither waits for nor
+ * holds up (the reference's MPI traffic has no ordering with HIP streams
+ * either): a kernel that is running may be waiting for just this put. */
 
 /* PE a context handle belongs to (rocshmem_ctx_t::ctx_opaque, as filled in by
  * rocshmem_ctx_create or a driver); the acting PE for NULL; -1 if the pointer

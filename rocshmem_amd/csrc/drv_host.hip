@@ -30,20 +30,28 @@ bool device_accessible(const void *p) {
 }
 
 // Pinned block the one-thread atomic kernel reads its operands from and writes
-// its result to, the staging buffer of the polling reads, and their stream.
+// its result to, the staging buffer of the polling reads, and the streams of
+// the host-side operations.  Both streams are non-blocking: the null stream
+// would line every host put, atomic or poll up behind whatever kernel is
+// running on an ordinary stream — and that kernel may be waiting for exactly
+// this operation.
 struct HostSide {
   std::mutex lock;
   uint64_t *args = nullptr;  // [0] pe, [1] value, [2] cond, [3] fetched
   char *staging = nullptr;
   size_t staging_bytes = 0;
-  hipStream_t poll = nullptr;
+  hipStream_t poll = nullptr;  // test / wait_until reads
+  hipStream_t work = nullptr;  // put / get / atomics
 
   void ensure() {
+    std::lock_guard<std::mutex> guard(init_lock);
     if (!args) {
-      DRV_CHECK_HIP(hipHostMalloc(reinterpret_cast<void **>(&args), 64, hipHostMallocDefault));
       DRV_CHECK_HIP(hipStreamCreateWithFlags(&poll, hipStreamNonBlocking));
+      DRV_CHECK_HIP(hipStreamCreateWithFlags(&work, hipStreamNonBlocking));
+      DRV_CHECK_HIP(hipHostMalloc(reinterpret_cast<void **>(&args), 64, hipHostMallocDefault));
     }
   }
+  std::mutex init_lock;
   char *stage(size_t bytes) {
     if (bytes > staging_bytes) {
       if (staging) DRV_CHECK_HIP(hipHostFree(staging));
@@ -115,13 +123,14 @@ int rocshmem_amd_host_putmem(void *dest, const void *source, size_t nbytes, int 
   auto &r = runtime::rt();
   char *target = static_cast<char *>(dest) +
                  static_cast<int64_t>(pe - my_pe) * static_cast<int64_t>(r.pe_stride);
+  g_host.ensure();
   if (device_accessible(source)) {
     if (!local_ok(source, nbytes)) return -1;
-    launch_bulk(target, static_cast<const char *>(source), nbytes, nullptr);
-    DRV_CHECK_HIP(hipStreamSynchronize(nullptr));
+    launch_bulk(target, static_cast<const char *>(source), nbytes, g_host.work);
   } else {
-    DRV_CHECK_HIP(hipMemcpy(target, source, nbytes, hipMemcpyHostToDevice));
+    DRV_CHECK_HIP(hipMemcpyAsync(target, source, nbytes, hipMemcpyHostToDevice, g_host.work));
   }
+  DRV_CHECK_HIP(hipStreamSynchronize(g_host.work));
   return 0;
 }
 
@@ -132,13 +141,14 @@ int rocshmem_amd_host_getmem(void *dest, const void *source, size_t nbytes, int 
   auto &r = runtime::rt();
   const char *origin = static_cast<const char *>(source) +
                        static_cast<int64_t>(pe - my_pe) * static_cast<int64_t>(r.pe_stride);
+  g_host.ensure();
   if (device_accessible(dest)) {
     if (!local_ok(dest, nbytes)) return -1;
-    launch_bulk(static_cast<char *>(dest), origin, nbytes, nullptr);
-    DRV_CHECK_HIP(hipStreamSynchronize(nullptr));
+    launch_bulk(static_cast<char *>(dest), origin, nbytes, g_host.work);
   } else {
-    DRV_CHECK_HIP(hipMemcpy(dest, origin, nbytes, hipMemcpyDeviceToHost));
+    DRV_CHECK_HIP(hipMemcpyAsync(dest, origin, nbytes, hipMemcpyDeviceToHost, g_host.work));
   }
+  DRV_CHECK_HIP(hipStreamSynchronize(g_host.work));
   return 0;
 }
 
@@ -148,8 +158,8 @@ int rocshmem_amd_host_amo(int amo_op, int dtype, void *dest, const void *value, 
   const size_t es = dtype_bytes(dtype);
   if (es != 4 && es != 8) return -1;
   if (amo_op == ROCSHMEM_AMD_AMO_COMPARE_SWAP && !cond) return -1;
-  std::lock_guard<std::mutex> guard(g_host.lock);
   g_host.ensure();
+  std::lock_guard<std::mutex> guard(g_host.lock);
   uint64_t *a = g_host.args;
   // One operation of the batched driver: a single "counter" per PE, so the
   // global id of the target is the PE number.
@@ -158,9 +168,9 @@ int rocshmem_amd_host_amo(int amo_op, int dtype, void *dest, const void *value, 
   memcpy(&a[1], value, es);
   if (cond) memcpy(&a[2], cond, es);
   const int rc = rocshmem_amd_amo(amo_op, dtype, dest, 1, reinterpret_cast<const uint32_t *>(&a[0]),
-                                  &a[1], &a[2], &a[3], 1, my_pe, 1, 1, nullptr);
+                                  &a[1], &a[2], &a[3], 1, my_pe, 1, 1, g_host.work);
   if (rc != 0) return rc;
-  DRV_CHECK_HIP(hipStreamSynchronize(nullptr));
+  DRV_CHECK_HIP(hipStreamSynchronize(g_host.work));
   if (fetched) memcpy(fetched, &a[3], es);
   return 0;
 }
@@ -169,8 +179,8 @@ int rocshmem_amd_host_peek(void *dst_host, const void *src_dev, size_t nbytes) {
   if (!runtime::rt().live || !dst_host || !src_dev) return -1;
   if (!nbytes) return 0;
   if (!local_ok(src_dev, nbytes)) return -1;
-  std::lock_guard<std::mutex> guard(g_host.lock);
   g_host.ensure();
+  std::lock_guard<std::mutex> guard(g_host.lock);
   char *stage = g_host.stage(nbytes);
   DRV_CHECK_HIP(hipMemcpyAsync(stage, src_dev, nbytes, hipMemcpyDeviceToHost, g_host.poll));
   DRV_CHECK_HIP(hipStreamSynchronize(g_host.poll));

@@ -43,6 +43,7 @@ def test_host_put_get_every_size_and_alignment(rt, L, orc, local):
         me, pe = (n % P), ((n * 3 + 1) % P)
         landing = l.pe_ptr(sym, pe) + GUARD + doff
         l.fill(landing - GUARD, 0xA5, n + 2 * GUARD)
+        l.stream_sync(None)  # host put/get are not ordered with work queued on HIP streams
         src = (dev + soff) if dev else (host.ctypes.data + soff)
         assert l.host_putmem(l.pe_ptr(sym, me) + GUARD + doff, src, n, me, pe) == 0
         got = rt.get_bytes(landing - GUARD, n + 2 * GUARD)
@@ -52,6 +53,7 @@ def test_host_put_get_every_size_and_alignment(rt, L, orc, local):
         # and back through get, into a guarded local buffer
         if dev:
             l.fill(back_dev, 0x5A, size + 32)
+            l.stream_sync(None)
             assert l.host_getmem(back_dev + 1, l.pe_ptr(sym, me) + GUARD + doff, n, me, pe) == 0
             back = rt.get_bytes(back_dev, n + 2)
         else:
@@ -246,6 +248,7 @@ def test_host_waits_are_released_by_a_later_put(rt, L, fn):
     sym = l.malloc(4 * 8)
     mine = l.pe_ptr(sym, 3)
     l.fill(mine, 0, 32)
+    l.stream_sync(None)
     seven = one(np.int64, 7)
 
     def release():
