@@ -336,6 +336,23 @@ def pingpong_config(b):
     return res
 
 
+def barrier_config(b):
+    """One work-group per PE, P=8: rounds of (store to the next PE, barrier,
+    read the received word).  Per-round time from two launches that differ
+    only in the number of rounds."""
+    l, L = b.l, b.L
+    scratch = l.malloc(8)
+    res = {}
+    for name, fn in (("barrier_all", L.BARRIER_ALL), ("sync_all", L.SYNC_ALL), ("team_sync", L.TEAM_SYNC)):
+        ms = {}
+        for rounds in (200, 2200):
+            assert l.fill_every_pe(scratch, 0, 8, None) == 0
+            ms[rounds] = b.time_ms(lambda: l.wg_sync(fn, l.team_world(), scratch, rounds, 64, None), 3, 1)
+        res[name + "_round_us"] = round((ms[2200] - ms[200]) / 2000 * 1e3, 3)
+    l.free(scratch)
+    return res
+
+
 def cpu_baseline():
     """The oracle's threaded routines on this host's cores, bounded samples.
     (The only place outside tests/ and smoke() that touches oracle/.)"""
@@ -409,6 +426,7 @@ def main():
         allc["alltoall_512x7168_bf16"] = alltoall_config(b, a.steps)
         allc["atomic_fetch_add_16Mi"] = amo_config(b, a.steps)
         allc["pingpong"] = pingpong_config(b)
+        allc["barrier_P8"] = barrier_config(b)
     allc["putmem_curve"] = head["curve"]
     allc["putmem_wg_64KiB_tiles_256MiB"] = head["tiled"]
     b.l.finalize()
