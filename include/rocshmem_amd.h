@@ -435,6 +435,14 @@ int rocshmem_amd_wait_test_woken(int wait_fn, int dtype, void *ivars, size_t nel
                                  uint64_t delay_ticks, size_t *ret_out,
                                  size_t *indices_out);
 
+/* A device-side wait with an end, for checking that something the HOST does
+ * while a kernel runs reaches that kernel: one thread polls
+ * rocshmem_<T>_test(ivar, cmp, value) (rocshmem_P2P_SYNC.hpp) up to max_polls
+ * times.  Only enqueues.  result_dev (device memory, 2 x uint64): [0] = 1 if
+ * the condition was seen, 0 if the polls ran out; [1] = polls made. */
+int rocshmem_amd_poll_until(int dtype, void *ivar, int cmp, const void *value, uint64_t max_polls,
+                            uint64_t *result_dev, rocshmem_amd_stream_t stream);
+
 /* Context lifecycle (rocshmem.hpp:334-370; src/rocshmem_gpu.cpp:286-325): each
  * of n_wgs work-groups creates per_wg contexts (rocshmem_wg_ctx_create, or
  * rocshmem_wg_team_create_ctx when team != NULL), records each return code in

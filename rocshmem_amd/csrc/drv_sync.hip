@@ -439,6 +439,24 @@ DRV_WAIT(unsigned int, uint)
 DRV_WAIT(unsigned long, ulong)
 DRV_WAIT(unsigned long long, ulonglong)
 
+// A wait with an end: rocshmem_<T>_test polled up to max_polls times.
+template <typename T>
+__global__ void poll_until_kernel(T *ivar, int cmp, T value, unsigned long long max_polls,
+                                  unsigned long long *result) {
+  unsigned long long polls = 0;
+  int seen = 0;
+  while (polls < max_polls) {
+    ++polls;
+    if (PublicWait<T>::test(ivar, cmp, value)) {
+      seen = 1;
+      break;
+    }
+    __builtin_amdgcn_s_sleep(8);
+  }
+  result[0] = static_cast<unsigned long long>(seen);
+  result[1] = polls;
+}
+
 template <typename T>
 struct WaitArgs {
   int fn;
@@ -858,6 +876,22 @@ int rocshmem_amd_wait_test_woken(int wait_fn, int dtype, void *ivars, size_t nel
                      delay_ticks, ret_out, indices_out);
   });
   return known ? rc : -1;
+}
+
+int rocshmem_amd_poll_until(int dtype, void *ivar, int cmp, const void *value, uint64_t max_polls,
+                            uint64_t *result_dev, rocshmem_amd_stream_t stream) {
+  if (!runtime::rt().live || !ivar || !value || !result_dev || !max_polls) return -1;
+  if (!local_ok(ivar, 8) || !local_ok(result_dev, 16)) return -1;
+  hipStream_t s = as_stream(stream);
+  const bool known = for_wait_dtype(dtype, [&](auto *tag) {
+    using T = typename std::remove_pointer<decltype(tag)>::type;
+    hipLaunchKernelGGL(poll_until_kernel<T>, dim3(1), dim3(1), 0, s, static_cast<T *>(ivar), cmp,
+                       *static_cast<const T *>(value), static_cast<unsigned long long>(max_polls),
+                       reinterpret_cast<unsigned long long *>(result_dev));
+  });
+  if (!known) return -1;
+  DRV_CHECK_HIP(hipGetLastError());
+  return 0;
 }
 
 int rocshmem_amd_ctx_cycle(rocshmem_amd_team_t team, int n_wgs, int wg_size, int per_wg,

@@ -103,6 +103,7 @@ SIGNATURES = {
     "rocshmem_amd_wait_test": (_i, [_i, _i, _vp, _sz, _vp, _i, _vp, C.POINTER(_sz), _vp]),
     "rocshmem_amd_wait_test_woken": (_i, [_i, _i, _vp, _sz, _vp, _i, _vp, _sz, _vp, _u64,
                                           C.POINTER(_sz), _vp]),
+    "rocshmem_amd_poll_until": (_i, [_i, _vp, _i, _vp, _u64, _vp, _vp]),
     "rocshmem_amd_ctx_cycle": (_i, [_vp, _i, _i, _i, _vp, _vp, _vp]),
 }
 

@@ -275,6 +275,36 @@ def test_host_waits_are_released_by_a_later_put(rt, L, fn):
     l.free(sym)
 
 
+@pytest.mark.parametrize("how", ["put", "atomic"])
+def test_host_put_reaches_a_kernel_that_is_already_waiting(rt, L, how):
+    """A kernel polls rocshmem_long_test on its PE's word (bounded: it gives up
+    after a few seconds); while it runs, the host, acting for another PE, puts
+    or atomically sets the value.  The host call must neither wait for the
+    kernel nor be invisible to it: the kernel reports that it saw the value,
+    after a number of polls that shows it was really waiting."""
+    l = rt.up(P, HEAP)
+    sym = l.malloc(8)
+    l.fill(l.pe_ptr(sym, 2), 0, 8)
+    res = l.dev_alloc(16)
+    l.fill(res, 0xFF, 16)
+    l.stream_sync(None)
+    seven = one(np.int64, 7)
+    assert l.poll_until(L.LONG, l.pe_ptr(sym, 2), L.CMP_EQ, seven.ctypes.data, 4_000_000, res, None) == 0
+    time.sleep(0.05)
+    t0 = time.time()
+    if how == "put":
+        assert l.host_putmem(l.pe_ptr(sym, 5), seven.ctypes.data, 8, 5, 2) == 0
+    else:
+        assert l.host_amo(L.AMO_SET, L.LONG, l.pe_ptr(sym, 5), seven.ctypes.data, None, 5, 2, None) == 0
+    host_call_s = time.time() - t0
+    l.stream_sync(None)
+    seen, polls = (int(x) for x in rt.get_bytes(res, 16, np.uint64))
+    assert seen == 1 and polls > 1000, (seen, polls)
+    assert host_call_s < 2.0, host_call_s
+    l.dev_free(res)
+    l.free(sym)
+
+
 def test_host_wait_argument_errors(rt, L):
     l = rt.up(P, HEAP)
     iv = l.malloc(64)
