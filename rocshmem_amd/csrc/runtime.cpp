@@ -494,6 +494,18 @@ __host__ void rocshmem_init(MPI_Comm) {
   WorldMeeting w;
   if (w.mine) {
     rt().init(runtime::pe_threads_count(), 0);
+    // Kernels of different PE threads that wait for each other must not share
+    // a hardware queue; HIP hands its queues (4 unless GPU_MAX_HW_QUEUES says
+    // otherwise) to streams in turn.
+    const int n = runtime::pe_threads_count();
+    const size_t queues = runtime::env_size("GPU_MAX_HW_QUEUES", 4);
+    if (n > 1 && queues < static_cast<size_t>(n) + 1)
+      fprintf(stderr,
+              "rocshmem: %d PE threads but GPU_MAX_HW_QUEUES=%zu: kernels of different PEs that "
+              "wait for each other can end up in one hardware queue and never finish; set "
+              "GPU_MAX_HW_QUEUES to at least the number of streams in use (PEs x streams per PE "
+              "+ 1)\n",
+              n, queues);
     w.done();
   }
   // A program built with -fgpu-default-stream=per-thread launches its
