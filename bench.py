@@ -137,6 +137,14 @@ def headline(b, steps, warmup):
         point["getmem_all_cus_gbs"] = round(2 * m / tget / 1e6, 3)
         curve[str(m)] = point
     out["curve"] = curve
+    # One-directional ceilings of the memory system, same buffers and rotation:
+    # a copy that reads N and writes N cannot beat 2 / (1/read + 1/write).
+    t_rd = b.time_ms(rotating(lambda me, pe: l.hbm_probe(0, srcs[me], n, None)), steps, warmup)
+    t_wr = b.time_ms(rotating(lambda me, pe: l.hbm_probe(1, dsts[pe], n, None)), steps, warmup)
+    rd, wr = n / t_rd / 1e6, n / t_wr / 1e6
+    out["ceilings"] = {"read_only_gbs": round(rd, 1), "write_only_gbs": round(wr, 1),
+                       "copy_bound_gbs": round(2 / (1 / rd + 1 / wr), 1),
+                       "copy_over_bound": round(out["gbs"] / (2 / (1 / rd + 1 / wr)), 4)}
     # Device API from every CU: rocshmem_ctx_putmem_wg on 64 KiB tiles, one
     # quiet per work-group, through a default and a NOSTORE context.
     tiled = {}
@@ -428,6 +436,7 @@ def main():
         allc["pingpong"] = pingpong_config(b)
         allc["barrier_P8"] = barrier_config(b)
     allc["putmem_curve"] = head["curve"]
+    allc["hbm_one_direction_256MiB"] = head["ceilings"]
     allc["putmem_wg_64KiB_tiles_256MiB"] = head["tiled"]
     b.l.finalize()
     cpu = None if (a.quick or a.no_cpu) else cpu_baseline()

@@ -108,6 +108,27 @@ void launch_bulk(char *dst, const char *src, size_t nbytes, hipStream_t stream) 
   DRV_CHECK_HIP(hipGetLastError());
 }
 
+// What the memory system sustains in one direction only, with the copy
+// kernel's shape (512 lanes, two 16-byte vectors per lane, non-temporal):
+// the yardstick the copy is read against.
+typedef unsigned int probe_u32x4 __attribute__((ext_vector_type(4)));
+__global__ void probe_read_kernel(const probe_u32x4 *src, size_t nvec, unsigned *sink) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * 1024 + threadIdx.x;
+  if (i + 512 >= nvec) return;
+  const probe_u32x4 a = __builtin_nontemporal_load(src + i);
+  const probe_u32x4 b = __builtin_nontemporal_load(src + i + 512);
+  const unsigned x = a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w;
+  if (x == 0x9e3779b9u) *sink = x;  // keeps the loads alive; practically never taken
+}
+__global__ void probe_write_kernel(probe_u32x4 *dst, size_t nvec) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * 1024 + threadIdx.x;
+  if (i + 512 >= nvec) return;
+  const probe_u32x4 v = {1u, 2u, 3u, static_cast<unsigned>(i)};
+  const probe_u32x4 w = {1u, 2u, 3u, static_cast<unsigned>(i + 512)};
+  __builtin_nontemporal_store(v, dst + i);
+  __builtin_nontemporal_store(w, dst + i + 512);
+}
+
 // The same byte range of every PE's slice set to one value: blockIdx.y is the PE.
 __global__ void fill_every_pe_kernel(char *base, uint64_t pe_stride, size_t nbytes, int byte) {
   char *p = base + static_cast<uint64_t>(blockIdx.y) * pe_stride;
@@ -172,6 +193,24 @@ int rocshmem_amd_rma(int rma_op, int gran, void *dest, const void *source, size_
   RMA_CASE(ROCSHMEM_AMD_GET, ROCSHMEM_AMD_WAVE)
   RMA_CASE(ROCSHMEM_AMD_GET, ROCSHMEM_AMD_WG)
 #undef RMA_CASE
+  DRV_CHECK_HIP(hipGetLastError());
+  return 0;
+}
+
+int rocshmem_amd_hbm_probe(int write, void *buf, size_t nbytes, rocshmem_amd_stream_t stream) {
+  if (!runtime::rt().live || !buf || nbytes < (1u << 20) || (reinterpret_cast<uintptr_t>(buf) & 15u))
+    return -1;
+  if (!local_ok(buf, nbytes)) return -1;
+  static unsigned *sink = nullptr;
+  if (!sink) DRV_CHECK_HIP(hipMalloc(&sink, sizeof(unsigned)));
+  const size_t nvec = nbytes / 16;
+  const unsigned grid = static_cast<unsigned>((nvec + 1023) / 1024);
+  if (write)
+    hipLaunchKernelGGL(probe_write_kernel, dim3(grid), dim3(512), 0, as_stream(stream),
+                       static_cast<probe_u32x4 *>(buf), nvec);
+  else
+    hipLaunchKernelGGL(probe_read_kernel, dim3(grid), dim3(512), 0, as_stream(stream),
+                       static_cast<const probe_u32x4 *>(buf), nvec, sink);
   DRV_CHECK_HIP(hipGetLastError());
   return 0;
 }

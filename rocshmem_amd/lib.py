@@ -61,6 +61,7 @@ SIGNATURES = {
     "rocshmem_amd_copy_in": (_i, [_vp, _vp, _sz]),
     "rocshmem_amd_copy_out": (_i, [_vp, _vp, _sz]),
     "rocshmem_amd_fill": (_i, [_vp, _i, _sz]),
+    "rocshmem_amd_hbm_probe": (_i, [_i, _vp, _sz, _vp]),
     "rocshmem_amd_fill_every_pe": (_i, [_vp, _i, _sz, _vp]),
     "rocshmem_amd_copy_dev": (_i, [_vp, _vp, _sz]),
     "rocshmem_amd_stream_sync": (_i, [_vp]),
