@@ -462,6 +462,9 @@ def main():
                      # FETCH_SIZE + WRITE_SIZE per launch under rocprofv3 --pmc, scaled by the
                      # HIP runtime's own copy kernel (profiles/bulk_copy_256MiB_hbm_traffic.txt)
                      "traffic": 536896718, "kernel": "bulk_copy_kernel<true>",
+                     # measured in this run: what a pure read / pure write stream of the
+                     # same shape sustains, and the copy rate those two allow
+                     "measured_ceilings": head["ceilings"],
                      "algorithmic_bytes_per_launch": head["bytes_per_step"]},
         # the reference's own convention (tests/functional_tests/tester.cpp:505-508):
         # payload bytes per second in GiB/s, counting each byte once
