@@ -203,19 +203,32 @@ def to_all_configs(b, steps, warmup):
 
 
 def alltoall_config(b, steps):
-    """configs[4] part 1: alltoall, 512 tokens x 7168 bf16 per PE pair."""
+    """configs[4] part 1: alltoall, 512 tokens x 7168 bf16 per PE pair; fcollect
+    and broadcast of the same block beside it."""
     l = b.l
     blk = 512 * 7168 * 2
     src, dst = l.malloc(P * blk), l.malloc(P * blk)
     assert src and dst
     for p in range(P):
         b.fill_random(l.pe_ptr(src, p), P * blk, p, 30 + p)
-    ms = b.time_ms(lambda: l.alltoallmem(l.team_world(), dst, src, blk, None), max(5, steps // 5), 3)
-    alg = 2 * P * P * blk
+    n = max(5, steps // 5)
+
+    def entry(ms, alg):
+        return {"ms": round(ms, 4), "gbs": round(alg / ms / 1e6, 1),
+                "frac": round(alg / ms / 1e6 / HBM_PEAK_GBS, 4)}
+
+    res = entry(b.time_ms(lambda: l.alltoallmem(l.team_world(), dst, src, blk, None), n, 3),
+                2 * P * P * blk)
+    # every block is read once and written P times (P-1 for the broadcast)
+    res["fcollect_same_block"] = entry(
+        b.time_ms(lambda: l.fcollectmem(l.team_world(), dst, src, blk, None), n, 3),
+        (P + P * P) * blk)
+    res["broadcast_P_blocks_from_pe0"] = entry(
+        b.time_ms(lambda: l.broadcastmem(l.team_world(), dst, src, P * blk, 0, None), n, 3),
+        P * P * blk)
     l.free(src)
     l.free(dst)
-    return {"ms": round(ms, 4), "gbs": round(alg / ms / 1e6, 1),
-            "frac": round(alg / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    return res
 
 
 def zipf_table(K, s):
@@ -461,7 +474,7 @@ def main():
                      "unit": "GB/s", "frac": round(head["gbs"] / HBM_PEAK_GBS, 4),
                      # FETCH_SIZE + WRITE_SIZE per launch under rocprofv3 --pmc, scaled by the
                      # HIP runtime's own copy kernel (profiles/bulk_copy_256MiB_hbm_traffic.txt)
-                     "traffic": 536896718, "kernel": "bulk_copy_kernel<true>",
+                     "traffic": 536870724, "kernel": "bulk_copy_kernel<true>",
                      # measured in this run: what a pure read / pure write stream of the
                      # same shape sustains, and the copy rate those two allow
                      "measured_ceilings": head["ceilings"],

@@ -186,8 +186,9 @@ int rocshmem_amd_copy_out(void *dst_host, const void *src_dev, size_t n);
 int rocshmem_amd_fill(void *dst_dev, int byte, size_t n);
 /* Measurement aid (no reference counterpart): reads (write == 0) or overwrites
  * (write != 0) nbytes (>= 1 MiB, 16-byte aligned) of device memory with the
- * whole GPU, in the launch shape of the bulk copy, and nothing else — the
- * one-directional rate of the memory system that a copy is judged against. */
+ * whole GPU, with the load and store instructions of the bulk copy, and nothing
+ * else — the one-directional rate of the memory system that a copy is judged
+ * against. */
 int rocshmem_amd_hbm_probe(int write, void *buf, size_t nbytes, rocshmem_amd_stream_t stream);
 /* The symmetric object `sym` (address on PE 0) set to `byte` on every PE with
  * one launch on `stream` — e.g. signal words cleared between dispatches. */

@@ -245,8 +245,8 @@ void launch_grid_reduce(void *dst0, const void *src0, int64_t hop, int np, size_
   DRV_CHECK_HIP(hipGetLastError());
 }
 
-// Whole-GPU alltoall / broadcast / fcollect: the P*P (or P) blocks are cut
-// into spans, and work-groups walk the list of all spans.
+// Whole-GPU alltoall / broadcast / fcollect.  One wavefront per work-group,
+// 1 KiB per work-group, as in the whole-GPU copy.
 struct GridMoveArgs {
   char *dest0;        // buffers on the first member
   const char *src0;
@@ -257,49 +257,84 @@ struct GridMoveArgs {
   size_t span;
 };
 
-template <int kMove, bool kNonTemporal>
-__global__ void grid_move_kernel(GridMoveArgs a) {
-  const size_t spans_per_block = (a.nbytes + a.span - 1) / a.span;
-  const size_t nblocks = kMove == MOVE_BROADCAST ? static_cast<size_t>(a.np)
-                                                 : static_cast<size_t>(a.np) * a.np;
-  const size_t total = nblocks * spans_per_block;
-  for (size_t s = blockIdx.x; s < total; s += gridDim.x) {
-    const size_t blk = s / spans_per_block;
-    const size_t off = (s % spans_per_block) * a.span;
+// alltoall: blockIdx.y names the block (sender, receiver), blockIdx.x walks
+// its spans.  Every byte is read once and written once.
+template <bool kNonTemporal>
+__global__ void grid_alltoall_kernel(GridMoveArgs a) {
+  const int i = static_cast<int>(blockIdx.y / a.np);  // sender
+  const int j = static_cast<int>(blockIdx.y % a.np);  // receiver
+  char *d = a.dest0 + j * a.hop + static_cast<size_t>(i) * a.nbytes;
+  const char *src = a.src0 + i * a.hop + static_cast<size_t>(j) * a.nbytes;
+  for (size_t off = blockIdx.x * a.span; off < a.nbytes; off += gridDim.x * a.span) {
     const size_t len = a.nbytes - off < a.span ? a.nbytes - off : a.span;
-    char *d;
-    const char *src;
-    if constexpr (kMove == MOVE_BROADCAST) {
-      const int j = static_cast<int>(blk);
-      if (j == a.root) continue;
-      d = a.dest0 + j * a.hop + off;
-      src = a.src0 + a.root * a.hop + off;
-    } else {
-      const int i = static_cast<int>(blk / a.np);  // sender
-      const int j = static_cast<int>(blk % a.np);  // receiver
-      d = a.dest0 + j * a.hop + static_cast<size_t>(i) * a.nbytes + off;
-      src = a.src0 + i * a.hop + (kMove == MOVE_ALLTOALL ? static_cast<size_t>(j) * a.nbytes : 0) + off;
-    }
-    detail::copy_lanes_impl<2, kNonTemporal>(d, src, len, threadIdx.x, blockDim.x);
+    detail::copy_lanes_impl<2, kNonTemporal>(d + off, src + off, len, threadIdx.x, blockDim.x);
   }
 }
+
+// broadcast / fcollect: a block goes to every member, so it is read once and
+// the registers are stored P (or P-1) times; the kernel is a pure write stream
+// with 1/P of its traffic in reads.  blockIdx.y names the sender.  All
+// receivers share the destination's alignment (the hop is a multiple of 16),
+// so one peel serves them all.
+template <int kMove, bool kNonTemporal>
+__global__ void grid_fanout_kernel(GridMoveArgs a) {
+  const int i = kMove == MOVE_BROADCAST ? a.root : static_cast<int>(blockIdx.y);
+  const int skip = kMove == MOVE_BROADCAST ? a.root : -1;
+  char *d = a.dest0 + (kMove == MOVE_FCOLLECT ? static_cast<size_t>(i) * a.nbytes : 0);
+  const char *s = a.src0 + i * a.hop;
+  size_t head = (16u - (reinterpret_cast<uintptr_t>(d) & 15u)) & 15u;
+  if (head > a.nbytes) head = a.nbytes;
+  const size_t body = a.nbytes - head;
+  const size_t nvec = body >> 4;
+  if (blockIdx.x == 0) {
+    const size_t tail = body & 15u, done = head + (nvec << 4);
+    for (int j = 0; j < a.np; ++j) {
+      if (j == skip) continue;
+      char *dj = d + j * a.hop;
+      if (threadIdx.x < head) dj[threadIdx.x] = s[threadIdx.x];
+      if (threadIdx.x < tail) dj[done + threadIdx.x] = s[done + threadIdx.x];
+    }
+  }
+  d += head;
+  s += head;
+  const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (size_t first = static_cast<size_t>(blockIdx.x) * blockDim.x; first < nvec; first += stride) {
+    const size_t v = first + threadIdx.x;
+    const size_t left = nvec - first;
+    const size_t bytes = (left < blockDim.x ? left : blockDim.x) << 4;
+    detail::u32x4 val{};
+    if (v < nvec) val = detail::load16<kNonTemporal>(s + (v << 4));
+    for (int j = 0; j < a.np; ++j) {
+      if (j == skip) continue;
+      const __amdgpu_buffer_rsrc_t w = detail::window_of(d + j * a.hop + (first << 4), bytes);
+      if (v < nvec)
+        detail::store16<kNonTemporal>(w, static_cast<uint32_t>(threadIdx.x << 4), val);
+    }
+  }
+}
+
+constexpr int kMoveThreads = 64;
+constexpr size_t kMoveMaxWgs = size_t{1} << 22;
 
 template <int kMove>
 void launch_grid_move(char *dest0, const char *src0, int64_t hop, int np, int root,
                       size_t nbytes, hipStream_t stream) {
   if (!nbytes) return;
-  GridMoveArgs a{dest0, src0, hop, np, root, nbytes, 0};
-  // Same shape as the whole-GPU copy: 16 KiB spans, 512 lanes.
-  a.span = nbytes <= (16u << 10) ? nbytes : (16u << 10);
-  const size_t spans_per_block = (nbytes + a.span - 1) / a.span;
-  const size_t nblocks = kMove == MOVE_BROADCAST ? np : static_cast<size_t>(np) * np;
-  const size_t total = nblocks * spans_per_block;
-  const size_t max_wgs = size_t{1} << 20;
-  const int grid = static_cast<int>(total < max_wgs ? total : max_wgs);
-  if (nbytes >= runtime::rt().state.nt_bytes)
-    hipLaunchKernelGGL((grid_move_kernel<kMove, true>), dim3(grid), dim3(512), 0, stream, a);
-  else
-    hipLaunchKernelGGL((grid_move_kernel<kMove, false>), dim3(grid), dim3(512), 0, stream, a);
+  GridMoveArgs a{dest0, src0, hop, np, root, nbytes, size_t{kMoveThreads} * 16};
+  const bool nt = nbytes >= runtime::rt().state.nt_bytes;
+  const size_t rows = kMove == MOVE_ALLTOALL ? static_cast<size_t>(np) * np
+                    : kMove == MOVE_FCOLLECT ? static_cast<size_t>(np) : 1;
+  const size_t spans = (nbytes + a.span - 1) / a.span;
+  const size_t max_x = kMoveMaxWgs / rows;
+  const dim3 grid(static_cast<unsigned>(spans < max_x ? spans : max_x), static_cast<unsigned>(rows));
+  const dim3 block(kMoveThreads);
+  if constexpr (kMove == MOVE_ALLTOALL) {
+    if (nt) hipLaunchKernelGGL(grid_alltoall_kernel<true>, grid, block, 0, stream, a);
+    else hipLaunchKernelGGL(grid_alltoall_kernel<false>, grid, block, 0, stream, a);
+  } else {
+    if (nt) hipLaunchKernelGGL((grid_fanout_kernel<kMove, true>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((grid_fanout_kernel<kMove, false>), grid, block, 0, stream, a);
+  }
   DRV_CHECK_HIP(hipGetLastError());
 }
 

@@ -61,46 +61,55 @@ __global__ void rma_kernel(RmaArgs a) {
 }
 
 // Whole-GPU copy: every thread of the grid is one lane of a single
-// cooperative copy.  Work-groups are handed contiguous spans so each one
-// streams through its own DRAM pages.
+// cooperative copy; consecutive work-groups take consecutive 1 KiB pieces.
 struct BulkArgs {
   char *dst;
   const char *src;
   size_t nbytes;
-  size_t span;  // bytes per work-group span, multiple of 16 after the head
 };
 
+// One wavefront per work-group, one 16-byte vector per lane: each work-group
+// moves 1 KiB and leaves.  The destination is peeled to 16-byte alignment by
+// block 0 (head and tail bytes); the source may sit at any byte offset.
 template <bool kNonTemporal>
 __global__ void bulk_copy_kernel(BulkArgs a) {
-  // Head bytes up to the first 16-byte boundary of dst are moved by block 0.
   size_t head = (16u - (reinterpret_cast<uintptr_t>(a.dst) & 15u)) & 15u;
   if (head > a.nbytes) head = a.nbytes;
-  if (blockIdx.x == 0 && threadIdx.x < head) a.dst[threadIdx.x] = a.src[threadIdx.x];
   const size_t body = a.nbytes - head;
-  const size_t nspans = (body + a.span - 1) / a.span;
-  for (size_t s = blockIdx.x; s < nspans; s += gridDim.x) {
-    const size_t off = head + s * a.span;
-    const size_t len = a.nbytes - off < a.span ? a.nbytes - off : a.span;
-    detail::copy_lanes_impl<2, kNonTemporal>(a.dst + off, a.src + off, len, threadIdx.x,
-                                             blockDim.x);
+  const size_t nvec = body >> 4;
+  if (blockIdx.x == 0) {
+    const size_t tail = body & 15u, done = head + (nvec << 4);
+    if (threadIdx.x < head) a.dst[threadIdx.x] = a.src[threadIdx.x];
+    if (threadIdx.x < tail) a.dst[done + threadIdx.x] = a.src[done + threadIdx.x];
+  }
+  char *d = a.dst + head;
+  const char *s = a.src + head;
+  const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (size_t first = static_cast<size_t>(blockIdx.x) * blockDim.x; first < nvec; first += stride) {
+    const size_t v = first + threadIdx.x;
+    const size_t left = nvec - first;
+    const __amdgpu_buffer_rsrc_t w =
+        detail::window_of(d + (first << 4), (left < blockDim.x ? left : blockDim.x) << 4);
+    if (v < nvec)
+      detail::store16<kNonTemporal>(w, static_cast<uint32_t>(threadIdx.x << 4),
+                                    detail::load16<kNonTemporal>(s + (v << 4)));
   }
 }
 
-// Launch shape of the whole-GPU copy, from a sweep on MI355X with the buffers
-// rotated so nothing is served from the 256 MB memory-side cache: 512 threads
-// moving one 16 KiB span per work-group (two 16-byte vectors per lane) with
-// non-temporal loads and stores sustains 6.4-6.5 TB/s of read+write traffic;
-// 64 KiB spans with 256 threads gave 5.9 TB/s.
-constexpr int kBulkThreads = 512;
-constexpr size_t kBulkSpan = 16u << 10;
-constexpr size_t kBulkMaxWgs = size_t{1} << 20;
+// Launch shape of the whole-GPU copy, from sweeps on MI355X with the buffers
+// rotated so nothing is served from the 256 MB memory-side cache.  With
+// write-through stores the smallest work-group wins: 64 lanes x one vector
+// (1 KiB per work-group) sustains 6.7-6.8 TB/s of read+write traffic, 512
+// lanes x two vectors 6.45, 1024 lanes 6.2 and less.  The same holds for a
+// pure write stream (6.96 TB/s at one vector per lane, 6.2 at two).
+constexpr int kBulkThreads = 64;
+constexpr size_t kBulkMaxWgs = size_t{1} << 22;
 
 void launch_bulk(char *dst, const char *src, size_t nbytes, hipStream_t stream) {
   if (!nbytes) return;
-  BulkArgs a{dst, src, nbytes, 0};
-  a.span = nbytes <= kBulkSpan ? ((nbytes + 15) / 16 * 16) : kBulkSpan;
-  const size_t nspans = (nbytes + a.span - 1) / a.span;
-  const int grid = static_cast<int>(nspans < kBulkMaxWgs ? nspans : kBulkMaxWgs);
+  BulkArgs a{dst, src, nbytes};
+  const size_t wgs = (nbytes / 16 + kBulkThreads - 1) / kBulkThreads;
+  const int grid = static_cast<int>(wgs < kBulkMaxWgs ? (wgs ? wgs : 1) : kBulkMaxWgs);
   if (nbytes >= runtime::rt().state.nt_bytes)
     hipLaunchKernelGGL(bulk_copy_kernel<true>, dim3(grid), dim3(kBulkThreads), 0, stream, a);
   else
@@ -109,24 +118,26 @@ void launch_bulk(char *dst, const char *src, size_t nbytes, hipStream_t stream) 
 }
 
 // What the memory system sustains in one direction only, with the copy
-// kernel's shape (512 lanes, two 16-byte vectors per lane, non-temporal):
-// the yardstick the copy is read against.
-typedef unsigned int probe_u32x4 __attribute__((ext_vector_type(4)));
-__global__ void probe_read_kernel(const probe_u32x4 *src, size_t nvec, unsigned *sink) {
-  const size_t i = static_cast<size_t>(blockIdx.x) * 1024 + threadIdx.x;
-  if (i + 512 >= nvec) return;
-  const probe_u32x4 a = __builtin_nontemporal_load(src + i);
-  const probe_u32x4 b = __builtin_nontemporal_load(src + i + 512);
-  const unsigned x = a.x ^ a.y ^ a.z ^ a.w ^ b.x ^ b.y ^ b.z ^ b.w;
-  if (x == 0x9e3779b9u) *sink = x;  // keeps the loads alive; practically never taken
+// kernel's instructions (one 16-byte vector per lane, non-temporal load,
+// write-through streaming store): the yardstick the copy is read against.
+// 128 lanes per work-group is where both directions peak (6.9 TB/s each); at
+// 64 lanes a one-direction kernel is bound by work-group dispatch (4.7 TB/s).
+constexpr int kProbeThreads = 128;
+__global__ void probe_read_kernel(const char *src, size_t nvec, unsigned *sink) {
+  const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= nvec) return;
+  const detail::u32x4 a = detail::load16<true>(src + (i << 4));
+  const unsigned x = a.x ^ a.y ^ a.z ^ a.w;
+  if (x == 0x9e3779b9u && a.y == 0x7f4a7c15u) *sink = x;  // keeps the load alive; practically never taken
 }
-__global__ void probe_write_kernel(probe_u32x4 *dst, size_t nvec) {
-  const size_t i = static_cast<size_t>(blockIdx.x) * 1024 + threadIdx.x;
-  if (i + 512 >= nvec) return;
-  const probe_u32x4 v = {1u, 2u, 3u, static_cast<unsigned>(i)};
-  const probe_u32x4 w = {1u, 2u, 3u, static_cast<unsigned>(i + 512)};
-  __builtin_nontemporal_store(v, dst + i);
-  __builtin_nontemporal_store(w, dst + i + 512);
+__global__ void probe_write_kernel(char *dst, size_t nvec) {
+  const size_t first = static_cast<size_t>(blockIdx.x) * blockDim.x;
+  const size_t i = first + threadIdx.x;
+  const size_t left = nvec - first;
+  const __amdgpu_buffer_rsrc_t w =
+      detail::window_of(dst + (first << 4), (left < blockDim.x ? left : blockDim.x) << 4);
+  const detail::u32x4 v = {1u, 2u, 3u, static_cast<unsigned>(i)};
+  if (i < nvec) detail::store16<true>(w, static_cast<uint32_t>(threadIdx.x << 4), v);
 }
 
 // The same byte range of every PE's slice set to one value: blockIdx.y is the PE.
@@ -204,13 +215,13 @@ int rocshmem_amd_hbm_probe(int write, void *buf, size_t nbytes, rocshmem_amd_str
   static unsigned *sink = nullptr;
   if (!sink) DRV_CHECK_HIP(hipMalloc(&sink, sizeof(unsigned)));
   const size_t nvec = nbytes / 16;
-  const unsigned grid = static_cast<unsigned>((nvec + 1023) / 1024);
+  const unsigned grid = static_cast<unsigned>((nvec + kProbeThreads - 1) / kProbeThreads);
   if (write)
-    hipLaunchKernelGGL(probe_write_kernel, dim3(grid), dim3(512), 0, as_stream(stream),
-                       static_cast<probe_u32x4 *>(buf), nvec);
+    hipLaunchKernelGGL(probe_write_kernel, dim3(grid), dim3(kProbeThreads), 0, as_stream(stream),
+                       static_cast<char *>(buf), nvec);
   else
-    hipLaunchKernelGGL(probe_read_kernel, dim3(grid), dim3(512), 0, as_stream(stream),
-                       static_cast<const probe_u32x4 *>(buf), nvec, sink);
+    hipLaunchKernelGGL(probe_read_kernel, dim3(grid), dim3(kProbeThreads), 0, as_stream(stream),
+                       static_cast<const char *>(buf), nvec, sink);
   DRV_CHECK_HIP(hipGetLastError());
   return 0;
 }
