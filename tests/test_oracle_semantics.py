@@ -164,7 +164,7 @@ def test_reduce_plan_thresholds(orc):
         edge = 1024 // P
         assert orc.reduce_plan(P, edge)["algo"] == 0
         assert orc.reduce_plan(P, edge + 1)["algo"] == 1
-    # config sizes quoted in the survey: 1 Mi ints on 2 PEs, 64 Mi on 8 PEs
+    # the two benchmark configurations: 1 Mi ints on 2 PEs, 64 Mi on 8 PEs
     p = orc.reduce_plan(2, 1 << 20)
     assert (p["algo"], p["chunk_size"], p["seg_size"], p["n_seg"]) == (1, 512, 1024, 1024)
     p = orc.reduce_plan(8, 1 << 26)
