@@ -48,6 +48,24 @@ __device__ __forceinline__ void getmem(Context *c, void *dest, const void *sourc
   fence_full();
 }
 
+// Non-blocking forms: the call only issues the copy; rocshmem_ctx_quiet (or
+// fence) by the same thread completes it.  The reference's _nbi calls are its
+// blocking ones; here a thread or wavefront that issues many small messages
+// pays for one completion instead of one per message.  A thread-level copy
+// leaves through plain stores, which only a full release makes visible, so on
+// a NOSTORE context (whose quiet does not write the L2 back) the call still
+// completes before it returns.
+__device__ __forceinline__ void putmem_nbi(Context *c, void *dest, const void *source,
+                                           size_t n, int pe) {
+  copy_thread(remote_addr(c, static_cast<char *>(dest), pe), source, n);
+  if (no_store_order(c)) fence_full();
+}
+__device__ __forceinline__ void getmem_nbi(Context *c, void *dest, const void *source,
+                                           size_t n, int pe) {
+  copy_thread(dest, remote_addr(c, static_cast<const char *>(source), pe), n);
+  if (no_store_order(c)) fence_full();
+}
+
 // ---- wavefront granularity (context_ipc_device.cpp:137-164) ---------------
 __device__ __forceinline__ void putmem_wave(Context *c, void *dest, const void *source,
                                             size_t n, int pe) {
@@ -59,6 +77,17 @@ __device__ __forceinline__ void getmem_wave(Context *c, void *dest, const void *
                                             size_t n, int pe) {
   copy_wave(dest, remote_addr(c, static_cast<const char *>(source), pe), n, g_state.nt_bytes);
   fence_full();
+}
+
+// Non-blocking wavefront forms: write-through stores, complete at the calling
+// wavefront's quiet on either kind of context.
+__device__ __forceinline__ void putmem_nbi_wave(Context *c, void *dest, const void *source,
+                                                size_t n, int pe) {
+  copy_wave(remote_addr(c, static_cast<char *>(dest), pe), source, n, g_state.nt_bytes);
+}
+__device__ __forceinline__ void getmem_nbi_wave(Context *c, void *dest, const void *source,
+                                                size_t n, int pe) {
+  copy_wave(dest, remote_addr(c, static_cast<const char *>(source), pe), n, g_state.nt_bytes);
 }
 
 // ---- work-group granularity: copy, then __syncthreads (:109-125) ----------

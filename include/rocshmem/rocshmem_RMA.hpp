@@ -4,7 +4,8 @@
 // Same names, argument order and PE-translation rule as the reference
 // (include/rocshmem/rocshmem_RMA.hpp; src/rocshmem_gpu.cpp:327-451): these
 // calls map a team-relative `pe` through the context's team; zero-length
-// calls do nothing; the _nbi forms complete like the blocking ones.
+// calls do nothing; the _nbi forms return once the copy is issued and complete
+// at the calling thread's rocshmem_ctx_quiet / rocshmem_ctx_fence.
 #ifndef ROCSHMEM_AMD_RMA_HPP_
 #define ROCSHMEM_AMD_RMA_HPP_
 
@@ -30,12 +31,14 @@ __device__ ATTR_NO_INLINE inline void rocshmem_ctx_getmem(rocshmem_ctx_t ctx, vo
 __device__ ATTR_NO_INLINE inline void rocshmem_ctx_putmem_nbi(rocshmem_ctx_t ctx, void *dest,
                                                        const void *source,
                                                        size_t nelems, int pe) {
-  rocshmem_ctx_putmem(ctx, dest, source, nelems, pe);
+  if (nelems == 0) return;
+  detail::putmem_nbi(detail::ctx_of(ctx), dest, source, nelems, detail::translate_pe(ctx, pe));
 }
 __device__ ATTR_NO_INLINE inline void rocshmem_ctx_getmem_nbi(rocshmem_ctx_t ctx, void *dest,
                                                        const void *source,
                                                        size_t nelems, int pe) {
-  rocshmem_ctx_getmem(ctx, dest, source, nelems, pe);
+  if (nelems == 0) return;
+  detail::getmem_nbi(detail::ctx_of(ctx), dest, source, nelems, detail::translate_pe(ctx, pe));
 }
 __device__ ATTR_NO_INLINE inline void rocshmem_putmem(void *dest, const void *source,
                                                size_t nelems, int pe) {
@@ -47,11 +50,11 @@ __device__ ATTR_NO_INLINE inline void rocshmem_getmem(void *dest, const void *so
 }
 __device__ ATTR_NO_INLINE inline void rocshmem_putmem_nbi(void *dest, const void *source,
                                                    size_t nelems, int pe) {
-  rocshmem_putmem(dest, source, nelems, pe);
+  rocshmem_ctx_putmem_nbi(rocshmem_ctx_t{nullptr, nullptr}, dest, source, nelems, pe);
 }
 __device__ ATTR_NO_INLINE inline void rocshmem_getmem_nbi(void *dest, const void *source,
                                                    size_t nelems, int pe) {
-  rocshmem_getmem(dest, source, nelems, pe);
+  rocshmem_ctx_getmem_nbi(rocshmem_ctx_t{nullptr, nullptr}, dest, source, nelems, pe);
 }
 
 #define ROCSHMEM_AMD_TYPED_RMA(T, TN)                                                    \
@@ -65,11 +68,11 @@ __device__ ATTR_NO_INLINE inline void rocshmem_getmem_nbi(void *dest, const void
   }                                                                                      \
   __device__ ATTR_NO_INLINE inline void rocshmem_ctx_##TN##_put_nbi(                     \
       rocshmem_ctx_t ctx, T *dest, const T *source, size_t nelems, int pe) {             \
-    rocshmem_ctx_putmem(ctx, dest, source, nelems * sizeof(T), pe);                      \
+    rocshmem_ctx_putmem_nbi(ctx, dest, source, nelems * sizeof(T), pe);                  \
   }                                                                                      \
   __device__ ATTR_NO_INLINE inline void rocshmem_##TN##_put_nbi(T *dest, const T *source,\
                                                                 size_t nelems, int pe) { \
-    rocshmem_putmem(dest, source, nelems * sizeof(T), pe);                               \
+    rocshmem_putmem_nbi(dest, source, nelems * sizeof(T), pe);                           \
   }                                                                                      \
   __device__ ATTR_NO_INLINE inline void rocshmem_ctx_##TN##_p(rocshmem_ctx_t ctx,        \
                                                               T *dest, T value, int pe) {\
@@ -88,11 +91,11 @@ __device__ ATTR_NO_INLINE inline void rocshmem_getmem_nbi(void *dest, const void
   }                                                                                      \
   __device__ ATTR_NO_INLINE inline void rocshmem_ctx_##TN##_get_nbi(                     \
       rocshmem_ctx_t ctx, T *dest, const T *source, size_t nelems, int pe) {             \
-    rocshmem_ctx_getmem(ctx, dest, source, nelems * sizeof(T), pe);                      \
+    rocshmem_ctx_getmem_nbi(ctx, dest, source, nelems * sizeof(T), pe);                  \
   }                                                                                      \
   __device__ ATTR_NO_INLINE inline void rocshmem_##TN##_get_nbi(T *dest, const T *source,\
                                                                 size_t nelems, int pe) { \
-    rocshmem_getmem(dest, source, nelems * sizeof(T), pe);                               \
+    rocshmem_getmem_nbi(dest, source, nelems * sizeof(T), pe);                           \
   }                                                                                      \
   __device__ ATTR_NO_INLINE inline T rocshmem_ctx_##TN##_g(rocshmem_ctx_t ctx,           \
                                                            const T *source, int pe) {    \

@@ -5,6 +5,9 @@
 // wavefront) must call with identical arguments.  As in the reference
 // (src/rocshmem_gpu.cpp:753-872) `pe` is a world PE here — these calls do not
 // translate through the context's team — and zero-length calls do nothing.
+// The _nbi_wave forms return once the copy is issued and complete at the
+// calling wavefront's quiet; the _nbi_wg forms complete like the blocking ones
+// (a quiet by one thread could not answer for the other wavefronts' stores).
 #ifndef ROCSHMEM_AMD_RMA_X_HPP_
 #define ROCSHMEM_AMD_RMA_X_HPP_
 
@@ -30,11 +33,11 @@ namespace rocshmem {
 ROCSHMEM_AMD_MEM_X(put, _wg, putmem_wg)
 ROCSHMEM_AMD_MEM_X(put, _nbi_wg, putmem_wg)
 ROCSHMEM_AMD_MEM_X(put, _wave, putmem_wave)
-ROCSHMEM_AMD_MEM_X(put, _nbi_wave, putmem_wave)
+ROCSHMEM_AMD_MEM_X(put, _nbi_wave, putmem_nbi_wave)
 ROCSHMEM_AMD_MEM_X(get, _wg, getmem_wg)
 ROCSHMEM_AMD_MEM_X(get, _nbi_wg, getmem_wg)
 ROCSHMEM_AMD_MEM_X(get, _wave, getmem_wave)
-ROCSHMEM_AMD_MEM_X(get, _nbi_wave, getmem_wave)
+ROCSHMEM_AMD_MEM_X(get, _nbi_wave, getmem_nbi_wave)
 #undef ROCSHMEM_AMD_MEM_X
 
 #define ROCSHMEM_AMD_TYPED_X1(T, TN, DIR, SFX)                                            \

@@ -70,7 +70,12 @@ enum rocshmem_amd_granularity {
   ROCSHMEM_AMD_WG = 2      /* rocshmem_putmem_wg / getmem_wg      */
 };
 
-enum rocshmem_amd_rma_op { ROCSHMEM_AMD_PUT = 0, ROCSHMEM_AMD_GET = 1 };
+enum rocshmem_amd_rma_op {
+  ROCSHMEM_AMD_PUT = 0,
+  ROCSHMEM_AMD_GET = 1,
+  ROCSHMEM_AMD_PUT_NBI = 2, /* rocshmem_putmem_nbi[_wave|_wg]: completes at the closing quiet */
+  ROCSHMEM_AMD_GET_NBI = 3
+};
 
 enum rocshmem_amd_amo_op {
   ROCSHMEM_AMD_AMO_FETCH_ADD = 0,
@@ -213,7 +218,10 @@ int rocshmem_amd_timer_destroy(void *timer);
  * nbytes is cut into tiles of tile_bytes (0 = one equal share per group,
  * rounded up to 16 bytes); group g — a work-group, a wavefront or a thread,
  * per `gran` — moves tiles g, g+G, g+2G ... with one API call each.  The whole
- * transfer is repeated `iters` times inside the kernel. */
+ * transfer is repeated `iters` times inside the kernel, which ends with one
+ * rocshmem_ctx_quiet per group.  The _NBI operations issue
+ * rocshmem_ctx_putmem_nbi[_wave|_wg] / getmem_nbi[_wave|_wg]
+ * (rocshmem_RMA.hpp:259-264,640-645) instead, which that quiet completes. */
 int rocshmem_amd_rma(int rma_op, int gran, void *dest, const void *source, size_t nbytes,
                      size_t tile_bytes, int my_pe, int pe, int n_wgs, int wg_size,
                      int iters, rocshmem_amd_stream_t stream);
@@ -380,8 +388,12 @@ int rocshmem_amd_signal_fetch(int gran, const uint64_t *sig_addr, int my_pe,
  * for pe_a, each with a receiver work-group acting for pe_b.  Per round a
  * producer fills a fresh pattern, calls rocshmem_ctx_putmem_wg of nbytes
  * (multiple of 4) into its slot of `data` on pe_b, calls rocshmem_ctx_quiet and
- * then sets its flag on pe_b with a relaxed store — or, with_signal != 0, does
+ * then sets its flag on pe_b with a relaxed store — or, with_signal == 1, does
  * all three with one rocshmem_ctx_putmem_signal_wg (rocshmem_SIG_OP.hpp:128-131);
+ * with_signal == 2 / 3: the message goes out as several
+ * rocshmem_ctx_putmem_nbi_wave calls per wavefront / rocshmem_ctx_putmem_nbi
+ * calls of 12 bytes per thread, every thread calls rocshmem_ctx_quiet, and
+ * thread 0 sets the flag after a work-group barrier;
  * the receiver waits for the flag, compares every word, and acknowledges.  data: pairs*nbytes symmetric bytes,
  * flags: 2*pairs symmetric uint64 (addresses on pe_a).  mismatches_out = words
  * that differed; timed_out_out = 1 if a bounded wait ran out (all work-groups

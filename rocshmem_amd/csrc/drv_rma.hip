@@ -46,13 +46,27 @@ __global__ void rma_kernel(RmaArgs a) {
           rocshmem_ctx_putmem_wave(a.ctx, a.dest + off, a.source + off, len, a.pe);
         else
           rocshmem_ctx_putmem(a.ctx, a.dest + off, a.source + off, len, a.pe);
-      } else {
+      } else if constexpr (kOp == ROCSHMEM_AMD_GET) {
         if constexpr (kGran == ROCSHMEM_AMD_WG)
           rocshmem_ctx_getmem_wg(a.ctx, a.dest + off, a.source + off, len, a.pe);
         else if constexpr (kGran == ROCSHMEM_AMD_WAVE)
           rocshmem_ctx_getmem_wave(a.ctx, a.dest + off, a.source + off, len, a.pe);
         else
           rocshmem_ctx_getmem(a.ctx, a.dest + off, a.source + off, len, a.pe);
+      } else if constexpr (kOp == ROCSHMEM_AMD_PUT_NBI) {
+        if constexpr (kGran == ROCSHMEM_AMD_WG)
+          rocshmem_ctx_putmem_nbi_wg(a.ctx, a.dest + off, a.source + off, len, a.pe);
+        else if constexpr (kGran == ROCSHMEM_AMD_WAVE)
+          rocshmem_ctx_putmem_nbi_wave(a.ctx, a.dest + off, a.source + off, len, a.pe);
+        else
+          rocshmem_ctx_putmem_nbi(a.ctx, a.dest + off, a.source + off, len, a.pe);
+      } else {
+        if constexpr (kGran == ROCSHMEM_AMD_WG)
+          rocshmem_ctx_getmem_nbi_wg(a.ctx, a.dest + off, a.source + off, len, a.pe);
+        else if constexpr (kGran == ROCSHMEM_AMD_WAVE)
+          rocshmem_ctx_getmem_nbi_wave(a.ctx, a.dest + off, a.source + off, len, a.pe);
+        else
+          rocshmem_ctx_getmem_nbi(a.ctx, a.dest + off, a.source + off, len, a.pe);
       }
     }
   }
@@ -173,11 +187,11 @@ int rocshmem_amd_rma(int rma_op, int gran, void *dest, const void *source, size_
                      int iters, rocshmem_amd_stream_t stream) {
   if (!valid_pe(my_pe) || !valid_pe(pe) || !valid_launch(n_wgs, wg_size) || iters < 0)
     return -1;
-  if (rma_op != ROCSHMEM_AMD_PUT && rma_op != ROCSHMEM_AMD_GET) return -1;
+  if (rma_op < ROCSHMEM_AMD_PUT || rma_op > ROCSHMEM_AMD_GET_NBI) return -1;
   if (gran < ROCSHMEM_AMD_THREAD || gran > ROCSHMEM_AMD_WG) return -1;
   // The remote side must be a symmetric address of my_pe; the local side may
   // be any device buffer.
-  if (rma_op == ROCSHMEM_AMD_PUT) {
+  if (rma_op == ROCSHMEM_AMD_PUT || rma_op == ROCSHMEM_AMD_PUT_NBI) {
     if (!sym_ok_on(dest, nbytes, my_pe) || !local_ok(source, nbytes)) return -1;
   } else {
     if (!sym_ok_on(source, nbytes, my_pe) || !local_ok(dest, nbytes)) return -1;
@@ -203,6 +217,12 @@ int rocshmem_amd_rma(int rma_op, int gran, void *dest, const void *source, size_
   RMA_CASE(ROCSHMEM_AMD_GET, ROCSHMEM_AMD_THREAD)
   RMA_CASE(ROCSHMEM_AMD_GET, ROCSHMEM_AMD_WAVE)
   RMA_CASE(ROCSHMEM_AMD_GET, ROCSHMEM_AMD_WG)
+  RMA_CASE(ROCSHMEM_AMD_PUT_NBI, ROCSHMEM_AMD_THREAD)
+  RMA_CASE(ROCSHMEM_AMD_PUT_NBI, ROCSHMEM_AMD_WAVE)
+  RMA_CASE(ROCSHMEM_AMD_PUT_NBI, ROCSHMEM_AMD_WG)
+  RMA_CASE(ROCSHMEM_AMD_GET_NBI, ROCSHMEM_AMD_THREAD)
+  RMA_CASE(ROCSHMEM_AMD_GET_NBI, ROCSHMEM_AMD_WAVE)
+  RMA_CASE(ROCSHMEM_AMD_GET_NBI, ROCSHMEM_AMD_WG)
 #undef RMA_CASE
   DRV_CHECK_HIP(hipGetLastError());
   return 0;

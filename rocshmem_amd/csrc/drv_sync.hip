@@ -279,7 +279,8 @@ struct PutFlagArgs {
   size_t nbytes;         // per pair, multiple of 4
   int rounds;
   int pe_a, pe_b;
-  int with_signal;       // 0: putmem_wg, quiet, relaxed flag store; 1: putmem_signal_wg
+  int with_signal;       // 0: putmem_wg, quiet, relaxed flag store; 1: putmem_signal_wg;
+                         // 2 / 3: putmem_nbi_wave / putmem_nbi pieces, quiet by all, flag
   unsigned spin_limit;
   rocshmem_ctx_t ctx_a;
   unsigned long long *mismatches;
@@ -330,11 +331,33 @@ __global__ void put_flag_kernel(PutFlagArgs a) {
     if (producer) {
       for (size_t i = threadIdx.x; i < nwords; i += blockDim.x) stage[i] = put_flag_word(pair, r, i);
       __syncthreads();
-      if (a.with_signal) {
+      if (a.with_signal == 1) {
         // flag_on_b is pe_b's address; the call wants pe_a's.
         uint64_t *flag_sym = reinterpret_cast<uint64_t *>(reinterpret_cast<char *>(flag_on_b) - a.a_to_b);
         rocshmem_ctx_putmem_signal_wg(a.ctx_a, data, stage, a.nbytes, flag_sym,
                                       static_cast<uint64_t>(r), ROCSHMEM_SIGNAL_SET, a.pe_b);
+      } else if (a.with_signal == 2 || a.with_signal == 3) {
+        // Non-blocking puts in pieces (four per wavefront, or 12 bytes per call
+        // per thread), completed by the quiet of whoever issued them.
+        if (a.with_signal == 2) {
+          const size_t waves = (blockDim.x + 63) / 64, w = threadIdx.x / 64;
+          const size_t piece = ((a.nbytes + waves * 4 - 1) / (waves * 4) + 3) & ~size_t{3};
+          for (size_t k = w; k * piece < a.nbytes; k += waves) {
+            const size_t off = k * piece;
+            const size_t len = a.nbytes - off < piece ? a.nbytes - off : piece;
+            rocshmem_ctx_putmem_nbi_wave(a.ctx_a, data + off, reinterpret_cast<char *>(stage) + off,
+                                         len, a.pe_b);
+          }
+        } else {
+          for (size_t off = threadIdx.x * size_t{12}; off < a.nbytes; off += blockDim.x * size_t{12}) {
+            const size_t len = a.nbytes - off < 12 ? a.nbytes - off : 12;
+            rocshmem_ctx_putmem_nbi(a.ctx_a, data + off, reinterpret_cast<char *>(stage) + off, len,
+                                    a.pe_b);
+          }
+        }
+        rocshmem_ctx_quiet(a.ctx_a);
+        __syncthreads();
+        if (threadIdx.x == 0) detail::store_through(flag_on_b, static_cast<uint64_t>(r));
       } else {
         rocshmem_ctx_putmem_wg(a.ctx_a, data, stage, a.nbytes, a.pe_b);
         if (threadIdx.x == 0) {
@@ -724,7 +747,8 @@ int rocshmem_amd_put_flag_check(void *data, uint64_t *flags, size_t nbytes, int 
                                 rocshmem_amd_stream_t stream) {
   auto &r = runtime::rt();
   if (!valid_pe(pe_a) || !valid_pe(pe_b) || pe_a == pe_b || pairs < 1 || pairs > 128 ||
-      !valid_launch(2 * pairs, wg_size) || rounds < 0 || nbytes == 0 || (nbytes & 3))
+      !valid_launch(2 * pairs, wg_size) || rounds < 0 || nbytes == 0 || (nbytes & 3) ||
+      with_signal < 0 || with_signal > 3)
     return -1;
   const size_t total = nbytes * static_cast<size_t>(pairs);
   if (!sym_ok_on(data, total, pe_a) || !sym_ok_on(flags, 16u * pairs, pe_a)) return -1;
@@ -752,7 +776,7 @@ int rocshmem_amd_put_flag_check(void *data, uint64_t *flags, size_t nbytes, int 
   a.rounds = rounds;
   a.pe_a = pe_a;
   a.pe_b = pe_b;
-  a.with_signal = with_signal != 0;
+  a.with_signal = with_signal;
   a.spin_limit = 1u << 22;
   a.ctx_a = r.driver_ctx_handle(pe_a);
   a.mismatches = d_bad;

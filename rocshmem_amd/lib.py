@@ -11,7 +11,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "librocshmem_amd.so")
  USHORT) = range(14)
 SUM, MAX, MIN, PROD, AND, OR, XOR = range(7)
 THREAD, WAVE, WG = range(3)
-PUT, GET = range(2)
+PUT, GET, PUT_NBI, GET_NBI = range(4)
 (AMO_FETCH_ADD, AMO_ADD, AMO_FETCH_INC, AMO_INC, AMO_COMPARE_SWAP, AMO_FETCH, AMO_SET,
  AMO_SWAP, AMO_FETCH_AND, AMO_FETCH_OR, AMO_FETCH_XOR) = range(11)
 CTX_NOSTORE = 1  # ROCSHMEM_CTX_NOSTORE

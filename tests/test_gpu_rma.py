@@ -31,7 +31,7 @@ def run_case(rt, L, orc, env, op, gran, n, soff, doff, n_wgs, wg_size, my_pe=0, 
     l = env["l"]
     src, dst, host = env["src"], env["dst"], env["host"]
     base = GUARD + 16  # room for the low guard
-    if op == L.PUT:
+    if op in (L.PUT, L.PUT_NBI):
         local = l.pe_ptr(src, my_pe) + soff
         remote_mine = l.pe_ptr(dst, my_pe) + base + doff
         landing = l.pe_ptr(dst, pe) + base + doff
@@ -127,7 +127,28 @@ def test_nostore_context_moves_the_same_bytes(rt, L, orc, env, gran):
         run_case(rt, L, orc, env, L.GET, g, n, 6, 0, n_wgs, wg, tile=tile, ctx_options=L.CTX_NOSTORE)
 
 
-@pytest.mark.parametrize("with_signal", [0, 1])
+@pytest.mark.parametrize("ctx_options", [0, 1])
+@pytest.mark.parametrize("gran", GRANS)
+@pytest.mark.parametrize("op", ["PUT_NBI", "GET_NBI"])
+def test_non_blocking_forms(rt, L, orc, env, op, gran, ctx_options):
+    """rocshmem_putmem_nbi / getmem_nbi and their _wave / _wg forms
+    (rocshmem_RMA.hpp:259-264,640-645): many calls per thread, wavefront or
+    work-group, one quiet at the end; the bytes that land are those of the
+    blocking calls."""
+    o, g = getattr(L, op), getattr(L, gran)
+    for n in list(range(0, 40)) + [255, 256, 1000, 4099, 65537]:
+        run_case(rt, L, orc, env, o, g, n, 3, 5, 1, 128, ctx_options=ctx_options)
+    for soff in range(0, 16, 5):
+        for doff in range(0, 16, 3):
+            run_case(rt, L, orc, env, o, g, 777, soff, doff, 2, 64, ctx_options=ctx_options)
+    # small tiles: every group issues many calls before its quiet
+    for n, n_wgs, wg, tile in [(1 << 18, 2, 256, 64), (100001, 3, 192, 17), (1 << 20, 64, 256, 4096)]:
+        if gran == "WG" and tile < 4096:
+            n = n // 16
+        run_case(rt, L, orc, env, o, g, n, 1, 9, n_wgs, wg, tile=tile, ctx_options=ctx_options)
+
+
+@pytest.mark.parametrize("with_signal", [0, 1, 2, 3])
 @pytest.mark.parametrize("ctx_options", [0, 1])
 @pytest.mark.parametrize("nbytes,pairs,wg", [(4096, 1, 64), (65536, 16, 256), (1 << 20, 64, 1024),
                                              (262144 + 4, 128, 256)])
@@ -136,7 +157,8 @@ def test_put_quiet_flag_seen_in_order(rt, L, env, ctx_options, with_signal, nbyt
     flag that follows rocshmem_ctx_quiet (src/ipc/context_ipc_device.cpp:100-102)
     or by the signal of putmem_signal_wg (:221-247), must find every word of the
     payload, on a default context and on a ROCSHMEM_CTX_NOSTORE one, over 20
-    rounds with a new pattern each."""
+    rounds with a new pattern each.  with_signal 2 / 3: the payload leaves as
+    many putmem_nbi_wave / putmem_nbi calls which only the quiet completes."""
     import ctypes as C
     l = env["l"]
     data = l.malloc(nbytes * pairs)
