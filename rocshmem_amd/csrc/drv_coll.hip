@@ -257,12 +257,12 @@ struct GridMoveArgs {
   size_t span;
 };
 
-// alltoall: blockIdx.y names the block (sender, receiver), blockIdx.x walks
-// its spans.  Every byte is read once and written once.
+// alltoall: blockIdx.z is the sender, blockIdx.y the receiver, blockIdx.x
+// walks the spans of their block.  Every byte is read once and written once.
 template <bool kNonTemporal>
 __global__ void grid_alltoall_kernel(GridMoveArgs a) {
-  const int i = static_cast<int>(blockIdx.y / a.np);  // sender
-  const int j = static_cast<int>(blockIdx.y % a.np);  // receiver
+  const int i = static_cast<int>(blockIdx.z);  // sender
+  const int j = static_cast<int>(blockIdx.y);  // receiver
   char *d = a.dest0 + j * a.hop + static_cast<size_t>(i) * a.nbytes;
   const char *src = a.src0 + i * a.hop + static_cast<size_t>(j) * a.nbytes;
   for (size_t off = blockIdx.x * a.span; off < a.nbytes; off += gridDim.x * a.span) {
@@ -326,7 +326,8 @@ void launch_grid_move(char *dest0, const char *src0, int64_t hop, int np, int ro
                     : kMove == MOVE_FCOLLECT ? static_cast<size_t>(np) : 1;
   const size_t spans = (nbytes + a.span - 1) / a.span;
   const size_t max_x = kMoveMaxWgs / rows;
-  const dim3 grid(static_cast<unsigned>(spans < max_x ? spans : max_x), static_cast<unsigned>(rows));
+  const unsigned gx = static_cast<unsigned>(spans < max_x ? spans : (max_x ? max_x : 1));
+  const dim3 grid = kMove == MOVE_ALLTOALL ? dim3(gx, np, np) : dim3(gx, static_cast<unsigned>(rows));
   const dim3 block(kMoveThreads);
   if constexpr (kMove == MOVE_ALLTOALL) {
     if (nt) hipLaunchKernelGGL(grid_alltoall_kernel<true>, grid, block, 0, stream, a);

@@ -179,3 +179,51 @@ def test_zero_length_collectives_do_nothing(rt, L):
     assert l.wg_broadcast(4, l.team_world(), buf, buf, 8, P, 64, None) == -1  # bad root
     assert l.wg_alltoall(3, l.team_world(), buf, buf, 8, 64, None) == -1      # bad element size
     l.free(buf)
+
+
+def test_the_largest_world(rt, L, orc):
+    """256 PEs, the most one heap is divided into: whole-GPU and per-work-group
+    block moves (65 536 sender-receiver pairs), an all-reduce over all of them
+    and barrier rounds with one work-group per PE."""
+    big = 256
+    l = rt.up(big, 2 << 20)
+    n = 48                                   # bytes per block
+    src, dst = l.malloc(big * n), l.malloc(big * n)
+    assert src and dst
+    srcs = [orc.fill_u8(big * n, 9, p) for p in range(big)]
+    for p in range(big):
+        rt.put_bytes(l.pe_ptr(src, p), srcs[p])
+    for mode in ("grid", "wg"):
+        for kind in ("alltoall", "fcollect", "broadcast"):
+            assert l.fill_every_pe(dst, 0xC3, big * n, None) == 0
+            if kind == "alltoall":
+                rc = (l.alltoallmem(l.team_world(), dst, src, n, None) if mode == "grid" else
+                      l.wg_alltoall(1, l.team_world(), dst, src, n, 64, None))
+                want = orc.alltoall(srcs, n)
+            elif kind == "fcollect":
+                rc = (l.fcollectmem(l.team_world(), dst, src, n, None) if mode == "grid" else
+                      l.wg_fcollect(1, l.team_world(), dst, src, n, 64, None))
+                want = orc.fcollect([s[:n] for s in srcs], n)
+            else:
+                rc = (l.broadcastmem(l.team_world(), dst, src, big * n, 200, None) if mode == "grid" else
+                      l.wg_broadcast(1, l.team_world(), dst, src, big * n, 200, 64, None))
+                want = [np.full(big * n, 0xC3, np.uint8) for _ in range(big)]
+                orc.broadcast(srcs, want, big * n, 200)
+            assert rc == 0, (mode, kind)
+            l.stream_sync(None)
+            for p in range(big):
+                got = rt.get_bytes(l.pe_ptr(dst, p), big * n)
+                assert np.array_equal(got, want[p]), (mode, kind, p)
+    ints = [s.view(np.int32) for s in srcs]
+    total = orc.to_all(L.INT, L.SUM, ints)
+    assert l.to_all(L.INT, L.SUM, dst, src, big * n // 4, 0, 0, big, None) == 0
+    l.stream_sync(None)
+    for p in (0, 1, 100, 255):
+        assert np.array_equal(rt.get_bytes(l.pe_ptr(dst, p), big * n, np.int32), total), p
+    word = l.malloc(8)
+    assert l.fill_every_pe(word, 0, 8, None) == 0
+    for fn in (L.BARRIER_ALL, L.SYNC_ALL, L.TEAM_SYNC):
+        assert l.wg_sync(fn, l.team_world(), word, 5, 64, None) == 0, fn
+    for b in (src, dst, word):
+        l.free(b)
+    rt.up(P, HEAP)
