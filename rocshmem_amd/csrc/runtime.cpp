@@ -609,15 +609,18 @@ __host__ int rocshmem_team_split_strided(rocshmem_team_t parent_team, int start,
   // Every member receives the same handle (the first member's object), so a
   // program that keeps it in a variable its PE threads share still works; the
   // host calls and, under the queue rule, the device calls resolve it to the
-  // caller's own object.
-  *new_team = ROCSHMEM_TEAM_INVALID;
+  // caller's own object.  That variable is written once, with the final value:
+  // another member may already be reading it (all members store the same
+  // handle), and a transient ROCSHMEM_TEAM_INVALID there would reach its kernel.
+  rocshmem_team_t result = ROCSHMEM_TEAM_INVALID;
   if (rc == 0 && slot >= 0) {
     const rocshmem_team_t mine = rt().team_on(rt().team_handle(slot, w.pe_start), rt().me());
     if (mine != ROCSHMEM_TEAM_INVALID) {
       const detail::Team *t = rt().host_team(mine);
-      *new_team = rt().team_handle(slot, t->wrt_world.pe_start);
+      result = rt().team_handle(slot, t->wrt_world.pe_start);
     }
   }
+  *new_team = result;
   return rc;
 }
 __host__ void rocshmem_team_destroy(rocshmem_team_t team) {
