@@ -174,7 +174,7 @@ def to_all_configs(b, steps, warmup):
         kind = {L.FLOAT: "f32", L.BF16: "bf16"}.get(dt, "u8")
         for p in range(P):
             b.fill_random(l.pe_ptr(src, p), n * es, p, 10 + p, kind)
-        ms = b.time_ms(lambda: l.to_all(dt, op, dst, src, n, 0, 0, P, None), max(5, steps // 5), 3)
+        ms = b.time_ms(lambda: l.to_all(dt, op, dst, src, n, 0, 0, P, None), max(10, steps), 5)
         alg = 2 * P * n * es
         res[name] = {"ms": round(ms, 4), "gbs": round(alg / ms / 1e6, 1),
                      "frac": round(alg / ms / 1e6 / HBM_PEAK_GBS, 4)}
@@ -211,20 +211,20 @@ def alltoall_config(b, steps):
     assert src and dst
     for p in range(P):
         b.fill_random(l.pe_ptr(src, p), P * blk, p, 30 + p)
-    n = max(5, steps // 5)
+    n = max(10, steps)
 
     def entry(ms, alg):
         return {"ms": round(ms, 4), "gbs": round(alg / ms / 1e6, 1),
                 "frac": round(alg / ms / 1e6 / HBM_PEAK_GBS, 4)}
 
-    res = entry(b.time_ms(lambda: l.alltoallmem(l.team_world(), dst, src, blk, None), n, 3),
+    res = entry(b.time_ms(lambda: l.alltoallmem(l.team_world(), dst, src, blk, None), n, 5),
                 2 * P * P * blk)
     # every block is read once and written P times (P-1 for the broadcast)
     res["fcollect_same_block"] = entry(
-        b.time_ms(lambda: l.fcollectmem(l.team_world(), dst, src, blk, None), n, 3),
+        b.time_ms(lambda: l.fcollectmem(l.team_world(), dst, src, blk, None), n, 5),
         (P + P * P) * blk)
     res["broadcast_P_blocks_from_pe0"] = entry(
-        b.time_ms(lambda: l.broadcastmem(l.team_world(), dst, src, P * blk, 0, None), n, 3),
+        b.time_ms(lambda: l.broadcastmem(l.team_world(), dst, src, P * blk, 0, None), n, 5),
         P * P * blk)
     l.free(src)
     l.free(dst)

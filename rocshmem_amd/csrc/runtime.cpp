@@ -207,7 +207,25 @@ int Runtime::init(int want_npes, size_t want_heap) {
   acting_pe = 0;
   driver_ctx_options = 0;
 
-  if (hipMalloc(reinterpret_cast<void **>(&heap_base), pe_stride * npes) != hipSuccess) {
+  // Where the block lands physically matters as much as the stride.  A block
+  // of 128 GiB fits twice into the 288 GB of an MI355X, the driver hands out
+  // the two places in turn (a freed block is not reused at once), and kernels
+  // with 16 concurrent streams run 2.5 % slower in one of them (the P = 8
+  // all-reduce: 6.28 instead of 6.45-6.48 TB/s, alternating from one
+  // rocshmem_init to the next, in one process or across processes).  A block of
+  // more than half of the memory fits in one place only, and that place is the
+  // good one: a heap of a quarter of the memory or more is therefore allocated
+  // as half of the memory plus 1 GiB when that much is free (the slices use the
+  // front of it).  ROCSHMEM_EMU_HEAP_ANCHOR=0 switches this off.
+  size_t alloc_bytes = pe_stride * npes;
+  if (env_size("ROCSHMEM_EMU_HEAP_ANCHOR", 1) != 0) {
+    size_t free_b = 0, total_b = 0;
+    RT_CHECK_HIP(hipMemGetInfo(&free_b, &total_b));
+    const size_t anchor = total_b / 2 + (size_t{1} << 30);
+    if (alloc_bytes >= total_b / 4 && alloc_bytes < anchor && free_b > anchor + (size_t{16} << 30))
+      alloc_bytes = anchor;
+  }
+  if (hipMalloc(reinterpret_cast<void **>(&heap_base), alloc_bytes) != hipSuccess) {
     (void)hipGetLastError();  // not enough room for the spread layout: pack the slices
     pe_stride = min_stride;
     RT_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&heap_base), pe_stride * npes));
