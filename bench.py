@@ -481,7 +481,7 @@ def main():
                      "unit": "GB/s", "frac": round(head["gbs"] / HBM_PEAK_GBS, 4),
                      # FETCH_SIZE + WRITE_SIZE per launch under rocprofv3 --pmc, scaled by the
                      # HIP runtime's own copy kernel (profiles/bulk_copy_256MiB_hbm_traffic.txt)
-                     "traffic": 536870698, "kernel": "bulk_copy_kernel<true>",
+                     "traffic": 536869499, "kernel": "bulk_copy_kernel<true>",
                      # measured in this run: what a pure read / pure write stream of the
                      # same shape sustains, and the copy rate those two allow
                      "measured_ceilings": head["ceilings"],
