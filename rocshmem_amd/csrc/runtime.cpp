@@ -187,9 +187,9 @@ int Runtime::init(int want_npes, size_t want_heap) {
   // Slice placement.  Slices start on 2 MiB boundaries and sit `pe_stride`
   // apart inside ONE device allocation, which the driver backs with contiguous
   // physical memory.  On MI355X a kernel that writes to all P slices at once
-  // (all-reduce, alltoall) sustains about 12 % more HBM bandwidth when the
-  // slices are 12-18 GiB apart than when they are 8 GiB or less apart
-  // (measured: 6.44 vs 5.73 TB/s for the P = 8 fp32 all-reduce; eight
+  // (all-reduce, alltoall) sustains about 10 % more HBM bandwidth when the
+  // slices are 16-17 GiB apart than when they are 12 GiB or less apart
+  // (measured: 6.45 vs 5.7-5.9 TB/s for the P = 8 fp32 all-reduce; eight
   // concurrent write streams alone: 7.2 vs 6.0 TB/s), so the default stride is
   // 16 GiB as long as all slices together stay within half of the device
   // memory.  ROCSHMEM_EMU_PE_STRIDE overrides it.
