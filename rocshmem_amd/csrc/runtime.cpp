@@ -225,7 +225,12 @@ int Runtime::init(int want_npes, size_t want_heap) {
     if (alloc_bytes >= total_b / 4 && alloc_bytes < anchor && free_b > anchor + (size_t{16} << 30))
       alloc_bytes = anchor;
   }
-  if (hipMalloc(reinterpret_cast<void **>(&heap_base), alloc_bytes) != hipSuccess) {
+  hipError_t got = hipMalloc(reinterpret_cast<void **>(&heap_base), alloc_bytes);
+  if (got != hipSuccess && alloc_bytes != pe_stride * npes) {
+    (void)hipGetLastError();  // no room for the larger block: just the slices
+    got = hipMalloc(reinterpret_cast<void **>(&heap_base), pe_stride * npes);
+  }
+  if (got != hipSuccess) {
     (void)hipGetLastError();  // not enough room for the spread layout: pack the slices
     pe_stride = min_stride;
     RT_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&heap_base), pe_stride * npes));
