@@ -191,15 +191,17 @@ int Runtime::init(int want_npes, size_t want_heap) {
   // slices are 16-17 GiB apart than when they are 12 GiB or less apart
   // (measured: 6.45 vs 5.7-5.9 TB/s for the P = 8 fp32 all-reduce; eight
   // concurrent write streams alone: 7.2 vs 6.0 TB/s), so the default stride is
-  // 16 GiB as long as all slices together stay within half of the device
-  // memory.  ROCSHMEM_EMU_PE_STRIDE overrides it.
+  // 16 GiB (32 GiB for three or four PEs) as long as all slices together stay
+  // within half of the device memory.  ROCSHMEM_EMU_PE_STRIDE overrides it.
   const size_t two_mib = size_t{2} << 20;
   const size_t min_stride = round_up(heap_size, two_mib);
   size_t want = env_size("ROCSHMEM_EMU_PE_STRIDE", 0);
   if (!want) {
     size_t free_b = 0, total_b = 0;
     RT_CHECK_HIP(hipMemGetInfo(&free_b, &total_b));
-    want = size_t{16} << 30;
+    // Three or four slices do better still at 32 GiB (all-reduce 6.61 and 6.56
+    // against 6.48 and 6.26 TB/s at 16 GiB); two do not care.
+    want = (npes == 3 || npes == 4) ? size_t{32} << 30 : size_t{16} << 30;
     const size_t budget = std::min(total_b / 2, free_b / 4 * 3);
     if (want * npes > budget) want = budget / npes;
   }

@@ -135,16 +135,18 @@ def test_team_pool_exhaustion(rt, L):
 
 
 def test_default_slice_stride_spreads_the_pes(rt, L, monkeypatch):
-    """Without an override the slices sit 16 GiB apart (or as far as half of
-    the device memory allows), never closer than the heap size."""
+    """Without an override the slices sit 16 GiB apart, 32 GiB for three or
+    four PEs (or as far as half of the device memory allows), never closer
+    than the heap size."""
     monkeypatch.delenv("ROCSHMEM_EMU_PE_STRIDE", raising=False)
     rt.down()
     l = L.load()
-    assert l.init(4, 1 << 24) == 0
-    assert l.pe_stride() == 16 << 30
-    a = l.malloc(64)
-    assert l.pe_ptr(a, 3) - a == 3 * (16 << 30)
-    l.finalize()
+    for npes, gib in ((2, 16), (3, 32), (4, 32), (8, 16)):
+        assert l.init(npes, 1 << 24) == 0
+        assert l.pe_stride() == gib << 30, npes
+        a = l.malloc(64)
+        assert l.pe_ptr(a, npes - 1) - a == (npes - 1) * (gib << 30)
+        l.finalize()
     monkeypatch.setenv("ROCSHMEM_EMU_PE_STRIDE", str(6 << 20))
     assert l.init(4, 1 << 22) == 0
     assert l.pe_stride() == 6 << 20
