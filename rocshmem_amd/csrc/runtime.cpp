@@ -190,19 +190,24 @@ int Runtime::init(int want_npes, size_t want_heap) {
   // (all-reduce, alltoall) sustains about 10 % more HBM bandwidth when the
   // slices are 16-17 GiB apart than when they are 12 GiB or less apart
   // (measured: 6.45 vs 5.7-5.9 TB/s for the P = 8 fp32 all-reduce; eight
-  // concurrent write streams alone: 7.2 vs 6.0 TB/s), so the default stride is
-  // 16 GiB (32 GiB for three or four PEs) as long as all slices together stay
-  // within half of the device memory.  ROCSHMEM_EMU_PE_STRIDE overrides it.
+  // concurrent write streams alone: 7.2 vs 6.0 TB/s).
+  // ROCSHMEM_EMU_PE_STRIDE overrides the default chosen below.
   const size_t two_mib = size_t{2} << 20;
   const size_t min_stride = round_up(heap_size, two_mib);
   size_t want = env_size("ROCSHMEM_EMU_PE_STRIDE", 0);
   if (!want) {
     size_t free_b = 0, total_b = 0;
     RT_CHECK_HIP(hipMemGetInfo(&free_b, &total_b));
-    // Three or four slices do better still at 32 GiB (all-reduce 6.61 and 6.56
-    // against 6.48 and 6.26 TB/s at 16 GiB); two do not care.
-    want = (npes == 3 || npes == 4) ? size_t{32} << 30 : size_t{16} << 30;
+    // What counts is that the slices are spread over about half of the device
+    // memory, whatever their number: P = 8 at 16 GiB, 12 at 12, 16 at 8 GiB
+    // all reach 6.45-6.5 TB/s in the all-reduce (8 at 8 GiB: 6.0, 16 at
+    // 4 GiB: 5.7), 3, 4 and 5 slices gain 2-5 % at 40, 32 and 28 GiB over
+    // 16 GiB.  Two slices do not care and keep 16 GiB.  Strides stay on a
+    // 4 GiB grid: some odd offsets (plus 1 MiB, plus 128 MiB) cost 5-9 %.
     const size_t budget = std::min(total_b / 2, free_b / 4 * 3);
+    const size_t grid = size_t{4} << 30;
+    want = npes <= 2 ? size_t{16} << 30 : budget / npes;
+    if (want >= grid) want = want / grid * grid;
     if (want * npes > budget) want = budget / npes;
   }
   pe_stride = std::max(min_stride, want / two_mib * two_mib);

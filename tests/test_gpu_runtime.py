@@ -135,13 +135,13 @@ def test_team_pool_exhaustion(rt, L):
 
 
 def test_default_slice_stride_spreads_the_pes(rt, L, monkeypatch):
-    """Without an override the slices sit 16 GiB apart, 32 GiB for three or
-    four PEs (or as far as half of the device memory allows), never closer
-    than the heap size."""
+    """Without an override the slices are spread over half of the device
+    memory on a 4 GiB grid (288 GB: 16 GiB for 8 PEs, 32 for 4, 44 for 3, 8
+    for 16; two PEs keep 16 GiB), never closer than the heap size."""
     monkeypatch.delenv("ROCSHMEM_EMU_PE_STRIDE", raising=False)
     rt.down()
     l = L.load()
-    for npes, gib in ((2, 16), (3, 32), (4, 32), (8, 16)):
+    for npes, gib in ((2, 16), (3, 44), (4, 32), (5, 28), (8, 16), (16, 8)):
         assert l.init(npes, 1 << 24) == 0
         assert l.pe_stride() == gib << 30, npes
         a = l.malloc(64)
