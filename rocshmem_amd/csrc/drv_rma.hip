@@ -1,6 +1,8 @@
 // Drivers for the copy path: device-API put/get at thread, wavefront and
 // work-group granularity, the host-initiated whole-GPU copy, and the
 // wavefront coalescing utility.
+#include <mutex>
+
 #include "drv_common.hpp"
 #include "rocshmem/detail/coalesce.hpp"
 #include "rocshmem_amd.h"
@@ -232,8 +234,9 @@ int rocshmem_amd_hbm_probe(int write, void *buf, size_t nbytes, rocshmem_amd_str
   if (!runtime::rt().live || !buf || nbytes < (1u << 20) || (reinterpret_cast<uintptr_t>(buf) & 15u))
     return -1;
   if (!local_ok(buf, nbytes)) return -1;
-  static unsigned *sink = nullptr;
-  if (!sink) DRV_CHECK_HIP(hipMalloc(&sink, sizeof(unsigned)));
+  static unsigned *sink = nullptr;  // never written in practice; allocated once
+  static std::once_flag sink_once;
+  std::call_once(sink_once, [] { DRV_CHECK_HIP(hipMalloc(&sink, sizeof(unsigned))); });
   const size_t nvec = nbytes / 16;
   const unsigned grid = static_cast<unsigned>((nvec + kProbeThreads - 1) / kProbeThreads);
   if (write)

@@ -1,5 +1,7 @@
 // Drivers for atomics, put-with-signal, point-to-point waits, the ping-pong
 // and MoE-dispatch patterns, and context lifecycle.
+#include <mutex>
+
 #include "drv_common.hpp"
 #include "rocshmem_amd.h"
 
@@ -800,6 +802,7 @@ int rocshmem_amd_put_flag_check(void *data, uint64_t *flags, size_t nbytes, int 
 // with the same tables only launches.
 namespace {
 struct DispatchTables {
+  std::mutex lock;             // one caller at a time rebuilds or reads the tables
   std::vector<uint32_t> host;  // count | send_row | recv_row | calls {pair, first row}
   uint32_t *dev = nullptr;
   size_t pp = 0;
@@ -820,6 +823,7 @@ int rocshmem_amd_dispatch_put_signal(void *recv, const void *send, uint64_t *sig
   if (!count || !send_row || !recv_row) return -1;
   const size_t pp = static_cast<size_t>(r.npes) * r.npes;
   DispatchTables &t = g_tables;
+  std::lock_guard<std::mutex> guard(t.lock);
   std::vector<uint32_t> h(3 * pp);
   std::copy(count, count + pp, h.begin());
   std::copy(send_row, send_row + pp, h.begin() + pp);
