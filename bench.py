@@ -5,12 +5,14 @@
 
 Prints ONE JSON line.  The headline (`metric`/`value`) is the bulk putmem
 workload of BASELINE.json's configs[1]: one 256 MiB message between two of
-P=8 PE slices of one symmetric heap, moved by the whole GPU; a step is one such
-message and `value` counts algorithmic bytes (N read + N written).  The same
-line carries the other configurations (all-reduce, alltoall, put_signal
-dispatch, atomics, ping-pong) under `all_configs`, the roofline of the
-headline kernel measured with HIP events on the launch stream, and a CPU
-baseline (the oracle's threaded routines on the host cores, bounded sample).
+P=8 PE slices of one symmetric heap, moved by all CUs through the device API
+(rocshmem_ctx_putmem_wg, one 16 KiB tile per work-group of 256, on a context
+created with ROCSHMEM_CTX_NOSTORE); a step is one such message and `value`
+counts algorithmic bytes (N read + N written).  The same workload through a
+default context and through the host-side rocshmem_putmem, and every other
+configuration (all-reduce, alltoall, put_signal dispatch, atomics, ping-pong),
+are carried as scalar keys of `roofline` (and in full under `all_configs`),
+beside a CPU baseline (the oracle's threaded routines on the host cores).
 
 Inputs are resident in HBM before any timed region starts.
 """
@@ -27,6 +29,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X, published
+# HBM bytes one launch of the headline kernel moves, from FETCH_SIZE + WRITE_SIZE
+# under rocprofv3 --pmc (profiles/putmem_wg_tiled_256MiB_hbm_traffic.txt); None
+# until that profile has been taken for the current kernel.
+PUT_TRAFFIC_BYTES = None
 P = 8
 MiB = 1 << 20
 
@@ -89,12 +95,23 @@ class Bench:
         l.stream_sync(None)
 
 
+# Launch shapes of the tiled device-API put, from a sweep over work-group size
+# {64..1024} x tile {1 KiB..256 KiB} x work-groups {256..262144} on MI355X:
+#   NOSTORE context: one 16 KiB tile per work-group of 256 (each lane moves four
+#     vectors, then the work-group leaves) — the closest a putmem_wg loop gets
+#     to the one-vector work-groups of the bulk kernel;
+#   default context: every work-group ends in a quiet, i.e. an L2 write-back
+#     that stalls its XCD for about 0.3 us, so few work-groups that loop:
+#     256 work-groups of 512, 32 KiB tiles.
+PUT_SHAPES = {"nostore_ctx": (256, 16384, None), "default_ctx": (512, 32768, 256)}
+
+
 def headline(b, steps, warmup):
     """configs[1]: bulk putmem, 256 MiB messages, all CUs.  Step k sends from
     PE k%8 to PE (k+1)%8, so consecutive steps touch different 256 MiB buffers
     (4 GiB in rotation): nothing is served from the 256 MB memory-side cache and
     the rate is what HBM sustains."""
-    l = b.l
+    l, L = b.l, b.L
     n = 256 * MiB
     src, dst = l.malloc(n), l.malloc(n)
     assert src and dst
@@ -111,8 +128,28 @@ def headline(b, steps, warmup):
             assert fn(me, (me + 1) % P) == 0
         return step
 
-    ms = b.time_ms(rotating(lambda me, pe: l.putmem(dsts[me], srcs[me], n, me, pe, None)), steps, warmup)
-    out = {"bytes_per_step": 2 * n, "ms": ms, "gbs": 2 * n / ms / 1e6}
+    def tiled_put(kind):
+        wg, tile, n_wgs = PUT_SHAPES[kind]
+        n_wgs = n_wgs or n // tile
+        return rotating(lambda me, pe: l.rma(L.PUT, L.WG, dsts[me], srcs[me], n, tile, me, pe, n_wgs, wg,
+                                             1, None))
+
+    out = {"bytes_per_step": 2 * n}
+    # The device API, rocshmem_ctx_putmem_wg from every CU: the headline.
+    l.set_ctx_options(1)
+    out["ms"] = b.time_ms(tiled_put("nostore_ctx"), steps, warmup)
+    out["gbs"] = 2 * n / out["ms"] / 1e6
+    l.set_ctx_options(0)
+    out["default_ctx_gbs"] = 2 * n / b.time_ms(tiled_put("default_ctx"), steps, warmup) / 1e6
+    # The host-side rocshmem_putmem (one whole-GPU kernel per message).
+    out["host_putmem_gbs"] = 2 * n / b.time_ms(
+        rotating(lambda me, pe: l.putmem(dsts[me], srcs[me], n, me, pe, None)), steps, warmup) / 1e6
+    out["host_getmem_gbs"] = 2 * n / b.time_ms(
+        rotating(lambda me, pe: l.getmem(dsts[me], srcs[me], n, me, pe, None)), steps, warmup) / 1e6
+    if b.quick:
+        l.free(src)
+        l.free(dst)
+        return out
     # The bandwidth curve, 8 B .. 256 MiB (26 sizes).  One work-group of 64, 256
     # and 1024 threads issuing rocshmem_putmem_wg / getmem_wg: the call is
     # repeated inside the kernel (as the reference's testers loop inside theirs)
@@ -125,10 +162,10 @@ def headline(b, steps, warmup):
         inner = 200 if e <= 16 else (20 if e <= 24 else 2)
         point = {}
         for threads in (64, 256, 1024):
-            t = b.time_ms(rotating(lambda me, pe: l.rma(b.L.PUT, b.L.WG, dsts[me], srcs[me], m, 0, me, pe,
+            t = b.time_ms(rotating(lambda me, pe: l.rma(L.PUT, L.WG, dsts[me], srcs[me], m, 0, me, pe,
                                                         1, threads, inner, None)), 3, 1) / inner
             point["putmem_wg_1wg_%dthr_gbs" % threads] = round(2 * m / t / 1e6, 3)
-        t = b.time_ms(rotating(lambda me, pe: l.rma(b.L.GET, b.L.WG, dsts[me], srcs[me], m, 0, me, pe,
+        t = b.time_ms(rotating(lambda me, pe: l.rma(L.GET, L.WG, dsts[me], srcs[me], m, 0, me, pe,
                                                     1, 1024, inner, None)), 3, 1) / inner
         point["getmem_wg_1wg_1024thr_gbs"] = round(2 * m / t / 1e6, 3)
         tg = b.time_ms(rotating(lambda me, pe: l.putmem(dsts[me], srcs[me], m, me, pe, None)), reps, 2)
@@ -143,17 +180,24 @@ def headline(b, steps, warmup):
     t_wr = b.time_ms(rotating(lambda me, pe: l.hbm_probe(1, dsts[pe], n, None)), steps, warmup)
     rd, wr = n / t_rd / 1e6, n / t_wr / 1e6
     out["ceilings"] = {"read_only_gbs": round(rd, 1), "write_only_gbs": round(wr, 1),
-                       "copy_bound_gbs": round(2 / (1 / rd + 1 / wr), 1),
-                       "copy_over_bound": round(out["gbs"] / (2 / (1 / rd + 1 / wr)), 4)}
-    # Device API from every CU: rocshmem_ctx_putmem_wg on 64 KiB tiles, one
-    # quiet per work-group, through a default and a NOSTORE context.
+                       "copy_bound_gbs": round(2 / (1 / rd + 1 / wr), 1)}
+    # What one agent-scope release (the write-back in a default context's quiet)
+    # costs while the copy runs: 1024 work-groups of 256, 16 KiB tiles.
+    rp = {}
+    for mode in (0, 1, 2):
+        rp[mode] = b.time_ms(rotating(lambda me, pe: l.release_probe(mode, dsts[pe], srcs[me], n, 16384,
+                                                                     1024, 256, None)), 5, 2)
+    out["release_ns_each_per_tile"] = round((rp[2] - rp[0]) * 1e6 / (n // 16384), 1)
+    out["release_ns_each_at_end"] = round((rp[1] - rp[0]) * 1e6 / 1024, 1)
+    # The tiled put of the headline in other shapes, both kinds of context.
     tiled = {}
     for name, opt in CTX_KINDS:
         l.set_ctx_options(opt)
-        for n_wgs in (1024, 4096):
-            t = b.time_ms(rotating(lambda me, pe: l.rma(b.L.PUT, b.L.WG, dsts[me], srcs[me], n, 65536, me,
-                                                        pe, n_wgs, 1024, 1, None)), max(3, min(steps, 20)), 2)
-            tiled["%s_%dwgs_gbs" % (name, n_wgs)] = round(2 * n / t / 1e6, 1)
+        for wg, tile, n_wgs in ((256, 16384, None), (512, 32768, 256), (1024, 65536, 1024),
+                                (1024, 65536, 4096)):
+            t = b.time_ms(rotating(lambda me, pe: l.rma(L.PUT, L.WG, dsts[me], srcs[me], n, tile, me, pe,
+                                                        n_wgs or n // tile, wg, 1, None)), 5, 2)
+            tiled["%s_wg%d_tile%d_%dwgs_gbs" % (name, wg, tile, n_wgs or n // tile)] = round(2 * n / t / 1e6, 1)
     l.set_ctx_options(0)
     out["tiled"] = tiled
     l.free(src)
@@ -185,16 +229,22 @@ def to_all_configs(b, steps, warmup):
             res["fp32_sum_wg_reduce_one_wg_per_pe"] = {"ms": round(ms, 4),
                                                        "gbs": round(alg / ms / 1e6, 1)}
             # ... and the way the reference's testers scale it: one team per
-            # work-group, 64 teams x 8 PEs at once (two work-groups per CU).
-            NT = 64
+            # work-group, 32 teams x 8 PEs at once (one work-group of 256 per CU),
+            # the call repeated four times inside the kernel.
+            NT, inner = 32, 4
             teams = (C.c_void_p * NT)()
             for t in range(NT):
                 h = C.c_void_p()
                 assert l.team_split_strided(l.team_world(), 0, 1, P, C.byref(h)) == 0 and h.value
                 teams[t] = h.value
-            ms = b.time_ms(lambda: l.wg_reduce_teams(dt, op, teams, NT, dst, src, n, 1024, None), 3, 1)
-            res["fp32_sum_wg_reduce_64_teams"] = {"ms": round(ms, 4), "gbs": round(alg / ms / 1e6, 1),
-                                                  "frac": round(alg / ms / 1e6 / HBM_PEAK_GBS, 4)}
+            for cname, opt in CTX_KINDS:
+                l.set_ctx_options(opt)
+                ms = b.time_ms(lambda: l.wg_reduce_teams(dt, op, teams, NT, dst, src, n, 256, inner, None),
+                               3, 1) / inner
+                res["fp32_sum_wg_reduce_32_teams_" + cname] = {
+                    "ms": round(ms, 4), "gbs": round(alg / ms / 1e6, 1),
+                    "frac": round(alg / ms / 1e6 / HBM_PEAK_GBS, 4)}
+            l.set_ctx_options(0)
             for t in range(NT):
                 l.team_destroy(teams[t])
         l.free(src)
@@ -238,7 +288,8 @@ def zipf_table(K, s):
 
 def dispatch_config(b, steps, shapes=((64, 1024),)):
     """configs[4] part 2: put_signal dispatch, 4096 tokens/PE, top-8 of 256
-    experts by Zipf(1.1), rows of 7168 bf16."""
+    experts by Zipf(1.1), rows of 7168 bf16.  shapes: (rows per
+    putmem_signal_wg call, work-group size)."""
     l = b.l
     tokens, experts, topk, row = 4096, 256, 8, 7168 * 2
     rng = np.random.default_rng(0)
@@ -268,13 +319,17 @@ def dispatch_config(b, steps, shapes=((64, 1024),)):
     for p in range(P):
         b.fill_random(l.pe_ptr(send, p), rows_out * row, p, 40 + p)
     tabs = [np.ascontiguousarray(a, np.uint32) for a in (counts, send_row, recv_row)]
+    # Signal words are never cleared: the receivers keep running totals.
+    expect = l.dev_alloc(8 * P * P)
+    l.fill(expect, 0, 8 * P * P)
+    assert l.fill_every_pe(sig, 0, 8 * P, None) == 0
+    l.stream_sync(None)
 
     shape = [shapes[0]]
 
     def step():
-        assert l.fill_every_pe(sig, 0, 8 * P, None) == 0  # signals start from zero each dispatch
         assert l.dispatch_put_signal(recv, send, sig, tabs[0].ctypes.data, tabs[1].ctypes.data,
-                                     tabs[2].ctypes.data, row, shape[0][0], shape[0][1], None) == 0
+                                     tabs[2].ctypes.data, row, shape[0][0], shape[0][1], expect, None) == 0
 
     alg = 2 * int(counts.sum()) * row
     res = {"rows": int(counts.sum())}
@@ -287,6 +342,7 @@ def dispatch_config(b, steps, shapes=((64, 1024),)):
             res[key] = {"ms": round(ms, 4), "gbs": round(alg / ms / 1e6, 1),
                         "frac": round(alg / ms / 1e6 / HBM_PEAK_GBS, 4)}
     l.set_ctx_options(0)
+    l.dev_free(expect)
     for x in (send, recv, sig):
         l.free(x)
     return res
@@ -375,13 +431,13 @@ def barrier_config(b):
 
 
 def cpu_baseline():
-    """The oracle's threaded routines on this host's cores, bounded samples.
-    (The only place outside tests/ and smoke() that touches oracle/.)"""
+    """The oracle's threaded routines on this host's cores, bounded samples of
+    the same workloads.  (The only place outside tests/ and smoke() that
+    touches oracle/.)"""
     from oracle import pyoracle as orc
-    cores = orc.lib.orc_hardware_threads()
-    threads = max(1, cores)
-    out = {}
-    # bulk copy: 256 MiB message, as the headline
+    # a one-GPU box gives a job 16 cores, whatever the machine has
+    threads = max(1, min(16, orc.lib.orc_hardware_threads()))
+    # bulk copy: 256 MiB messages, as the headline
     n = 256 * MiB
     src = np.random.default_rng(0).integers(0, 256, n, dtype=np.uint8)
     # eight buffer pairs taken in turn, as on the GPU: 4 GiB in all, more than the
@@ -397,33 +453,37 @@ def cpu_baseline():
         orc.lib.orc_copy_threaded(dsts[(k + 1) % P].ctypes.data, srcs[k].ctypes.data, n, threads)
         reps += 1
     copy_gbs = 2 * n * reps / (time.perf_counter() - t0) / 1e9
-    del srcs, dsts
-    # fp32 sum all-reduce, P=8 x 4 Mi elements (1/16 of the GPU workload)
-    m = 1 << 22
-    srcs = [np.random.default_rng(p).standard_normal(m).astype(np.float32) for p in range(P)]
+    del srcs, dsts, src
+    # fp32 sum all-reduce at the GPU's size: P=8 x 64 Mi elements, result written to
+    # all 8 destinations (4 GiB of host memory), at least two passes
+    m = 1 << 26
+    tile = np.random.default_rng(1).standard_normal(1 << 22).astype(np.float32)
+    srcs = [np.tile(np.roll(tile, p), m // tile.size) for p in range(P)]
+    orc.to_all(orc.FLOAT, orc.SUM, srcs, ndst=P, nthreads=threads)
     t0 = time.perf_counter()
     reps = 0
-    while time.perf_counter() - t0 < 4.0:
+    while reps < 2 or time.perf_counter() - t0 < 4.0:
         orc.to_all(orc.FLOAT, orc.SUM, srcs, ndst=P, nthreads=threads)
         reps += 1
     red_gbs = 2 * P * m * 4 * reps / (time.perf_counter() - t0) / 1e9
-    # atomics: 4 Mi fetch_adds onto 4096 counters
-    k = 1 << 22
+    del srcs
+    # atomics at the GPU's size: 16 Mi seq_cst fetch_adds onto 4096 counters
+    k = 1 << 24
     ids = np.random.default_rng(1).integers(0, 4096, k, dtype=np.uint32)
     counters = np.zeros(4096, np.int64)
     fetched = np.zeros(k, np.int64)
     sec = orc.lib.orc_amo_fetch_add_threaded(counters.ctypes.data, ids.ctypes.data, None,
                                              fetched.ctypes.data, k, threads)
     pp = orc.lib.orc_pingpong_threaded(8, 200000) / 200000 / 2 * 1e6
-    out = {"value": round(copy_gbs, 2), "unit": "GB/s", "cores": threads, "kind": "port",
-           "sample": "threaded memcpy of 256 MiB messages for 4 s, eight buffer pairs in turn "
-                     "(2N bytes per message)",
-           "other": {"fp32_sum_to_all_gbs": round(red_gbs, 2),
-                     "fp32_sum_sample": "P=8 x 4 Mi elements, ascending fold, 4 s",
-                     "amo_fetch_add_mops": round(k / sec / 1e6, 1),
-                     "amo_sample": "4 Mi seq_cst fetch_add on 4096 counters, uniform",
-                     "pingpong_8B_latency_us": round(pp, 3)}}
-    return out
+    return {"value": round(copy_gbs, 2), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": "threaded memcpy of 256 MiB messages for 4 s, eight buffer pairs in turn "
+                      "(2N bytes per message); all-reduce: P=8 x 64 Mi fp32, ascending fold, all 8 "
+                      "destinations written, >= 2 passes; atomics: 16 Mi seq_cst fetch_add on 4096 "
+                      "counters, uniform; ping-pong: 200000 round trips of 8 B between two threads",
+            "putmem_256MiB_gbs": round(copy_gbs, 2),
+            "to_all_fp32_sum_gbs": round(red_gbs, 2),
+            "amo_fetch_add_mops": round(k / sec / 1e6, 1),
+            "pingpong_8B_us": round(pp, 3)}
 
 
 def main():
@@ -432,13 +492,18 @@ def main():
         print("bench.py measures one GPU: every PE is a slice of one symmetric heap on a single "
               "MI355X; --gpus %d is not supported (use --gpus 1)." % a.gpus, file=sys.stderr)
         sys.exit(2)
+    # The slices spread over half of the device memory (16 GiB apart): kernels that
+    # write to all 8 slices at once sustain about 10 % more than with packed slices.
+    os.environ.setdefault("ROCSHMEM_EMU_SPREAD", "1")
+    os.environ.setdefault("ROCSHMEM_MAX_NUM_TEAMS", "40")
     from rocshmem_amd import lib as L
     b = Bench(L)
+    b.quick = a.quick
     # 8 slices of 8 GiB: with Zipf(1.1) routing the busiest PE receives 2.3 GiB
     # of rows, a 4 GiB block of the power-of-two allocator.  That request goes
     # first because the allocator never merges freed blocks.
-    os.environ.setdefault("ROCSHMEM_MAX_NUM_TEAMS", "72")  # the many-teams all-reduce uses 64
     assert b.l.init(P, 8 << 30) == 0
+    layout = {"pe_stride_bytes": b.l.pe_stride(), "heap_alloc_bytes": b.l.heap_alloc_bytes()}
     allc = {}
     if not a.quick:
         allc["dispatch_put_signal"] = dispatch_config(b, a.steps)
@@ -455,11 +520,61 @@ def main():
         allc["atomic_fetch_add_16Mi"] = amo_config(b, a.steps)
         allc["pingpong"] = pingpong_config(b)
         allc["barrier_P8"] = barrier_config(b)
-    allc["putmem_curve"] = head["curve"]
-    allc["hbm_one_direction_256MiB"] = head["ceilings"]
-    allc["putmem_wg_64KiB_tiles_256MiB"] = head["tiled"]
+        allc["putmem_curve"] = head["curve"]
+        allc["hbm_one_direction_256MiB"] = head["ceilings"]
+        allc["putmem_wg_tiled_256MiB"] = head["tiled"]
     b.l.finalize()
     cpu = None if (a.quick or a.no_cpu) else cpu_baseline()
+
+    def frac(gbs):
+        return round(gbs / HBM_PEAK_GBS, 4)
+
+    roof = {"bound": "hbm", "achieved": round(head["gbs"], 1), "peak": HBM_PEAK_GBS,
+            "unit": "GB/s", "frac": frac(head["gbs"]),
+            # FETCH_SIZE + WRITE_SIZE per launch under rocprofv3 --pmc, scaled by the
+            # HIP runtime's own copy kernel (profiles/putmem_wg_tiled_256MiB_hbm_traffic.txt)
+            "traffic": PUT_TRAFFIC_BYTES, "kernel": "rma_kernel<PUT, WG> (rocshmem_ctx_putmem_wg)",
+            "algorithmic_bytes_per_launch": head["bytes_per_step"],
+            # the same message through the other two routes
+            "putmem_wg_all_cus_gbs_nostore": round(head["gbs"], 1),
+            "putmem_wg_all_cus_frac_nostore": frac(head["gbs"]),
+            "putmem_wg_all_cus_gbs": round(head["default_ctx_gbs"], 1),
+            "putmem_wg_all_cus_frac": frac(head["default_ctx_gbs"]),
+            "host_putmem_gbs": round(head["host_putmem_gbs"], 1),
+            "host_putmem_frac": frac(head["host_putmem_gbs"]),
+            "host_getmem_gbs": round(head["host_getmem_gbs"], 1)}
+    if not a.quick:
+        ta, a2a = allc["to_all_P8_64Mi"], allc["alltoall_512x7168_bf16"]
+        dp, amo, pp = allc["dispatch_put_signal"], allc["atomic_fetch_add_16Mi"], allc["pingpong"]
+        roof.update({
+            "hbm_read_only_gbs": head["ceilings"]["read_only_gbs"],
+            "hbm_write_only_gbs": head["ceilings"]["write_only_gbs"],
+            "l2_release_ns_each_per_tile": head["release_ns_each_per_tile"],
+            "l2_release_ns_each_at_end": head["release_ns_each_at_end"],
+            "to_all_fp32_sum_gbs": ta["fp32_sum"]["gbs"], "to_all_fp32_sum_frac": ta["fp32_sum"]["frac"],
+            "to_all_fp32_max_gbs": ta["fp32_max"]["gbs"], "to_all_fp32_max_frac": ta["fp32_max"]["frac"],
+            "to_all_bf16_sum_gbs": ta["bf16_sum"]["gbs"], "to_all_bf16_sum_frac": ta["bf16_sum"]["frac"],
+            "to_all_int64_xor_gbs": ta["int64_xor"]["gbs"], "to_all_int64_xor_frac": ta["int64_xor"]["frac"],
+            "wg_reduce_fp32_sum_32_teams_gbs": ta["fp32_sum_wg_reduce_32_teams_default_ctx"]["gbs"],
+            "wg_reduce_fp32_sum_32_teams_frac": ta["fp32_sum_wg_reduce_32_teams_default_ctx"]["frac"],
+            "wg_reduce_fp32_sum_32_teams_gbs_nostore": ta["fp32_sum_wg_reduce_32_teams_nostore_ctx"]["gbs"],
+            "wg_reduce_fp32_sum_32_teams_frac_nostore": ta["fp32_sum_wg_reduce_32_teams_nostore_ctx"]["frac"],
+            "wg_reduce_fp32_sum_one_wg_per_pe_gbs": ta["fp32_sum_wg_reduce_one_wg_per_pe"]["gbs"],
+            "alltoall_gbs": a2a["gbs"], "alltoall_frac": a2a["frac"],
+            "fcollect_frac": a2a["fcollect_same_block"]["frac"],
+            "broadcast_frac": a2a["broadcast_P_blocks_from_pe0"]["frac"],
+            "dispatch_gbs": dp["default_ctx"]["gbs"], "dispatch_frac": dp["default_ctx"]["frac"],
+            "dispatch_gbs_nostore": dp["nostore_ctx"]["gbs"], "dispatch_frac_nostore": dp["nostore_ctx"]["frac"],
+            "amo_uniform_mops": amo["uniform"]["default_ctx"]["mops"],
+            "amo_uniform_mops_nostore": amo["uniform"]["nostore_ctx"]["mops"],
+            "amo_zipf_mops": amo["zipf"]["default_ctx"]["mops"],
+            "amo_zipf_mops_nostore": amo["zipf"]["nostore_ctx"]["mops"],
+            "pingpong_8B_us": pp["8"]["default_ctx"]["latency_us"],
+            "pingpong_8B_us_nostore": pp["8"]["nostore_ctx"]["latency_us"],
+            "pingpong_64KiB_us": pp["65536"]["default_ctx"]["latency_us"],
+            "pingpong_32pairs_msg_per_s": pp["8_x32pairs"]["nostore_ctx"]["msg_per_s"],
+            "barrier_all_round_us": allc["barrier_P8"]["barrier_all_round_us"],
+        })
     line = {
         "metric": "HBM GB/s (% of MI355X peak) for to_all/alltoall/putmem; atomic Mops/s",
         "value": round(head["gbs"], 1),
@@ -473,19 +588,17 @@ def main():
         "vs_baseline": None,
         "dtype": "u8",
         "data": "synthetic",
-        "config": {"workload": "bulk putmem, one 256 MiB message per step from PE k%8 to PE (k+1)%8 "
-                               "of P=8 slices in one symmetric heap, all CUs (BASELINE configs[1], "
-                               "largest size; buffers rotate so no step re-reads cached data)",
-                   "n_pes": P, "message_bytes": 256 * MiB, "heap_bytes_per_pe": 8 << 30},
-        "roofline": {"bound": "hbm", "achieved": round(head["gbs"], 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(head["gbs"] / HBM_PEAK_GBS, 4),
-                     # FETCH_SIZE + WRITE_SIZE per launch under rocprofv3 --pmc, scaled by the
-                     # HIP runtime's own copy kernel (profiles/bulk_copy_256MiB_hbm_traffic.txt)
-                     "traffic": 536869499, "kernel": "bulk_copy_kernel<true>",
-                     # measured in this run: what a pure read / pure write stream of the
-                     # same shape sustains, and the copy rate those two allow
-                     "measured_ceilings": head["ceilings"],
-                     "algorithmic_bytes_per_launch": head["bytes_per_step"]},
+        "config": {"workload": "bulk putmem through the device API: one 256 MiB message per step from PE "
+                               "k%8 to PE (k+1)%8 of P=8 slices in one symmetric heap, every CU calling "
+                               "rocshmem_ctx_putmem_wg on 16 KiB tiles (one tile per work-group of 256) "
+                               "through a ROCSHMEM_CTX_NOSTORE context, one quiet per work-group "
+                               "(BASELINE configs[1], largest size; buffers rotate so no step re-reads "
+                               "cached data)",
+                   "n_pes": P, "message_bytes": 256 * MiB, "heap_bytes_per_pe": 8 << 30,
+                   "layout": "ROCSHMEM_EMU_SPREAD=%s" % os.environ.get("ROCSHMEM_EMU_SPREAD"),
+                   "pe_stride_bytes": layout["pe_stride_bytes"],
+                   "heap_alloc_bytes": layout["heap_alloc_bytes"]},
+        "roofline": roof,
         # the reference's own convention (tests/functional_tests/tester.cpp:505-508):
         # payload bytes per second in GiB/s, counting each byte once
         "reference_convention_payload_gib_s": round(256 * MiB / (head["ms"] * 1e-3) / 2**30, 1),

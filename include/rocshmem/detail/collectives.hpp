@@ -17,14 +17,22 @@ namespace detail {
 
 #if defined(__HIPCC__)
 
-__device__ __forceinline__ void team_pad_sync(const Context *c, Team *t, int kind) {
+// What a synchronisation the user asked for publishes on context c: all of
+// the work-group's stores, unless the context was created with
+// ROCSHMEM_CTX_NOSTORE (include/rocshmem/rocshmem_common.hpp; the reference
+// switches its flush off for that option, src/fence_policy.hpp:45-63).
+__device__ __forceinline__ int publish_of(const Context *c) {
+  return (c->options & static_cast<unsigned>(ROCSHMEM_CTX_NOSTORE)) ? PUBLISH_LIBRARY : PUBLISH_ALL;
+}
+
+__device__ __forceinline__ void team_pad_sync(const Context *c, Team *t, int kind, int publish) {
   sync_pes(c, &t->sync[kind], t->wrt_world.pe_start, t->wrt_world.stride,
-           t->num_pes, t->my_pe);
+           t->num_pes, t->my_pe, publish);
 }
 
 // src/ipc/context_ipc_device_coll.cpp:101-123
 __device__ __forceinline__ void sync_all(Context *c) {
-  sync_pes(c, c->world_sync, 0, 1, c->num_pes, c->my_pe);
+  sync_pes(c, c->world_sync, 0, 1, c->num_pes, c->my_pe, publish_of(c));
 }
 __device__ __forceinline__ void barrier_all(Context *c) {
   // quiet() of the calling PE is the release half of the barrier's first step.
@@ -34,9 +42,9 @@ __device__ __forceinline__ void barrier_all(Context *c) {
 // All-reduce over the team.  Replaces the reference's direct / ring selector
 // and its two algorithms (src/ipc/context_ipc_tmpl_device.hpp:166-418) by a
 // direct reduce-scatter + all-gather in one pass: after every member has
-// arrived, member k folds the k-th chunk of all P sources in ascending member
-// order and stores the result into the k-th chunk of all P destinations; a
-// second barrier ends the operation.  Each element is computed once, so all
+// arrived, member k folds its share of the index range (every P-th block of
+// one vector per lane) from all P sources in ascending member order and stores
+// the result into all P destinations; a second barrier ends the operation.  Each element is computed once, so all
 // members hold bit-identical results.  Keeps the reference's refusal of teams
 // with 2*P > ROCSHMEM_REDUCE_SYNC_SIZE (:412-415).
 template <typename E, ROCSHMEM_OP Op>
@@ -48,27 +56,30 @@ __device__ __forceinline__ int wg_reduce(Context *c, Team *t,
   const int P = t->num_pes;
   if (static_cast<size_t>(2 * P) > ROCSHMEM_REDUCE_SYNC_SIZE) return ROCSHMEM_ERROR;
 
-  team_pad_sync(c, t, SYNC_REDUCE);
+  // Entry: every member's source, which its caller may have written with plain
+  // stores, is final.
+  team_pad_sync(c, t, SYNC_REDUCE, publish_of(c));
 
   const size_t n = static_cast<size_t>(nreduce);
-  constexpr size_t per = 16 / sizeof(S);
-  size_t chunk = (n + P - 1) / P;
-  chunk = (chunk + per - 1) / per * per;
-  size_t lo = static_cast<size_t>(t->my_pe) * chunk;
-  if (lo > n) lo = n;
-  size_t hi = lo + chunk;
-  if (hi > n) hi = n;
-
   const int64_t to_first = static_cast<int64_t>(t->wrt_world.pe_start - c->my_pe) *
                            static_cast<int64_t>(c->pe_stride);
   const int64_t hop = static_cast<int64_t>(t->wrt_world.stride) *
                       static_cast<int64_t>(c->pe_stride);
   S *dst0 = reinterpret_cast<S *>(reinterpret_cast<char *>(dest) + to_first);
   const S *src0 = reinterpret_cast<const S *>(reinterpret_cast<const char *>(source) + to_first);
-  if (hi > lo)
-    fold_span_any<E, Op, false>(dst0, src0, hop, P, lo, hi, flat_thread_id(), flat_block_size());
+  // The members share the whole range block by block (see fold_window).  Arrays
+  // that are streamed once are read and written with the non-temporal hint, as
+  // the bulk copy does.
+  const size_t part = static_cast<size_t>(t->my_pe), nparts = static_cast<size_t>(P);
+  if (n * sizeof(S) >= g_state.nt_bytes)
+    fold_span_any<E, Op, true>(dst0, src0, hop, P, 0, n, flat_thread_id(), flat_block_size(), part,
+                               nparts);
+  else
+    fold_span_any<E, Op, false>(dst0, src0, hop, P, 0, n, flat_thread_id(), flat_block_size(), part,
+                                nparts);
 
-  team_pad_sync(c, t, SYNC_REDUCE);
+  // Exit: the results were written by the fold, through to memory.
+  team_pad_sync(c, t, SYNC_REDUCE, PUBLISH_LIBRARY);
   return ROCSHMEM_SUCCESS;
 }
 
@@ -80,13 +91,13 @@ __device__ __forceinline__ int wg_reduce(Context *c, Team *t,
 __device__ __forceinline__ void wg_broadcast(Context *c, Team *t, void *dest,
                                              const void *source, size_t bytes,
                                              int pe_root) {
-  team_pad_sync(c, t, SYNC_BCAST);
+  team_pad_sync(c, t, SYNC_BCAST, publish_of(c));
   if (t->my_pe != pe_root) {
     const int root_world = t->wrt_world.pe_start + t->wrt_world.stride * pe_root;
     copy_lanes(dest, remote_addr(c, static_cast<const char *>(source), root_world),
                bytes, flat_thread_id(), flat_block_size(), g_state.nt_bytes);
   }
-  team_pad_sync(c, t, SYNC_BCAST);
+  team_pad_sync(c, t, SYNC_BCAST, PUBLISH_LIBRARY);
 }
 
 // dst_j[me*n + k] = src_me[j*n + k] for every member j, self included
@@ -101,7 +112,7 @@ __device__ __forceinline__ void wg_alltoall(Context *c, Team *t, void *dest,
     copy_lanes(remote_addr(c, d, pe), s + static_cast<size_t>(j) * block_bytes,
                block_bytes, tid, bs, g_state.nt_bytes);
   }
-  team_pad_sync(c, t, SYNC_ALLTOALL);
+  team_pad_sync(c, t, SYNC_ALLTOALL, PUBLISH_LIBRARY);
 }
 
 // dst_j[me*n + k] = src_me[k] (src/ipc/context_ipc_tmpl_device.hpp:509-531).
@@ -113,7 +124,7 @@ __device__ __forceinline__ void wg_fcollect(Context *c, Team *t, void *dest,
     const int pe = t->wrt_world.pe_start + t->wrt_world.stride * j;
     copy_lanes(remote_addr(c, d, pe), source, block_bytes, tid, bs, g_state.nt_bytes);
   }
-  team_pad_sync(c, t, SYNC_ALLTOALL);
+  team_pad_sync(c, t, SYNC_ALLTOALL, PUBLISH_LIBRARY);
 }
 
 #endif  // __HIPCC__

@@ -34,7 +34,7 @@ typedef uint32_t u32_any __attribute__((aligned(1)));
 typedef uint16_t u16_any __attribute__((aligned(1)));
 
 // Messages at least this large are moved with the non-temporal hint.
-constexpr size_t kNonTemporalBytes = size_t{64} << 10;
+constexpr size_t kNonTemporalBytes = size_t{4} << 10;
 
 // ---- write-through stores ---------------------------------------------------
 // Every store of a cooperative copy or fold goes out as a buffer store with

@@ -172,11 +172,14 @@ __device__ __forceinline__ Context *ctx_of(rocshmem_ctx_t ctx) {
 // from the queue they were dispatched on (one host thread per PE), a handle
 // may come from a variable that the PE threads share, so it is re-read as
 // "this team" and resolved to the acting PE's object: the objects of one team
-// are consecutive, indexed by world PE.
+// are consecutive, indexed by world PE.  Returns nullptr for
+// ROCSHMEM_TEAM_INVALID and for the object of a PE that is not a member;
+// callers treat that as an error instead of dereferencing it.
 __device__ __forceinline__ Team *team_of(rocshmem_team_t team) {
   Team *t = reinterpret_cast<Team *>(team);
-  if (t && g_state.pe_rule == PE_RULE_QUEUE) t = t - t->my_pe_in_world + acting_pe();
-  return t;
+  if (!t) return nullptr;
+  if (g_state.pe_rule == PE_RULE_QUEUE) t = t - t->my_pe_in_world + acting_pe();
+  return t->my_pe < 0 ? nullptr : t;
 }
 
 // Address of the same symmetric object on PE `pe`.

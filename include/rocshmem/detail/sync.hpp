@@ -362,16 +362,34 @@ __device__ __forceinline__ size_t wait_until_some(T *ivars, size_t nelems,
 // this round's epoch in member j's pad and polls member j's announcement in
 // the local pad.  (The reference's thread 0 walks the flags one by one and
 // resets them: src/ipc/context_ipc_device_coll.cpp:31-99.)
+//
+// What the arrival publishes:
+//   PUBLISH_ALL     everything the work-group has stored, plain stores
+//                   included: an agent-scope release, i.e. an L2 write-back.
+//                   On MI355X one write-back stalls its XCD's L2 for about
+//                   0.3 us whenever the kernel has loads in flight, whether or
+//                   not a line is dirty (measured: a P = 8 team reduce with a
+//                   write-back in both of its barriers loses 3 % with 32
+//                   teams on the GPU and 11 % with 128).
+//   PUBLISH_LIBRARY what the library itself has stored for the work-group
+//                   (cooperative copies and folds are write-through stores):
+//                   every wavefront waits for its own stores, no write-back.
+//                   Right for the barrier that ends a collective, whose
+//                   payload the library wrote, and for contexts created with
+//                   ROCSHMEM_CTX_NOSTORE.
+enum PublishKind : int { PUBLISH_ALL = 0, PUBLISH_LIBRARY = 1 };
+
 __device__ __forceinline__ void sync_pes(const Context *c, SyncPad *pad,
                                          int pe_start, int stride, int size,
-                                         int my_index) {
+                                         int my_index, int publish = PUBLISH_ALL) {
+  if (publish == PUBLISH_LIBRARY) drain_own_stores();
   __syncthreads();
   const unsigned tid = flat_thread_id();
   if (tid < 64u) {
     unsigned nl = flat_block_size();
     if (nl > 64u) nl = 64u;
     const unsigned long long round = load_through(&pad->epoch) + 1ull;
-    fence_release();
+    if (publish == PUBLISH_ALL) fence_release();
     for (unsigned j = tid; j < static_cast<unsigned>(size); j += nl) {
       SyncPad *peer = remote_ws(c, pad, pe_start + static_cast<int>(j) * stride);
       store_through(&peer->slots[my_index], round);

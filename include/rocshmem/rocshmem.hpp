@@ -97,8 +97,12 @@ __device__ ATTR_NO_INLINE inline int rocshmem_wg_ctx_create(int64_t options,
 __device__ ATTR_NO_INLINE inline int rocshmem_wg_team_create_ctx(rocshmem_team_t team,
                                                                  long options,
                                                                  rocshmem_ctx_t *ctx) {
-  if (team == ROCSHMEM_TEAM_INVALID) return -1;
   detail::Team *t = detail::team_of(team);
+  if (!t) {  // ROCSHMEM_TEAM_INVALID, or the acting PE is not a member
+    if (detail::is_block_leader()) *ctx = rocshmem_ctx_t{nullptr, nullptr};
+    __syncthreads();
+    return -1;
+  }
   return detail::wg_ctx_create_for(t->my_pe_in_world, &t->wrt_world, options, ctx);
 }
 __device__ ATTR_NO_INLINE inline void rocshmem_wg_ctx_destroy(rocshmem_ctx_t *ctx) {
@@ -149,6 +153,7 @@ __device__ inline int rocshmem_team_translate_pe(rocshmem_team_t src_team, int s
   if (src_team == ROCSHMEM_TEAM_INVALID || dest_team == ROCSHMEM_TEAM_INVALID) return -1;
   const detail::Team *s = detail::team_of(src_team);
   const detail::Team *d = detail::team_of(dest_team);
+  if (!s || !d) return -1;
   const int world = s->wrt_world.pe_start + s->wrt_world.stride * src_pe;
   const int off = world - d->wrt_world.pe_start;
   if (off < 0 || off % d->wrt_world.stride) return -1;
@@ -170,7 +175,11 @@ __device__ ATTR_NO_INLINE inline void rocshmem_wg_sync_all() {
 }
 __device__ ATTR_NO_INLINE inline void rocshmem_ctx_wg_team_sync(rocshmem_ctx_t ctx,
                                                                 rocshmem_team_t team) {
-  detail::team_pad_sync(detail::ctx_of(ctx), detail::team_of(team), detail::SYNC_BARRIER);
+  detail::Team *t = detail::team_of(team);
+  if (t) {
+    detail::Context *c = detail::ctx_of(ctx);
+    detail::team_pad_sync(c, t, detail::SYNC_BARRIER, detail::publish_of(c));
+  }
 }
 __device__ ATTR_NO_INLINE inline void rocshmem_wg_team_sync(rocshmem_team_t team) {
   rocshmem_ctx_wg_team_sync(rocshmem_ctx_t{nullptr, nullptr}, team);

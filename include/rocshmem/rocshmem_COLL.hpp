@@ -7,8 +7,8 @@
 //
 // Additions that have no counterpart in the reference: bf16 sums with fp32
 // accumulation (rocshmem_ctx_bf16_sum_wg_reduce) and the OpenSHMEM-style
-// aliases rocshmem_ctx_<T>_<op>_wg_to_all, rocshmem_ctx_alltoallmem_wg and
-// rocshmem_ctx_broadcastmem_wg.
+// aliases rocshmem_ctx_<T>_<op>_wg_to_all, rocshmem_ctx_alltoallmem[_wg],
+// rocshmem_ctx_broadcastmem[_wg] and rocshmem_ctx_broadcast (bytes).
 #ifndef ROCSHMEM_AMD_COLL_HPP_
 #define ROCSHMEM_AMD_COLL_HPP_
 
@@ -23,8 +23,9 @@ namespace rocshmem {
   __device__ ATTR_NO_INLINE inline int rocshmem_ctx_##TN##_##OPN##_wg_reduce(             \
       rocshmem_ctx_t ctx, rocshmem_team_t team, T *dest, const T *source, int nreduce) {  \
     if (nreduce == 0) return ROCSHMEM_SUCCESS;                                            \
-    return detail::wg_reduce<T, OP>(detail::ctx_of(ctx), detail::team_of(team), dest,     \
-                                    source, nreduce);                                     \
+    detail::Team *t = detail::team_of(team);                                              \
+    if (!t) return ROCSHMEM_ERROR;                                                        \
+    return detail::wg_reduce<T, OP>(detail::ctx_of(ctx), t, dest, source, nreduce);       \
   }                                                                                       \
   __device__ ATTR_NO_INLINE inline int rocshmem_ctx_##TN##_##OPN##_wg_to_all(             \
       rocshmem_ctx_t ctx, rocshmem_team_t team, T *dest, const T *source, int nreduce) {  \
@@ -52,8 +53,10 @@ __device__ ATTR_NO_INLINE inline int rocshmem_ctx_bf16_sum_wg_reduce(
     rocshmem_ctx_t ctx, rocshmem_team_t team, rocshmem_bf16 *dest,
     const rocshmem_bf16 *source, int nreduce) {
   if (nreduce == 0) return ROCSHMEM_SUCCESS;
+  detail::Team *t = detail::team_of(team);
+  if (!t) return ROCSHMEM_ERROR;
   return detail::wg_reduce<detail::Bf16Tag, ROCSHMEM_SUM>(
-      detail::ctx_of(ctx), detail::team_of(team), reinterpret_cast<uint16_t *>(dest),
+      detail::ctx_of(ctx), t, reinterpret_cast<uint16_t *>(dest),
       reinterpret_cast<const uint16_t *>(source), nreduce);
 }
 __device__ ATTR_NO_INLINE inline int rocshmem_ctx_bf16_sum_wg_to_all(
@@ -66,21 +69,46 @@ __device__ ATTR_NO_INLINE inline int rocshmem_ctx_bf16_sum_wg_to_all(
 __device__ ATTR_NO_INLINE inline void rocshmem_ctx_alltoallmem_wg(
     rocshmem_ctx_t ctx, rocshmem_team_t team, void *dest, const void *source,
     size_t nelems) {
-  if (nelems == 0) return;
-  detail::wg_alltoall(detail::ctx_of(ctx), detail::team_of(team), dest, source, nelems);
+  detail::Team *t = detail::team_of(team);
+  if (nelems == 0 || !t) return;  // not a member of `team`: nothing to take part in
+  detail::wg_alltoall(detail::ctx_of(ctx), t, dest, source, nelems);
 }
 __device__ ATTR_NO_INLINE inline void rocshmem_ctx_broadcastmem_wg(
     rocshmem_ctx_t ctx, rocshmem_team_t team, void *dest, const void *source,
     size_t nelems, int pe_root) {
-  if (nelems == 0) return;
-  detail::wg_broadcast(detail::ctx_of(ctx), detail::team_of(team), dest, source, nelems,
-                       pe_root);
+  detail::Team *t = detail::team_of(team);
+  if (nelems == 0 || !t) return;
+  detail::wg_broadcast(detail::ctx_of(ctx), t, dest, source, nelems, pe_root);
 }
 __device__ ATTR_NO_INLINE inline void rocshmem_ctx_fcollectmem_wg(
     rocshmem_ctx_t ctx, rocshmem_team_t team, void *dest, const void *source,
     size_t nelems) {
-  if (nelems == 0) return;
-  detail::wg_fcollect(detail::ctx_of(ctx), detail::team_of(team), dest, source, nelems);
+  detail::Team *t = detail::team_of(team);
+  if (nelems == 0 || !t) return;
+  detail::wg_fcollect(detail::ctx_of(ctx), t, dest, source, nelems);
+}
+
+// The same three under the OpenSHMEM 1.5 spellings (no granularity suffix):
+// still work-group calls, every thread of the work-group with equal arguments.
+__device__ inline void rocshmem_ctx_alltoallmem(rocshmem_ctx_t ctx, rocshmem_team_t team,
+                                                void *dest, const void *source,
+                                                size_t nelems) {
+  rocshmem_ctx_alltoallmem_wg(ctx, team, dest, source, nelems);
+}
+__device__ inline void rocshmem_ctx_broadcastmem(rocshmem_ctx_t ctx, rocshmem_team_t team,
+                                                 void *dest, const void *source, size_t nelems,
+                                                 int pe_root) {
+  rocshmem_ctx_broadcastmem_wg(ctx, team, dest, source, nelems, pe_root);
+}
+__device__ inline void rocshmem_ctx_broadcast(rocshmem_ctx_t ctx, rocshmem_team_t team,
+                                              void *dest, const void *source, size_t nelems,
+                                              int pe_root) {
+  rocshmem_ctx_broadcastmem_wg(ctx, team, dest, source, nelems, pe_root);
+}
+__device__ inline void rocshmem_ctx_fcollectmem(rocshmem_ctx_t ctx, rocshmem_team_t team,
+                                                void *dest, const void *source,
+                                                size_t nelems) {
+  rocshmem_ctx_fcollectmem_wg(ctx, team, dest, source, nelems);
 }
 
 #define ROCSHMEM_AMD_COLL(T, TN)                                                          \

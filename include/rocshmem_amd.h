@@ -144,6 +144,11 @@ size_t rocshmem_amd_heap_size(void);
 size_t rocshmem_amd_heap_used(void);
 size_t rocshmem_amd_heap_avail(void);
 size_t rocshmem_amd_pe_stride(void);
+/* Bytes of the one device allocation that holds the P slices (no reference
+ * counterpart: there every PE allocates its own heap, src/memory/heap_memory.hpp).
+ * pe_stride x P by default (stride = heap size rounded up to 2 MiB);
+ * ROCSHMEM_EMU_SPREAD=1 spreads the slices over half of the device memory. */
+size_t rocshmem_amd_heap_alloc_bytes(void);
 
 /* The allocator on its own, usable without a GPU (planning and host-side
  * tests): a model heap of heap_bytes whose base has the alignment of
@@ -173,6 +178,22 @@ rocshmem_amd_team_t rocshmem_amd_team_on(rocshmem_amd_team_t team, int pe);
 /* World PEs of a team: PE_start, PE_start + PE_stride, ... (PE_size of them). */
 int rocshmem_amd_team_active_set(rocshmem_amd_team_t team, int *PE_start, int *PE_stride,
                                  int *PE_size);
+/* Launch rules of the drivers whose work-groups wait for each other (wg_reduce,
+ * wg_reduce_teams, wg_alltoall / broadcast / fcollect, wg_sync, pingpong,
+ * put_flag_check, wait_test_woken).  No reference counterpart: the reference
+ * leaves co-residency to the caller (its barriers spin without bound,
+ * src/ipc/context_ipc_device_coll.cpp:31-99).  Such a grid is launched only if
+ * all of it can be resident at once, n_wgs <= wgs_per_cu x n_cus with
+ * wgs_per_cu from hipOccupancyMaxActiveBlocksPerMultiprocessor for the kernel
+ * and work-group size; otherwise the driver returns -1 and launches nothing.
+ * This is that arithmetic (1 = fits). */
+int rocshmem_amd_coresident(long n_wgs, int wgs_per_cu, int n_cus);
+/* With one host thread per PE (rocshmem_emu_run_pes) every stream a PE thread
+ * launches on needs a hardware queue of its own, plus one for the library:
+ * 1 if pe_streams + 1 <= hw_queues (GPU_MAX_HW_QUEUES, HIP's default 4).
+ * rocshmem_init and the stream binding end the process with a message,
+ * before enqueueing anything, when this is 0. */
+int rocshmem_amd_hw_queues_suffice(size_t pe_streams, size_t hw_queues);
 /* Meeting point of the host collectives when every PE is a thread of this
  * process (rocshmem_emu_run_pes, include/rocshmem/rocshmem_emu.hpp; the
  * reference's PEs are processes that meet inside MPI).  Each member of the
@@ -184,6 +205,7 @@ int rocshmem_amd_pe_threads_enter(int PE_start, int PE_stride, int PE_size);
 void rocshmem_amd_pe_threads_leave(int PE_start, int PE_stride, int PE_size);
 
 /* Plain device memory and staging for callers without a HIP binding. */
+int rocshmem_amd_dev_mem_info(size_t *free_bytes, size_t *total_bytes); /* hipMemGetInfo */
 void *rocshmem_amd_dev_alloc(size_t size);
 int rocshmem_amd_dev_free(void *ptr);
 int rocshmem_amd_copy_in(void *dst_dev, const void *src_host, size_t n);
@@ -195,6 +217,17 @@ int rocshmem_amd_fill(void *dst_dev, int byte, size_t n);
  * else — the one-directional rate of the memory system that a copy is judged
  * against. */
 int rocshmem_amd_hbm_probe(int write, void *buf, size_t nbytes, rocshmem_amd_stream_t stream);
+/* Measurement aid (no reference counterpart): what one agent-scope release —
+ * the L2 write-back that rocshmem_ctx_quiet / fence and every barrier perform
+ * on a default context — costs while a copy is running.  n_wgs work-groups of
+ * wg_size threads copy nbytes from src to dst in tiles of tile_bytes (tile t
+ * to work-group t mod n_wgs) with the cooperative copy of putmem_wg and issue a
+ * release never (mode 0), once per work-group at its end (mode 1) or after
+ * every tile (mode 2).  Time modes 1 / 2 against mode 0 and divide by the
+ * number of releases. */
+int rocshmem_amd_release_probe(int mode, void *dst, const void *src, size_t nbytes,
+                               size_t tile_bytes, int n_wgs, int wg_size,
+                               rocshmem_amd_stream_t stream);
 /* The symmetric object `sym` (address on PE 0) set to `byte` on every PE with
  * one launch on `stream` — e.g. signal words cleared between dispatches. */
 int rocshmem_amd_fill_every_pe(void *sym, int byte, size_t n, rocshmem_amd_stream_t stream);
@@ -250,15 +283,19 @@ int rocshmem_amd_wf_coalesce(const int *pe, const uint64_t *src, const uint64_t 
 int rocshmem_amd_wg_reduce(int dtype, int op, rocshmem_amd_team_t team, void *dest,
                            const void *source, int nreduce, int wg_size,
                            rocshmem_amd_stream_t stream);
-/* The same call made by n_teams (<= 64) work-groups per PE at once, each with a
+/* The same call made by n_teams (<= 256) work-groups per PE at once, each with a
  * team of its own over the same PEs — how the reference's testers spread a
  * device collective over the GPU (one team per work-group,
  * tests/functional_tests/team_reduction_tester.cpp:60-110).  Team t reduces
  * the t-th slice of the arrays (equal slices, whole 16-byte vectors).  teams:
- * host array of handles of distinct teams with the same members. */
+ * host array of handles of distinct teams with the same members.  Every
+ * work-group makes the call `iters` (>= 1) times in a row inside the kernel, as
+ * the reference's testers loop inside theirs.  Returns the largest device
+ * status any team saw, after waiting for the kernel; -1 if nothing was
+ * launched (bad argument, or the grid n_teams x P cannot be resident at once). */
 int rocshmem_amd_wg_reduce_teams(int dtype, int op, const rocshmem_amd_team_t *teams, int n_teams,
                                  void *dest, const void *source, int nreduce, int wg_size,
-                                 rocshmem_amd_stream_t stream);
+                                 int iters, rocshmem_amd_stream_t stream);
 /* rocshmem_ctx_<T>_wg_alltoall / _wg_broadcast / _wg_fcollect
  * (rocshmem_COLL.hpp:44-258; context_ipc_tmpl_device.hpp:420-531).
  * elem_size in {1,2,4,8} selects the typed entry point (char/short/int/long). */
@@ -427,11 +464,19 @@ int rocshmem_amd_pingpong(void *buf, uint64_t *sig, size_t nbytes, int iters, in
  * rocshmem_ulong_wait_until(sig[s], GE, count[s*P+d]) for every s.
  * count/send_row/recv_row: host arrays of P*P uint32 (a device copy is kept
  * and reused while consecutive calls pass the same tables).  send/recv/sig:
- * addresses on PE 0.  sig must be zero when the kernel starts. */
+ * addresses on PE 0.
+ * expect == NULL: sig must be zero when the kernel starts.  Otherwise expect is
+ * P*P uint64 of device memory that the caller zeroes once together with sig:
+ * the receivers keep in expect[d*P+s] the total they have waited for on d's
+ * word s and wait for that total plus this dispatch's count, so the signal
+ * words just keep growing and one dispatch follows the other with nothing to
+ * clear in between (how an application that dispatches every step uses
+ * ROCSHMEM_SIGNAL_ADD with rocshmem_wait_until(..., GE, running total),
+ * examples/rocshmem_put_signal_test.cc:31-47). */
 int rocshmem_amd_dispatch_put_signal(void *recv, const void *send, uint64_t *sig,
                                      const uint32_t *count, const uint32_t *send_row,
                                      const uint32_t *recv_row, size_t row_bytes,
-                                     int rows_per_call, int wg_size,
+                                     int rows_per_call, int wg_size, uint64_t *expect,
                                      rocshmem_amd_stream_t stream);
 
 /* rocshmem_<T>_test / _wait_until / _wait_until_any / _all / _some
@@ -440,8 +485,9 @@ int rocshmem_amd_dispatch_put_signal(void *recv, const void *send, uint64_t *sig
  * points at one host element of dtype.  ret_out: the function's return value
  * (test: 0/1; any: index or SIZE_MAX; some: count; others 0); indices_out
  * (host, nelems entries, optional) receives wait_until_some's indices.
- * Blocking forms return only once satisfied: use them on values that already
- * hold, or with the waker below. */
+ * A blocking form whose condition does not hold yet would spin for ever (there
+ * is nobody to change ivars): it is refused with -2 and nothing is launched;
+ * use the waker below for those. */
 int rocshmem_amd_wait_test(int wait_fn, int dtype, void *ivars, size_t nelems,
                            const int *status, int cmp, const void *value,
                            size_t *ret_out, size_t *indices_out);

@@ -37,6 +37,17 @@ int64_t rocshmem_amd_set_ctx_options(int64_t options) {
   rt().driver_ctx_options = options;
   return before;
 }
+int rocshmem_amd_coresident(long n_wgs, int wgs_per_cu, int n_cus) {
+  return rocshmem::drv::coresident(n_wgs, wgs_per_cu, n_cus) ? 1 : 0;
+}
+int rocshmem_amd_hw_queues_suffice(size_t pe_streams, size_t hw_queues) {
+  return rocshmem::runtime::hw_queues_suffice(pe_streams, hw_queues) ? 1 : 0;
+}
+int rocshmem_amd_dev_mem_info(size_t *free_bytes, size_t *total_bytes) {
+  if (!free_bytes || !total_bytes) return -1;
+  return hipMemGetInfo(free_bytes, total_bytes) == hipSuccess ? 0 : -1;
+}
+size_t rocshmem_amd_heap_alloc_bytes(void) { return rt().live ? rt().heap_alloc_bytes : 0; }
 int rocshmem_amd_pe_threads_enter(int PE_start, int PE_stride, int PE_size) {
   return rocshmem::runtime::pe_threads_enter(PE_start, PE_stride, PE_size, nullptr) ? 1 : 0;
 }

@@ -1,5 +1,7 @@
 // Drivers for collectives: the per-work-group device API (one work-group per
 // team member) and the host-called whole-GPU forms.
+#include <mutex>
+
 #include "drv_common.hpp"
 #include "rocshmem_amd.h"
 
@@ -87,7 +89,7 @@ __global__ void wg_reduce_kernel(WgCollArgs a) {
 // scale a device collective (one team per work-group,
 // tests/functional_tests/team_reduction_tester.cpp): work-group (x, y) acts
 // for member x of team y and reduces the y-th slice of the arrays.
-constexpr int kMaxTeamsPerLaunch = 64;
+constexpr int kMaxTeamsPerLaunch = 256;
 struct WgTeamsArgs {
   detail::Team *rows[kMaxTeamsPerLaunch];  // team objects of each team, indexed by world PE
   detail::Context *ctx_row;
@@ -98,7 +100,8 @@ struct WgTeamsArgs {
   int stride;
   int nelems;       // all slices together
   int slice_elems;  // per team
-  int *status;
+  int iters;        // calls per work-group, one after the other
+  int *status;      // [teams] largest return code each team saw
 };
 
 template <typename T, ROCSHMEM_OP Op>
@@ -113,8 +116,10 @@ __global__ void wg_reduce_teams_kernel(WgTeamsArgs a) {
   if (cnt < 0) cnt = 0;
   T *dest = reinterpret_cast<T *>(a.dest0 + static_cast<uint64_t>(pe) * a.pe_stride) + lo;
   const T *source = reinterpret_cast<const T *>(a.src0 + static_cast<uint64_t>(pe) * a.pe_stride) + lo;
-  const int rc = PublicReduce<T, Op>::call(ctx, team, dest, source, static_cast<int>(cnt));
-  if (threadIdx.x == 0 && rc != ROCSHMEM_SUCCESS) atomicMax(a.status, rc);
+  for (int it = 0; it < a.iters; ++it) {
+    const int rc = PublicReduce<T, Op>::call(ctx, team, dest, source, static_cast<int>(cnt));
+    if (threadIdx.x == 0 && rc != ROCSHMEM_SUCCESS) atomicMax(a.status + blockIdx.y, rc);
+  }
 }
 
 enum WgMove { MOVE_ALLTOALL, MOVE_BROADCAST, MOVE_FCOLLECT };
@@ -362,8 +367,10 @@ inline bool in_heap(const void *p) {
 }
 
 template <typename T, ROCSHMEM_OP Op>
-void launch_wg_reduce(const WgCollArgs &a, int size, int wg_size, hipStream_t s) {
+bool launch_wg_reduce(const WgCollArgs &a, int size, int wg_size, hipStream_t s) {
+  if (!grid_fits(wg_reduce_kernel<T, Op>, size, wg_size)) return false;
   hipLaunchKernelGGL((wg_reduce_kernel<T, Op>), dim3(size), dim3(wg_size), 0, s, a);
+  return true;
 }
 
 }  // namespace drv
@@ -443,7 +450,7 @@ WgCollArgs make_wg_args(const TeamView &v, void *dest, const void *source, int n
   auto &r = runtime::rt();
   WgCollArgs a;
   a.team_row = v.row;
-  a.ctx_row = r.d_default_ctx;
+  a.ctx_row = r.driver_ctx_row();
   a.dest0 = on_pe0(dest);
   a.src0 = on_pe0(source);
   a.pe_stride = r.pe_stride;
@@ -470,13 +477,19 @@ int wg_move_common(int elem_size, rocshmem_amd_team_t team, void *dest, const vo
   if (kMove == MOVE_BROADCAST && (root < 0 || root >= v.host->num_pes)) return -1;
   const WgCollArgs a = make_wg_args(v, dest, source, nelems, root, nullptr);
   const dim3 g(v.host->num_pes), b(wg_size);
+#define DRV_MOVE_CASE(BYTES, T)                                              \
+  case BYTES:                                                                \
+    if (!grid_fits(wg_move_kernel<T, kMove>, g.x, wg_size)) return -1;       \
+    hipLaunchKernelGGL((wg_move_kernel<T, kMove>), g, b, 0, s, a);           \
+    break;
   switch (elem_size) {
-    case 1: hipLaunchKernelGGL((wg_move_kernel<char, kMove>), g, b, 0, s, a); break;
-    case 2: hipLaunchKernelGGL((wg_move_kernel<short, kMove>), g, b, 0, s, a); break;
-    case 4: hipLaunchKernelGGL((wg_move_kernel<int, kMove>), g, b, 0, s, a); break;
-    case 8: hipLaunchKernelGGL((wg_move_kernel<long, kMove>), g, b, 0, s, a); break;
+    DRV_MOVE_CASE(1, char)
+    DRV_MOVE_CASE(2, short)
+    DRV_MOVE_CASE(4, int)
+    DRV_MOVE_CASE(8, long)
     default: return -1;
   }
+#undef DRV_MOVE_CASE
   DRV_CHECK_HIP(hipGetLastError());
   return 0;
 }
@@ -520,12 +533,13 @@ int rocshmem_amd_wg_reduce(int dtype, int op, rocshmem_amd_team_t team, void *de
   DRV_CHECK_HIP(hipMemset(d_status, 0, sizeof(int)));
   const WgCollArgs a = make_wg_args(v, dest, source, nreduce, 0, d_status);
   hipStream_t s = as_stream(stream);
+  bool launched = false;
   const bool ok = for_dtype_op(dtype, op, [&](auto *tag, auto opc) {
     using T = typename std::remove_pointer<decltype(tag)>::type;
-    launch_wg_reduce<T, decltype(opc)::value>(a, v.host->num_pes, wg_size, s);
+    launched = launch_wg_reduce<T, decltype(opc)::value>(a, v.host->num_pes, wg_size, s);
   });
   int status = -1;
-  if (ok) {
+  if (ok && launched) {
     DRV_CHECK_HIP(hipGetLastError());
     DRV_CHECK_HIP(hipStreamSynchronize(s));
     DRV_CHECK_HIP(hipMemcpy(&status, d_status, sizeof(int), hipMemcpyDeviceToHost));
@@ -534,11 +548,13 @@ int rocshmem_amd_wg_reduce(int dtype, int op, rocshmem_amd_team_t team, void *de
   return status;
 }
 
-int rocshmem_amd_wg_reduce_teams(int dtype, int op, const rocshmem_amd_team_t *teams, int n_teams,
-                                 void *dest, const void *source, int nreduce, int wg_size,
-                                 rocshmem_amd_stream_t stream) {
+// Validates and enqueues the many-teams reduce; d_status: n_teams zeroed device
+// words.  0 = enqueued, -1 = refused (nothing enqueued).
+static int enqueue_reduce_teams(int dtype, int op, const rocshmem_amd_team_t *teams, int n_teams,
+                                void *dest, const void *source, int nreduce, int wg_size,
+                                int iters, int *d_status, hipStream_t s) {
   if (!teams || n_teams < 1 || n_teams > kMaxTeamsPerLaunch || !valid_launch(1, wg_size) ||
-      nreduce < 0)
+      nreduce < 0 || iters < 1)
     return -1;
   TeamView first;
   if (!view_team(teams[0], &first)) return -1;
@@ -559,10 +575,7 @@ int rocshmem_amd_wg_reduce_teams(int dtype, int op, const rocshmem_amd_team_t *t
     if (!es || !sym_ok_on(dest, bytes, me) || !sym_ok_on(source, bytes, me)) return -1;
   }
   auto &r = runtime::rt();
-  int *d_status;
-  DRV_CHECK_HIP(hipMalloc(&d_status, sizeof(int)));
-  DRV_CHECK_HIP(hipMemset(d_status, 0, sizeof(int)));
-  a.ctx_row = r.d_default_ctx;
+  a.ctx_row = r.driver_ctx_row();
   a.dest0 = on_pe0(dest);
   a.src0 = on_pe0(source);
   a.pe_stride = r.pe_stride;
@@ -574,18 +587,38 @@ int rocshmem_amd_wg_reduce_teams(int dtype, int op, const rocshmem_amd_team_t *t
   int slice = (nreduce + n_teams - 1) / n_teams;
   slice = (slice + per_vec - 1) / per_vec * per_vec;
   a.slice_elems = slice > 0 ? slice : per_vec;
+  a.iters = iters;
   a.status = d_status;
-  hipStream_t s = as_stream(stream);
   const dim3 grid(first.host->num_pes, n_teams), block(wg_size);
+  bool launched = false;
   const bool ok = for_dtype_op(dtype, op, [&](auto *tag, auto opc) {
     using T = typename std::remove_pointer<decltype(tag)>::type;
+    if (!grid_fits(wg_reduce_teams_kernel<T, decltype(opc)::value>,
+                   static_cast<long>(grid.x) * grid.y, wg_size))
+      return;
     hipLaunchKernelGGL((wg_reduce_teams_kernel<T, decltype(opc)::value>), grid, block, 0, s, a);
+    launched = true;
   });
-  int status = -1;
-  if (ok) {
-    DRV_CHECK_HIP(hipGetLastError());
+  if (!ok || !launched) return -1;
+  DRV_CHECK_HIP(hipGetLastError());
+  return 0;
+}
+
+int rocshmem_amd_wg_reduce_teams(int dtype, int op, const rocshmem_amd_team_t *teams, int n_teams,
+                                 void *dest, const void *source, int nreduce, int wg_size,
+                                 int iters, rocshmem_amd_stream_t stream) {
+  if (n_teams < 1 || n_teams > kMaxTeamsPerLaunch) return -1;
+  hipStream_t s = as_stream(stream);
+  int *d_status;
+  DRV_CHECK_HIP(hipMalloc(&d_status, sizeof(int) * n_teams));
+  DRV_CHECK_HIP(hipMemsetAsync(d_status, 0, sizeof(int) * n_teams, s));
+  int status = enqueue_reduce_teams(dtype, op, teams, n_teams, dest, source, nreduce, wg_size,
+                                    iters, d_status, s);
+  if (status == 0) {
+    int seen[kMaxTeamsPerLaunch];
     DRV_CHECK_HIP(hipStreamSynchronize(s));
-    DRV_CHECK_HIP(hipMemcpy(&status, d_status, sizeof(int), hipMemcpyDeviceToHost));
+    DRV_CHECK_HIP(hipMemcpy(seen, d_status, sizeof(int) * n_teams, hipMemcpyDeviceToHost));
+    for (int t = 0; t < n_teams; ++t) status = seen[t] > status ? seen[t] : status;
   }
   DRV_CHECK_HIP(hipFree(d_status));
   return status;
@@ -621,12 +654,13 @@ int rocshmem_amd_wg_sync(int sync_fn, rocshmem_amd_team_t team, uint64_t *scratc
   } else {
     if (!view_team(r.team_handle(0, r.me()), &v)) return -1;
   }
+  if (!grid_fits(wg_sync_kernel, v.host->num_pes, wg_size)) return -1;
   int *d_err;
   DRV_CHECK_HIP(hipMalloc(&d_err, sizeof(int)));
   DRV_CHECK_HIP(hipMemset(d_err, 0, sizeof(int)));
   SyncArgs a;
   a.team_row = v.row;
-  a.ctx_row = r.d_default_ctx;
+  a.ctx_row = r.driver_ctx_row();
   a.scratch0 = reinterpret_cast<uint64_t *>(on_pe0(scratch));
   a.pe_stride = r.pe_stride;
   a.pe_start = v.host->wrt_world.pe_start;

@@ -54,6 +54,43 @@ inline bool local_ok(const void *p, size_t bytes) {
   return true;
 }
 
+// ---- co-residency of grids whose work-groups wait for each other --------------
+// A barrier, a ping-pong or a reduce between work-groups only ends if all of
+// them are on the GPU at the same time: a work-group that has not been
+// scheduled cannot answer, and the ones that wait for it never leave.  The
+// drivers of such kernels therefore refuse (return -1, nothing launched) a
+// grid larger than what the device holds resident for that kernel and
+// work-group size.  The bound is for a GPU that runs nothing else.
+inline bool coresident(long n_wgs, int wgs_per_cu, int n_cus) {
+  return n_wgs >= 0 && wgs_per_cu > 0 && n_cus > 0 &&
+         n_wgs <= static_cast<long>(wgs_per_cu) * static_cast<long>(n_cus);
+}
+inline int device_cu_count() {
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  return cus;
+}
+template <typename Kernel>
+inline bool grid_fits(Kernel kernel, long n_wgs, int wg_size, size_t dynamic_lds = 0) {
+  int per_cu = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, wg_size, dynamic_lds) !=
+      hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  const bool ok = coresident(n_wgs, per_cu, device_cu_count());
+  if (!ok)
+    fprintf(stderr,
+            "rocshmem: refused a launch of %ld work-groups of %d threads that wait for each "
+            "other: the GPU holds %d per CU on %d CUs at once\n",
+            n_wgs, wg_size, per_cu, device_cu_count());
+  return ok;
+}
+
 // Bytes per tile when the caller leaves the choice to the driver: an equal
 // share per group, rounded up to 16 bytes.
 inline size_t auto_tile(size_t nbytes, size_t groups) {

@@ -156,6 +156,29 @@ __global__ void probe_write_kernel(char *dst, size_t nvec) {
   if (i < nvec) detail::store16<true>(w, static_cast<uint32_t>(threadIdx.x << 4), v);
 }
 
+// What an agent-scope release (the L2 write-back behind quiet and fence on a
+// default context) costs in the middle of a copy: work-groups loop over tiles
+// with the cooperative copy and release never (mode 0), once at their end
+// (mode 1) or after every tile (mode 2).  The difference to mode 0, divided by
+// the number of releases, is the cost of one.
+template <int kMode>
+__global__ void release_probe_kernel(char *dst, const char *src, size_t n, size_t tile) {
+  const size_t ntiles = (n + tile - 1) / tile;
+  for (size_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
+    const size_t off = t * tile;
+    const size_t len = n - off < tile ? n - off : tile;
+    detail::copy_lanes(dst + off, src + off, len, threadIdx.x, blockDim.x, 0);
+    if constexpr (kMode == 2) {
+      __syncthreads();
+      if (threadIdx.x == 0) detail::fence_release();
+    }
+  }
+  if constexpr (kMode == 1) {
+    __syncthreads();
+    if (threadIdx.x == 0) detail::fence_release();
+  }
+}
+
 // The same byte range of every PE's slice set to one value: blockIdx.y is the PE.
 __global__ void fill_every_pe_kernel(char *base, uint64_t pe_stride, size_t nbytes, int byte) {
   char *p = base + static_cast<uint64_t>(blockIdx.y) * pe_stride;
@@ -245,6 +268,24 @@ int rocshmem_amd_hbm_probe(int write, void *buf, size_t nbytes, rocshmem_amd_str
   else
     hipLaunchKernelGGL(probe_read_kernel, dim3(grid), dim3(kProbeThreads), 0, as_stream(stream),
                        static_cast<const char *>(buf), nvec, sink);
+  DRV_CHECK_HIP(hipGetLastError());
+  return 0;
+}
+
+int rocshmem_amd_release_probe(int mode, void *dst, const void *src, size_t nbytes,
+                               size_t tile_bytes, int n_wgs, int wg_size,
+                               rocshmem_amd_stream_t stream) {
+  if (!runtime::rt().live || !dst || !src || !nbytes || tile_bytes < 16 || mode < 0 || mode > 2 ||
+      !valid_launch(n_wgs, wg_size))
+    return -1;
+  if (!local_ok(dst, nbytes) || !local_ok(src, nbytes)) return -1;
+  const dim3 g(n_wgs), b(wg_size);
+  hipStream_t s = as_stream(stream);
+  char *d = static_cast<char *>(dst);
+  const char *c = static_cast<const char *>(src);
+  if (mode == 0) hipLaunchKernelGGL(release_probe_kernel<0>, g, b, 0, s, d, c, nbytes, tile_bytes);
+  else if (mode == 1) hipLaunchKernelGGL(release_probe_kernel<1>, g, b, 0, s, d, c, nbytes, tile_bytes);
+  else hipLaunchKernelGGL(release_probe_kernel<2>, g, b, 0, s, d, c, nbytes, tile_bytes);
   DRV_CHECK_HIP(hipGetLastError());
   return 0;
 }

@@ -397,6 +397,7 @@ struct DispatchArgs {
   uint32_t n_calls;
   detail::Context *ctx_row;
   detail::Team *world_row;
+  uint64_t *expect;     // [P*P], [d*P+s]: what d's signal word s has been waited up to; may be null
 };
 
 // Work-groups walk the list of all calls (a call = up to rows_per_call rows of
@@ -427,10 +428,18 @@ __global__ void dispatch_kernel(DispatchArgs a) {
     const int d = blockIdx.x - senders;
     uint64_t *sig_d = reinterpret_cast<uint64_t *>(reinterpret_cast<char *>(a.sig0) +
                                                    static_cast<uint64_t>(d) * a.pe_stride);
-    // Lane s of the receiver waits for sender s.
-    for (int s = threadIdx.x; s < P; s += blockDim.x)
-      rocshmem_ulong_wait_until(reinterpret_cast<unsigned long *>(sig_d + s), ROCSHMEM_CMP_GE,
-                                static_cast<unsigned long>(a.count[s * P + d]));
+    // Lane s of the receiver waits for sender s.  The signal words only ever
+    // grow: with `expect` the receiver keeps, per word, the total it has
+    // waited for so far, as an application that dispatches every step would,
+    // and nobody has to clear the words between dispatches.
+    for (int s = threadIdx.x; s < P; s += blockDim.x) {
+      unsigned long target = a.count[s * P + d];
+      if (a.expect) {
+        target += a.expect[d * P + s];
+        a.expect[d * P + s] = target;
+      }
+      rocshmem_ulong_wait_until(reinterpret_cast<unsigned long *>(sig_d + s), ROCSHMEM_CMP_GE, target);
+    }
   }
 }
 
@@ -574,10 +583,52 @@ bool for_wait_dtype(int dtype, Fn &&fn) {
   return for_amo_dtype(dtype, fn);
 }
 
+// Comparator table of rocshmem_<T>_test on the host (src/context_tmpl_device.hpp:337-377).
+template <typename T>
+bool host_compare(T x, int cmp, T val) {
+  switch (cmp) {
+    case ROCSHMEM_CMP_EQ: return x == val;
+    case ROCSHMEM_CMP_NE: return x != val;
+    case ROCSHMEM_CMP_GT: return x > val;
+    case ROCSHMEM_CMP_GE: return x >= val;
+    case ROCSHMEM_CMP_LT: return x < val;
+    case ROCSHMEM_CMP_LE: return x <= val;
+    default: return false;
+  }
+}
+
+// Would the blocking call return without anybody changing ivars?  Read on the
+// host from the values as they are now.
+template <typename T>
+bool wait_already_satisfied(int wait_fn, const T *ivars_dev, size_t nelems, const int *status,
+                            int cmp, T value) {
+  const size_t n = wait_fn == ROCSHMEM_AMD_WAIT_UNTIL ? 1 : nelems;
+  if (!n) return true;  // the vector forms return at once for an empty vector
+  std::vector<T> now(n);
+  DRV_CHECK_HIP(hipMemcpy(now.data(), ivars_dev, n * sizeof(T), hipMemcpyDeviceToHost));
+  if (wait_fn == ROCSHMEM_AMD_WAIT_UNTIL) return host_compare(now[0], cmp, value);
+  size_t unmasked = 0, holding = 0;
+  for (size_t i = 0; i < n; ++i) {
+    if (status && status[i]) continue;
+    ++unmasked;
+    holding += host_compare(now[i], cmp, value) ? 1 : 0;
+  }
+  if (!unmasked) return true;
+  return wait_fn == ROCSHMEM_AMD_WAIT_UNTIL_ALL ? holding == unmasked : holding > 0;
+}
+
 template <typename T>
 int run_wait(int wait_fn, void *ivars, size_t nelems, const int *status, int cmp,
              const void *value, int woken, size_t wake_index, const void *wake_value,
              uint64_t delay_ticks, size_t *ret_out, size_t *indices_out) {
+  if (!local_ok(ivars, (nelems ? nelems : 1) * sizeof(T))) return -1;
+  // A blocking form with nobody to wake it would spin for ever on a condition
+  // that does not hold yet: refused, nothing launched.
+  if (!woken && wait_fn != ROCSHMEM_AMD_TEST &&
+      !wait_already_satisfied<T>(wait_fn, static_cast<const T *>(ivars), nelems, status, cmp,
+                                 *static_cast<const T *>(value)))
+    return -2;
+  if (woken && !grid_fits(wait_kernel<T>, 2, 64)) return -1;
   WaitArgs<T> a;
   a.fn = wait_fn;
   a.ivars = static_cast<T *>(ivars);
@@ -708,6 +759,7 @@ int rocshmem_amd_pingpong(void *buf, uint64_t *sig, size_t nbytes, int iters, in
   const size_t slot = (nbytes + 255) / 256 * 256;
   if (!sym_ok_on(buf, slot * (pairs - 1) + nbytes, pe_a) || !sym_ok_on(sig, 8u * pairs, pe_a))
     return -1;
+  if (!grid_fits(pingpong_kernel, 2L * pairs, wg_size)) return -1;
   auto &r = runtime::rt();
   unsigned long long *d_ticks;
   DRV_CHECK_HIP(hipMalloc(&d_ticks, sizeof(unsigned long long) * pairs));
@@ -755,6 +807,7 @@ int rocshmem_amd_put_flag_check(void *data, uint64_t *flags, size_t nbytes, int 
   const size_t total = nbytes * static_cast<size_t>(pairs);
   if (!sym_ok_on(data, total, pe_a) || !sym_ok_on(flags, 16u * pairs, pe_a)) return -1;
   if (!mismatches_out || !timed_out_out) return -1;
+  if (!grid_fits(put_flag_kernel, 2L * pairs, wg_size)) return -1;
   const int64_t a_to_b = static_cast<int64_t>(pe_b - pe_a) * static_cast<int64_t>(r.pe_stride);
   uint32_t *staging;
   unsigned long long *d_bad;
@@ -816,10 +869,11 @@ DispatchTables g_tables;
 int rocshmem_amd_dispatch_put_signal(void *recv, const void *send, uint64_t *sig,
                                      const uint32_t *count, const uint32_t *send_row,
                                      const uint32_t *recv_row, size_t row_bytes,
-                                     int rows_per_call, int wg_size,
+                                     int rows_per_call, int wg_size, uint64_t *expect,
                                      rocshmem_amd_stream_t stream) {
   auto &r = runtime::rt();
   if (!r.live || rows_per_call < 1 || !valid_launch(1, wg_size) || !row_bytes) return -1;
+  if (expect && !local_ok(expect, 8 * static_cast<size_t>(r.npes) * r.npes)) return -1;
   if (!count || !send_row || !recv_row) return -1;
   const size_t pp = static_cast<size_t>(r.npes) * r.npes;
   DispatchTables &t = g_tables;
@@ -870,6 +924,7 @@ int rocshmem_amd_dispatch_put_signal(void *recv, const void *send, uint64_t *sig
   a.n_calls = t.n_calls;
   a.ctx_row = r.driver_ctx_row();
   a.world_row = r.d_teams;
+  a.expect = expect;
   const uint32_t max_senders = 256 * 64;
   const uint32_t senders = a.n_calls < max_senders ? (a.n_calls ? a.n_calls : 1) : max_senders;
   hipLaunchKernelGGL(dispatch_kernel, dim3(senders + r.npes), dim3(wg_size), 0, as_stream(stream), a);

@@ -103,6 +103,28 @@ bool tracing() {
   return on;
 }
 
+// ---- hardware queues under PE threads ------------------------------------------
+// HIP multiplexes streams onto GPU_MAX_HW_QUEUES hardware queues (4 unless the
+// variable says otherwise).  Kernels of different PE threads wait for each
+// other inside the GPU; two such kernels in one hardware queue run one after
+// the other, so the first can wait for ever for the second.  Every stream a PE
+// thread launches on therefore needs a queue of its own, and one more is kept
+// for the library's own streams and the null stream.
+size_t hw_queue_limit() { return env_size("GPU_MAX_HW_QUEUES", 4); }
+bool hw_queues_suffice(size_t pe_streams, size_t hw_queues) {
+  return pe_streams + 1 <= hw_queues;
+}
+[[noreturn]] void refuse_for_queues(size_t pe_streams) {
+  fprintf(stderr,
+          "rocshmem: %zu streams of PE threads (plus one for the library) need %zu hardware "
+          "queues but GPU_MAX_HW_QUEUES=%zu: kernels of different PEs that wait for each other "
+          "would share a queue and never finish.  Set GPU_MAX_HW_QUEUES to at least the number "
+          "of streams in use (PEs x streams per PE + 1).  Nothing was launched.\n",
+          pe_streams, pe_streams + 1, hw_queue_limit());
+  fflush(nullptr);
+  _Exit(EXIT_FAILURE);
+}
+
 bool pe_threads_enter(int start, int stride, int size, uint64_t *result) {
   if (tl_pe < 0 || g_threads.npes == 0 || size <= 1) return true;
   MeetingPoint &p = g_threads.at(start, stride, size);
@@ -185,25 +207,26 @@ int Runtime::init(int want_npes, size_t want_heap) {
   max_teams = static_cast<int>(env_size("ROCSHMEM_MAX_NUM_TEAMS", 40));
   if (max_teams < 1) max_teams = 1;
   // Slice placement.  Slices start on 2 MiB boundaries and sit `pe_stride`
-  // apart inside ONE device allocation, which the driver backs with contiguous
-  // physical memory.  On MI355X a kernel that writes to all P slices at once
-  // (all-reduce, alltoall) sustains about 10 % more HBM bandwidth when the
-  // slices are 16-17 GiB apart than when they are 12 GiB or less apart
-  // (measured: 6.45 vs 5.7-5.9 TB/s for the P = 8 fp32 all-reduce; eight
-  // concurrent write streams alone: 7.2 vs 6.0 TB/s).
-  // ROCSHMEM_EMU_PE_STRIDE overrides the default chosen below.
+  // apart inside ONE device allocation.  By default the allocation holds the
+  // slices and nothing else: stride = heap size rounded up to 2 MiB.
+  //
+  // ROCSHMEM_EMU_SPREAD=1 trades device memory for bandwidth: the slices are
+  // spread over about half of the device memory on a 4 GiB grid (16 GiB apart
+  // for 8 PEs) and, when the GPU is otherwise empty, the block is placed by
+  // allocating half of the memory plus 1 GiB.  On MI355X a kernel that writes
+  // to all P slices at once (all-reduce, alltoall) then sustains about 10 %
+  // more HBM bandwidth (measured: 6.45 instead of 5.7-5.9 TB/s for the P = 8
+  // fp32 all-reduce) and is steadier from run to run.  That is a property of
+  // hosting P PEs inside one memory; it is off unless asked for.
+  // ROCSHMEM_EMU_PE_STRIDE=<bytes> sets the stride directly;
+  // ROCSHMEM_EMU_HEAP_ANCHOR=0 keeps the spread but not the placement.
   const size_t two_mib = size_t{2} << 20;
   const size_t min_stride = round_up(heap_size, two_mib);
+  const bool spread = env_size("ROCSHMEM_EMU_SPREAD", 0) != 0;
   size_t want = env_size("ROCSHMEM_EMU_PE_STRIDE", 0);
-  if (!want) {
+  if (!want && spread) {
     size_t free_b = 0, total_b = 0;
     RT_CHECK_HIP(hipMemGetInfo(&free_b, &total_b));
-    // What counts is that the slices are spread over about half of the device
-    // memory, whatever their number: P = 8 at 16 GiB, 12 at 12, 16 at 8 GiB
-    // all reach 6.45-6.5 TB/s in the all-reduce (8 at 8 GiB: 6.0, 16 at
-    // 4 GiB: 5.7), 3, 4 and 5 slices gain 2-5 % at 40, 32 and 28 GiB over
-    // 16 GiB.  Two slices do not care and keep 16 GiB.  Strides stay on a
-    // 4 GiB grid: some odd offsets (plus 1 MiB, plus 128 MiB) cost 5-9 %.
     const size_t budget = std::min(total_b / 2, free_b / 4 * 3);
     const size_t grid = size_t{4} << 30;
     want = npes <= 2 ? size_t{16} << 30 : budget / npes;
@@ -214,34 +237,38 @@ int Runtime::init(int want_npes, size_t want_heap) {
   acting_pe = 0;
   driver_ctx_options = 0;
 
-  // Where the block lands physically matters as much as the stride.  A block
-  // of 128 GiB fits twice into the 288 GB of an MI355X, the driver hands out
-  // the two places in turn (a freed block is not reused at once), and kernels
-  // with 16 concurrent streams run 2.5 % slower in one of them (the P = 8
-  // all-reduce: 6.28 instead of 6.45-6.48 TB/s, alternating from one
-  // rocshmem_init to the next, in one process or across processes).  A block of
-  // more than half of the memory fits in one place only, and that place is the
-  // good one: a heap of a quarter of the memory or more is therefore allocated
-  // as half of the memory plus 1 GiB when that much is free (the slices use the
-  // front of it).  ROCSHMEM_EMU_HEAP_ANCHOR=0 switches this off.
   size_t alloc_bytes = pe_stride * npes;
-  if (env_size("ROCSHMEM_EMU_HEAP_ANCHOR", 1) != 0) {
+  bool anchored = false;
+  if (spread && env_size("ROCSHMEM_EMU_HEAP_ANCHOR", 1) != 0) {
     size_t free_b = 0, total_b = 0;
     RT_CHECK_HIP(hipMemGetInfo(&free_b, &total_b));
     const size_t anchor = total_b / 2 + (size_t{1} << 30);
-    if (alloc_bytes >= total_b / 4 && alloc_bytes < anchor && free_b > anchor + (size_t{16} << 30))
+    if (alloc_bytes >= total_b / 4 && alloc_bytes < anchor && free_b > anchor + (size_t{16} << 30)) {
       alloc_bytes = anchor;
+      anchored = true;
+    }
   }
   hipError_t got = hipMalloc(reinterpret_cast<void **>(&heap_base), alloc_bytes);
-  if (got != hipSuccess && alloc_bytes != pe_stride * npes) {
+  if (got != hipSuccess && anchored) {
     (void)hipGetLastError();  // no room for the larger block: just the slices
-    got = hipMalloc(reinterpret_cast<void **>(&heap_base), pe_stride * npes);
+    anchored = false;
+    alloc_bytes = pe_stride * npes;
+    got = hipMalloc(reinterpret_cast<void **>(&heap_base), alloc_bytes);
   }
-  if (got != hipSuccess) {
-    (void)hipGetLastError();  // not enough room for the spread layout: pack the slices
+  if (got != hipSuccess && pe_stride != min_stride) {
+    (void)hipGetLastError();
+    fprintf(stderr,
+            "rocshmem: no room for %d slices %zu bytes apart; packing them (stride = heap size)\n",
+            npes, pe_stride);
     pe_stride = min_stride;
-    RT_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&heap_base), pe_stride * npes));
+    alloc_bytes = pe_stride * npes;
+    got = hipMalloc(reinterpret_cast<void **>(&heap_base), alloc_bytes);
   }
+  RT_CHECK_HIP(got);
+  heap_alloc_bytes = alloc_bytes;
+  if (env_size("ROCSHMEM_EMU_VERBOSE", 0) != 0)
+    fprintf(stderr, "rocshmem: %d PEs, heap %zu B per PE, slices %zu B apart, %zu B allocated%s\n",
+            npes, heap_size, pe_stride, alloc_bytes, anchored ? " (placed)" : "");
   allocator.reset(reinterpret_cast<uint64_t>(heap_base), heap_size);
 
   ws_stride = ws_bytes_per_pe();
@@ -311,6 +338,12 @@ int Runtime::init(int want_npes, size_t want_heap) {
     RT_CHECK_HIP(hipMemcpy(d_queue_table, none.data(), sizeof(detail::QueueBinding) * none.size(),
                            hipMemcpyHostToDevice));
   }
+  // Pinned words the stream bindings report through, allocated here because a
+  // pinned allocation or release later on may wait for the whole device, and by
+  // then another PE's kernel may be running and waiting for this PE.
+  RT_CHECK_HIP(hipHostMalloc(reinterpret_cast<void **>(&h_bind_problem),
+                             sizeof(int) * detail::kQueueTableSize, hipHostMallocDefault));
+  memset(h_bind_problem, 0, sizeof(int) * detail::kQueueTableSize);
   state.queue_table = d_queue_table;
   state.heap_base = heap_base;
   state.pe_stride = pe_stride;
@@ -326,7 +359,7 @@ int Runtime::init(int want_npes, size_t want_heap) {
   state.world_team = d_teams;
   state.ctx_pool = d_pools;
   state.ws_base = d_ws;
-  state.nt_bytes = env_size("ROCSHMEM_NT_THRESHOLD", size_t{64} << 10);
+  state.nt_bytes = env_size("ROCSHMEM_NT_THRESHOLD", detail::kNonTemporalBytes);
   live = true;
   push_state();
   ROCSHMEM_TEAM_WORLD = team_handle(0, acting_pe);
@@ -338,6 +371,8 @@ void Runtime::finalize() {
   RT_CHECK_HIP(hipDeviceSynchronize());
   RT_CHECK_HIP(hipFree(d_queue_table));
   d_queue_table = nullptr;
+  RT_CHECK_HIP(hipHostFree(h_bind_problem));
+  h_bind_problem = nullptr;
   RT_CHECK_HIP(hipFree(d_pools));
   RT_CHECK_HIP(hipFree(d_ctx_slots));
   RT_CHECK_HIP(hipFree(d_default_ctx));
@@ -366,6 +401,11 @@ rocshmem_team_t Runtime::team_handle(int pool_index, int pe) const {
 }
 
 const detail::Team *Runtime::host_team(rocshmem_team_t team) const {
+  std::lock_guard<std::mutex> guard(team_lock);
+  return host_team_unlocked(team);
+}
+
+const detail::Team *Runtime::host_team_unlocked(rocshmem_team_t team) const {
   if (team == ROCSHMEM_TEAM_INVALID || !live) return nullptr;
   const detail::Team *p = reinterpret_cast<const detail::Team *>(team);
   if (p < d_teams || p >= d_teams + static_cast<size_t>(max_teams) * npes) return nullptr;
@@ -411,12 +451,18 @@ void *Runtime::pe_ptr(const void *ptr, int pe) const {
 
 // src/rocshmem.cpp:221-303.  One call creates the team object of every member.
 int Runtime::team_split_strided(rocshmem_team_t parent, int start, int stride, int size,
-                                rocshmem_team_t *new_team) {
+                                rocshmem_team_t *new_team, int *slot_out) {
   require_live("rocshmem_team_split_strided");
   *new_team = ROCSHMEM_TEAM_INVALID;
+  if (slot_out) *slot_out = -1;
+  // The lock covers validation and the claim of a slot; the device writes
+  // below touch only the claimed slot and run unlocked, so that a thread which
+  // has to launch a kernel for this one to get past a device-wide wait is not
+  // held up in a team lookup.
+  std::unique_lock<std::mutex> guard(team_lock);
   if (num_user_teams >= max_teams - 1) return -1;
   if (parent == ROCSHMEM_TEAM_INVALID) return 0;
-  const detail::Team *pt = host_team(parent);
+  const detail::Team *pt = host_team_unlocked(parent);
   if (!pt) return -1;
   if (start < 0 || start >= pt->num_pes || size < 1 || size > pt->num_pes || stride < 1)
     return -1;
@@ -433,6 +479,7 @@ int Runtime::team_split_strided(rocshmem_team_t parent, int start, int stride, i
   if (slot < 0) return -1;
   team_slot_used[slot] = true;
   ++num_user_teams;
+  guard.unlock();
 
   // Fresh sync pads for the new team on every PE.
   const size_t pad_bytes = sizeof(detail::SyncPad) * detail::SYNC_KINDS;
@@ -449,20 +496,22 @@ int Runtime::team_split_strided(rocshmem_team_t parent, int start, int stride, i
   RT_CHECK_HIP(hipDeviceSynchronize());
   if (h_teams[static_cast<size_t>(slot) * npes + me()].my_pe >= 0)
     *new_team = team_handle(slot, me());
-  last_created_slot = slot;
+  if (slot_out) *slot_out = slot;
   return 0;
 }
 
 void Runtime::team_destroy(rocshmem_team_t team) {
   if (team == ROCSHMEM_TEAM_INVALID || !live) return;
-  const detail::Team *t = host_team(team);
+  std::lock_guard<std::mutex> guard(team_lock);
+  const detail::Team *t = host_team_unlocked(team);
   if (!t || t->pool_index == 0) return;
   team_slot_used[t->pool_index] = false;
   --num_user_teams;
 }
 
 rocshmem_team_t Runtime::team_on(rocshmem_team_t team, int pe) const {
-  const detail::Team *t = host_team(team);
+  std::lock_guard<std::mutex> guard(team_lock);
+  const detail::Team *t = host_team_unlocked(team);
   if (!t || pe < 0 || pe >= npes) return ROCSHMEM_TEAM_INVALID;
   if (h_teams[static_cast<size_t>(t->pool_index) * npes + pe].my_pe < 0) return ROCSHMEM_TEAM_INVALID;
   return team_handle(t->pool_index, pe);
@@ -521,21 +570,21 @@ struct WorldMeeting {
 }  // namespace
 
 __host__ void rocshmem_init(MPI_Comm) {
+  // Kernels of different PE threads wait for each other, so no two PE threads
+  // may share a hardware queue: refused here, before anything is allocated or
+  // enqueued, when there cannot be enough queues.
+  // (A program that only uses the host API binds no stream and needs no queue
+  // per PE; one built with a per-thread default stream binds one per PE right
+  // below.  Streams bound later are counted as they are bound.)
+  {
+    const int n = runtime::pe_threads_count();
+    if (n > 1 && runtime::tl_pe >= 0 && runtime::g_per_thread_default_stream &&
+        !runtime::hw_queues_suffice(n, runtime::hw_queue_limit()))
+      runtime::refuse_for_queues(n);
+  }
   WorldMeeting w;
   if (w.mine) {
     rt().init(runtime::pe_threads_count(), 0);
-    // Kernels of different PE threads that wait for each other must not share
-    // a hardware queue; HIP hands its queues (4 unless GPU_MAX_HW_QUEUES says
-    // otherwise) to streams in turn.
-    const int n = runtime::pe_threads_count();
-    const size_t queues = runtime::env_size("GPU_MAX_HW_QUEUES", 4);
-    if (n > 1 && queues < static_cast<size_t>(n) + 1)
-      fprintf(stderr,
-              "rocshmem: %d PE threads but GPU_MAX_HW_QUEUES=%zu: kernels of different PEs that "
-              "wait for each other can end up in one hardware queue and never finish; set "
-              "GPU_MAX_HW_QUEUES to at least the number of streams in use (PEs x streams per PE "
-              "+ 1)\n",
-              n, queues);
     w.done();
   }
   // A program built with -fgpu-default-stream=per-thread launches its
@@ -629,9 +678,9 @@ __host__ int rocshmem_team_split_strided(rocshmem_team_t parent_team, int start,
   uint64_t packed = 0;  // (return code + 1) << 32 | (slot + 1)
   if (runtime::pe_threads_enter(w.pe_start, w.stride, w.size, &packed)) {
     rocshmem_team_t unused;
-    const int rc = rt().team_split_strided(parent_team, start, stride, size, &unused);
-    packed = (static_cast<uint64_t>(rc + 1) << 32) |
-             static_cast<uint64_t>(rc == 0 ? rt().last_created_slot + 1 : 0);
+    int created = -1;
+    const int rc = rt().team_split_strided(parent_team, start, stride, size, &unused, &created);
+    packed = (static_cast<uint64_t>(rc + 1) << 32) | static_cast<uint64_t>(created + 1);
     runtime::pe_threads_leave(w.pe_start, w.stride, w.size, packed);
   }
   const int rc = static_cast<int>(packed >> 32) - 1;
@@ -691,13 +740,22 @@ __host__ void rocshmem_global_exit(int status) {
 }
 
 namespace {
-__global__ void bind_queue_kernel(detail::QueueBinding *table, int pe) {
+// Records "this hardware queue belongs to PE `pe`".  A slot that already names
+// another PE for the same queue means two PE threads share the queue; a slot
+// that names another queue is a collision in the table.  Either is reported
+// through *problem (1 / 2) and leaves the table as it was.
+__global__ void bind_queue_kernel(detail::QueueBinding *table, int pe, int *problem) {
   const unsigned long long id = detail::dispatch_queue_id();
-  table[id % detail::kQueueTableSize] = detail::QueueBinding{id, pe, 0};
+  detail::QueueBinding &slot = table[id % detail::kQueueTableSize];
+  if (slot.queue_id == id && slot.pe != pe) {
+    *problem = 1;
+  } else if (slot.queue_id != ~0ull && slot.queue_id != id) {
+    *problem = 2;
+  } else {
+    slot = detail::QueueBinding{id, pe, 0};
+  }
 }
-}  // namespace
 
-namespace {
 // Streams the calling PE thread has bound since the runtime came up.
 std::vector<hipStream_t> &bound_streams() {
   static thread_local std::vector<hipStream_t> bound;
@@ -708,15 +766,45 @@ std::vector<hipStream_t> &bound_streams() {
   }
   return bound;
 }
+
+// Streams bound by all PE threads of the current runtime.
+std::mutex g_bind_lock;
+size_t g_bound_total = 0;
+const void *g_bound_total_for = nullptr;
 }  // namespace
 
 void rocshmem_emu_bind_stream(hipStream_t stream) {
   if (runtime::tl_pe < 0 || !rt().live) return;
   std::vector<hipStream_t> &bound = bound_streams();
   if (std::find(bound.begin(), bound.end(), stream) != bound.end()) return;
+  std::lock_guard<std::mutex> guard(g_bind_lock);
+  if (g_bound_total_for != rt().d_queue_table) {
+    g_bound_total_for = rt().d_queue_table;
+    g_bound_total = 0;
+  }
+  // One more stream than there are hardware queues left would alias an
+  // earlier one: refuse before its first kernel is enqueued.
+  if (!runtime::hw_queues_suffice(g_bound_total + 1, runtime::hw_queue_limit()) ||
+      g_bound_total >= static_cast<size_t>(detail::kQueueTableSize))
+    runtime::refuse_for_queues(g_bound_total + 1);
+  int *problem = rt().h_bind_problem + g_bound_total;  // pinned word the kernel reports through
+  *problem = 0;
   hipLaunchKernelGGL(bind_queue_kernel, dim3(1), dim3(1), 0, stream, rt().d_queue_table,
-                     runtime::tl_pe);
+                     runtime::tl_pe, problem);
   RT_CHECK_HIP(hipGetLastError());
+  RT_CHECK_HIP(hipStreamSynchronize(stream));
+  const int seen = *problem;
+  if (seen) {
+    fprintf(stderr,
+            seen == 1 ? "rocshmem: the stream PE %d launches on shares its hardware queue with a "
+                        "stream of another PE thread; raise GPU_MAX_HW_QUEUES (now %zu)\n"
+                      : "rocshmem: PE %d: no room in the queue table for another hardware queue "
+                        "(GPU_MAX_HW_QUEUES=%zu)\n",
+            runtime::tl_pe, runtime::hw_queue_limit());
+    fflush(nullptr);
+    _Exit(EXIT_FAILURE);
+  }
+  ++g_bound_total;
   bound.push_back(stream);
 }
 

@@ -5,6 +5,7 @@
 
 #include <cstddef>
 #include <cstdint>
+#include <mutex>
 #include <vector>
 
 #include "pow2_allocator.hpp"
@@ -26,10 +27,10 @@ struct Runtime {
   int max_ctxs = 0;
   int max_teams = 0;
   int num_user_teams = 0;
-  int last_created_slot = -1;
   size_t heap_size = 0;
   size_t pe_stride = 0;
   size_t ws_stride = 0;
+  size_t heap_alloc_bytes = 0;  // size of the device allocation that holds the slices
   char *heap_base = nullptr;
   char *d_ws = nullptr;
   detail::Team *d_teams = nullptr;         // [max_teams][npes]
@@ -37,6 +38,7 @@ struct Runtime {
   detail::Context *d_ctx_slots = nullptr;  // [npes][max_ctxs]
   detail::CtxPool *d_pools = nullptr;      // [npes]
   detail::QueueBinding *d_queue_table = nullptr;  // [kQueueTableSize]
+  int *h_bind_problem = nullptr;  // pinned, [kQueueTableSize]: what each stream binding reported
   std::vector<detail::Team> h_teams;       // host mirror of d_teams
   std::vector<bool> team_slot_used;
   Pow2Allocator allocator;
@@ -53,8 +55,12 @@ struct Runtime {
   int pe_of(const void *ptr) const;
   void *pe_ptr(const void *ptr, int pe) const;
 
+  // Team creation, destruction and lookup may come from several host threads
+  // at once (PE threads whose sub-teams are disjoint meet at different
+  // rendezvous points): team_lock serialises them.  slot_out, when given,
+  // receives the team's slot (-1 on failure).
   int team_split_strided(rocshmem_team_t parent, int start, int stride, int size,
-                         rocshmem_team_t *new_team);
+                         rocshmem_team_t *new_team, int *slot_out = nullptr);
   void team_destroy(rocshmem_team_t team);
   rocshmem_team_t team_handle(int pool_index, int pe) const;
   rocshmem_team_t team_on(rocshmem_team_t team, int pe) const;
@@ -65,6 +71,7 @@ struct Runtime {
     return tl_pe < 0 ? team : team_on(team, tl_pe);
   }
   const detail::Team *host_team(rocshmem_team_t team) const;
+  mutable std::mutex team_lock;
 
   void set_pe(int pe);
   void set_pe_rule(int rule);
@@ -91,6 +98,7 @@ struct Runtime {
   }
 
  private:
+  const detail::Team *host_team_unlocked(rocshmem_team_t team) const;
   size_t ws_bytes_per_pe() const;
   detail::SyncPad *team_pads(int pool_index, int pe) const;
   void write_team(int pool_index, int pe, const detail::TeamInfo &world,
@@ -109,6 +117,12 @@ Runtime &rt();
 bool pe_threads_enter(int start, int stride, int size, uint64_t *result);
 void pe_threads_leave(int start, int stride, int size, uint64_t result);
 int pe_threads_count();  // P while PE threads run, else 0
+// Hardware queues HIP will use (GPU_MAX_HW_QUEUES, default 4); whether
+// `pe_streams` streams of PE threads plus one for the library fit; and the
+// fatal refusal (message, exit status 1, nothing launched) when they do not.
+size_t hw_queue_limit();
+bool hw_queues_suffice(size_t pe_streams, size_t hw_queues);
+[[noreturn]] void refuse_for_queues(size_t pe_streams);
 void pe_threads_start(int npes);
 
 }  // namespace runtime

@@ -39,6 +39,9 @@ SIGNATURES = {
     "rocshmem_amd_heap_used": (_sz, []),
     "rocshmem_amd_heap_avail": (_sz, []),
     "rocshmem_amd_pe_stride": (_sz, []),
+    "rocshmem_amd_heap_alloc_bytes": (_sz, []),
+    "rocshmem_amd_coresident": (_i, [C.c_long, _i, _i]),
+    "rocshmem_amd_hw_queues_suffice": (_i, [_sz, _sz]),
     "rocshmem_amd_heap_model_create": (_vp, [_u64, _u64]),
     "rocshmem_amd_heap_model_destroy": (None, [_vp]),
     "rocshmem_amd_heap_model_alloc": (_u64, [_vp, _u64]),
@@ -56,12 +59,14 @@ SIGNATURES = {
     "rocshmem_amd_team_active_set": (_i, [_vp, C.POINTER(_i), C.POINTER(_i), C.POINTER(_i)]),
     "rocshmem_amd_pe_threads_enter": (_i, [_i, _i, _i]),
     "rocshmem_amd_pe_threads_leave": (None, [_i, _i, _i]),
+    "rocshmem_amd_dev_mem_info": (_i, [C.POINTER(_sz), C.POINTER(_sz)]),
     "rocshmem_amd_dev_alloc": (_vp, [_sz]),
     "rocshmem_amd_dev_free": (_i, [_vp]),
     "rocshmem_amd_copy_in": (_i, [_vp, _vp, _sz]),
     "rocshmem_amd_copy_out": (_i, [_vp, _vp, _sz]),
     "rocshmem_amd_fill": (_i, [_vp, _i, _sz]),
     "rocshmem_amd_hbm_probe": (_i, [_i, _vp, _sz, _vp]),
+    "rocshmem_amd_release_probe": (_i, [_i, _vp, _vp, _sz, _sz, _i, _i, _vp]),
     "rocshmem_amd_fill_every_pe": (_i, [_vp, _i, _sz, _vp]),
     "rocshmem_amd_copy_dev": (_i, [_vp, _vp, _sz]),
     "rocshmem_amd_stream_sync": (_i, [_vp]),
@@ -85,7 +90,7 @@ SIGNATURES = {
     "rocshmem_amd_getmem": (_i, [_vp, _vp, _sz, _i, _i, _vp]),
     "rocshmem_amd_wf_coalesce": (_i, [_vp, _vp, _vp, _vp, _u64, _vp, _vp]),
     "rocshmem_amd_wg_reduce": (_i, [_i, _i, _vp, _vp, _vp, _i, _i, _vp]),
-    "rocshmem_amd_wg_reduce_teams": (_i, [_i, _i, C.POINTER(_vp), _i, _vp, _vp, _i, _i, _vp]),
+    "rocshmem_amd_wg_reduce_teams": (_i, [_i, _i, C.POINTER(_vp), _i, _vp, _vp, _i, _i, _i, _vp]),
     "rocshmem_amd_wg_alltoall": (_i, [_i, _vp, _vp, _vp, _i, _i, _vp]),
     "rocshmem_amd_wg_broadcast": (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "rocshmem_amd_wg_fcollect": (_i, [_i, _vp, _vp, _vp, _i, _i, _vp]),
@@ -100,7 +105,7 @@ SIGNATURES = {
     "rocshmem_amd_signal_fetch": (_i, [_i, _vp, _i, C.POINTER(_u64)]),
     "rocshmem_amd_pingpong": (_i, [_vp, _vp, _sz, _i, _i, _i, _i, _i, C.POINTER(_u64),
                                    C.POINTER(C.c_double), _vp]),
-    "rocshmem_amd_dispatch_put_signal": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _vp]),
+    "rocshmem_amd_dispatch_put_signal": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _i, _i, _vp, _vp]),
     "rocshmem_amd_wait_test": (_i, [_i, _i, _vp, _sz, _vp, _i, _vp, C.POINTER(_sz), _vp]),
     "rocshmem_amd_wait_test_woken": (_i, [_i, _i, _vp, _sz, _vp, _i, _vp, _sz, _vp, _u64,
                                           C.POINTER(_sz), _vp]),

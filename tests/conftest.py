@@ -9,10 +9,11 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 
-# Slices are packed (stride = heap size) in the tests so that bring-up stays
-# quick; the spread 16 GiB layout only changes bandwidth, not results, and is
-# exercised by the full-size test and by bench.py.
-os.environ.setdefault("ROCSHMEM_EMU_PE_STRIDE", "1")
+# The tests run in the library's default layout (slices packed, stride = heap
+# size).  The spread layout (ROCSHMEM_EMU_SPREAD=1) only changes bandwidth, not
+# results; the full-size tests, test_spread_layout_is_opt_in and bench.py run in it.
+os.environ.pop("ROCSHMEM_EMU_SPREAD", None)
+os.environ.pop("ROCSHMEM_EMU_PE_STRIDE", None)
 
 
 def pytest_configure(config):

@@ -352,11 +352,23 @@ def test_dispatch_put_signal(rt, L, orc, rows_per_call):
     assert l.fill_every_pe(sig, 0, 8 * P, None) == 0
     counts, send_row, recv_row = (np.ascontiguousarray(a, np.uint32) for a in (counts, send_row, recv_row))
     assert l.dispatch_put_signal(recv, send, sig, counts.ctypes.data, send_row.ctypes.data,
-                                 recv_row.ctypes.data, row, rows_per_call, 256, None) == 0
+                                 recv_row.ctypes.data, row, rows_per_call, 256, None, None) == 0
     l.stream_sync(None)
+    # ... and twice more with running totals instead of cleared signal words
+    expect = l.dev_alloc(8 * P * P)
+    l.fill(expect, 0, 8 * P * P)
+    assert l.fill_every_pe(sig, 0, 8 * P, None) == 0
+    rounds = 3 if rows_per_call != 1 else 1
+    for _ in range(rounds):
+        assert l.dispatch_put_signal(recv, send, sig, counts.ctypes.data, send_row.ctypes.data,
+                                     recv_row.ctypes.data, row, rows_per_call, 256, expect, None) == 0
+    l.stream_sync(None)
+    totals = rt.get_bytes(expect, 8 * P * P, np.uint64).reshape(P, P)  # [d][s]
+    assert np.array_equal(totals, rounds * counts.T.astype(np.uint64))
+    l.dev_free(expect)
     for d in range(P):
         sigs = rt.get_bytes(l.pe_ptr(sig, d), 8 * P, np.uint64)
-        assert np.array_equal(sigs, counts[:, d].astype(np.uint64))
+        assert np.array_equal(sigs, rounds * counts[:, d].astype(np.uint64))
         got = rt.get_bytes(l.pe_ptr(recv, d), max_rows * row)
         for s in range(P):
             c = int(counts[s, d])

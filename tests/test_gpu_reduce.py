@@ -191,7 +191,7 @@ def test_many_teams_reduce_their_slices_at_once(rt, L, orc, n_teams):
             for k, p in enumerate(pes):
                 rt.put_bytes(l.pe_ptr(b.src, p), srcs[k])
             assert l.wg_reduce_teams(getattr(L, dtype_name), getattr(L, op_name), teams, n_teams,
-                                     l.pe_ptr(b.dst, pes[0]), l.pe_ptr(b.src, pes[0]), n, 256, None) == 0
+                                     l.pe_ptr(b.dst, pes[0]), l.pe_ptr(b.src, pes[0]), n, 256, 1, None) == 0
             want = orc.to_all(getattr(orc, dtype_name), getattr(orc, op_name), srcs)
             for p in range(8):
                 got = rt.get_bytes(l.pe_ptr(b.dst, p), (n + 8) * es, np_t)
@@ -205,7 +205,7 @@ def test_many_teams_reduce_their_slices_at_once(rt, L, orc, n_teams):
         if n_teams >= 2:
             twice = (ctypes.c_void_p * 2)(teams[0], teams[0])
             assert l.wg_reduce_teams(L.INT, L.SUM, twice, 2, l.pe_ptr(b.src, pes[0]), l.pe_ptr(b.src, pes[0]),
-                                     0, 64, None) == -1
+                                     0, 64, 1, None) == -1
         for t in range(n_teams):
             l.team_destroy(teams[t])
     l.set_pe(0)
@@ -280,14 +280,15 @@ def test_unsupported_combinations_are_rejected(rt, L):
 @pytest.mark.parametrize("dtype_name,op_name", [("FLOAT", "SUM"), ("BF16", "SUM"), ("FLOAT", "MAX"),
                                                 ("LONG", "XOR")])
 def test_full_size_64mi_properties(rt, L, orc, dtype_name, op_name, monkeypatch):
-    """P=8 x 64 Mi elements, slices in the default spread layout.  Inputs are made on the CPU for windows only; the
+    """P=8 x 64 Mi elements, slices in the spread layout (ROCSHMEM_EMU_SPREAD=1,
+    as bench.py runs).  Inputs are made on the CPU for windows only; the
     bulk is checked through size-independent properties: all P destinations are
     identical, the windows match the oracle, and for xor reducing the result
     with itself gives zero / reducing twice with P even returns to zero."""
-    monkeypatch.delenv("ROCSHMEM_EMU_PE_STRIDE", raising=False)
+    monkeypatch.setenv("ROCSHMEM_EMU_SPREAD", "1")
     rt.down()
     l = rt.up(8, 2 << 30)
-    assert l.pe_stride() >= 2 << 30
+    assert l.pe_stride() >= 16 << 30
     n = 1 << 26
     np_t = orc.NP_DTYPE[getattr(orc, dtype_name)]
     es = np.dtype(np_t).itemsize

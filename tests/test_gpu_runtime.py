@@ -9,6 +9,7 @@ pytestmark = pytest.mark.gpu
 
 
 def test_malloc_matches_the_oracle_allocator(rt, L, orc):
+    rt.down()  # a fresh heap: freed blocks are never merged, so history matters
     l = rt.up(4, 1 << 26)
     base = l.malloc(1)
     l.free(base)
@@ -134,11 +135,47 @@ def test_team_pool_exhaustion(rt, L):
         l.team_destroy(x)
 
 
-def test_default_slice_stride_spreads_the_pes(rt, L, monkeypatch):
-    """Without an override the slices are spread over half of the device
-    memory on a 4 GiB grid (288 GB: 16 GiB for 8 PEs, 32 for 4, 44 for 3, 8
-    for 16; two PEs keep 16 GiB), never closer than the heap size."""
+def test_default_layout_allocates_what_the_slices_need(rt, L, monkeypatch):
+    """By default the slices are packed: stride = heap size rounded up to
+    2 MiB, one allocation of P strides.  A default rocshmem_init with 8 PEs and
+    the default 1 GiB per PE leaves the rest of the device memory to the user:
+    free memory afterwards is within 1 GiB of what was free before minus the
+    8 GiB of slices."""
     monkeypatch.delenv("ROCSHMEM_EMU_PE_STRIDE", raising=False)
+    monkeypatch.delenv("ROCSHMEM_EMU_SPREAD", raising=False)
+    monkeypatch.delenv("ROCSHMEM_HEAP_SIZE", raising=False)
+    rt.down()
+    l = L.load()
+    free0, free1, total = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
+    assert l.dev_mem_info(ctypes.byref(free0), ctypes.byref(total)) == 0
+    assert l.init(8, 0) == 0
+    try:
+        assert l.heap_size() == 1 << 30 and l.pe_stride() == 1 << 30
+        assert l.heap_alloc_bytes() == 8 << 30
+        assert l.dev_mem_info(ctypes.byref(free1), ctypes.byref(total)) == 0
+        taken = free0.value - free1.value  # slices + work/sync area + contexts and teams
+        assert (8 << 30) - (64 << 20) <= taken <= (9 << 30), taken
+        # and the user can still allocate most of the device
+        big = l.dev_alloc(free1.value // 2)
+        assert big
+        l.dev_free(big)
+    finally:
+        l.finalize()
+    for npes, heap in ((3, (1 << 24) + 5), (5, 3 << 20)):
+        assert l.init(npes, heap) == 0
+        want = (heap + (2 << 20) - 1) // (2 << 20) * (2 << 20)
+        assert l.pe_stride() == want and l.heap_alloc_bytes() == want * npes
+        l.finalize()
+
+
+def test_spread_layout_is_opt_in(rt, L, monkeypatch):
+    """ROCSHMEM_EMU_SPREAD=1 spreads the slices over half of the device
+    memory on a 4 GiB grid (288 GB: 16 GiB for 8 PEs, 32 for 4, 44 for 3, 8
+    for 16; two PEs keep 16 GiB), never closer than the heap size;
+    ROCSHMEM_EMU_PE_STRIDE sets the stride directly.  Results do not depend on
+    the layout: an all-reduce in the spread layout matches the packed one."""
+    monkeypatch.delenv("ROCSHMEM_EMU_PE_STRIDE", raising=False)
+    monkeypatch.setenv("ROCSHMEM_EMU_SPREAD", "1")
     rt.down()
     l = L.load()
     for npes, gib in ((2, 16), (3, 44), (4, 32), (5, 28), (8, 16), (16, 8)):
@@ -151,6 +188,22 @@ def test_default_slice_stride_spreads_the_pes(rt, L, monkeypatch):
     assert l.init(4, 1 << 22) == 0
     assert l.pe_stride() == 6 << 20
     l.finalize()
+    monkeypatch.delenv("ROCSHMEM_EMU_PE_STRIDE")
+    results = []
+    for spread in ("1", "0"):
+        monkeypatch.setenv("ROCSHMEM_EMU_SPREAD", spread)
+        assert l.init(8, 1 << 24) == 0
+        n = 100003
+        src, dst = l.malloc(n * 4), l.malloc(n * 4)
+        for p in range(8):
+            host = np.random.default_rng(p).standard_normal(n).astype(np.float32)
+            l.copy_in(l.pe_ptr(src, p), host.ctypes.data, n * 4)
+        assert l.wg_reduce(L.FLOAT, L.SUM, l.team_world(), dst, src, n, 256, None) == 0
+        out = np.empty(n, np.float32)
+        l.copy_out(out.ctypes.data, l.pe_ptr(dst, 5), n * 4)
+        results.append(out)
+        l.finalize()
+    assert np.array_equal(results[0].view(np.uint32), results[1].view(np.uint32))
 
 
 def test_reinit_and_environment_defaults(rt, L, monkeypatch):
