@@ -296,6 +296,19 @@ int rocshmem_amd_wg_reduce(int dtype, int op, rocshmem_amd_team_t team, void *de
 int rocshmem_amd_wg_reduce_teams(int dtype, int op, const rocshmem_amd_team_t *teams, int n_teams,
                                  void *dest, const void *source, int nreduce, int wg_size,
                                  int iters, rocshmem_amd_stream_t stream);
+/* rocshmem_amd_wg_reduce_teams for callers that cannot allocate device memory
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc).  It has no counterpart in the reference.  Same arguments, same
+ * results; the per-team status words, which rocshmem_amd_wg_reduce_teams
+ * allocates and frees on every call, live in a fixed array inside the library's
+ * code object instead: 256 words (1 KiB) per GPU, held until the process ends.
+ * The call makes no hipMalloc / hipFree.  n_teams beyond 256 is refused with a
+ * message on stderr.  All calls on one GPU share the array: it is cleared on the
+ * stream before each launch, and two calls that overlap in time on one GPU
+ * race on it (run them one after the other). */
+int rocshmem_amd_wg_reduce_teams_static(int dtype, int op, const rocshmem_amd_team_t *teams,
+                                        int n_teams, void *dest, const void *source, int nreduce,
+                                        int wg_size, int iters, rocshmem_amd_stream_t stream);
 /* rocshmem_ctx_<T>_wg_alltoall / _wg_broadcast / _wg_fcollect
  * (rocshmem_COLL.hpp:44-258; context_ipc_tmpl_device.hpp:420-531).
  * elem_size in {1,2,4,8} selects the typed entry point (char/short/int/long). */

@@ -122,6 +122,18 @@ __global__ void wg_reduce_teams_kernel(WgTeamsArgs a) {
   }
 }
 
+// Sets n words to zero from the stream (a plain kernel: safe to record in a
+// HIP graph, which a memset node is not on every driver).
+__global__ void clear_words_kernel(int *words, int n) {
+  for (int i = threadIdx.x; i < n; i += blockDim.x) words[i] = 0;
+}
+
+// Status words of rocshmem_amd_wg_reduce_teams_static: one per team of a
+// launch.  Lives in the code object, so the entry point needs no allocation;
+// every call on a GPU shares it.
+constexpr int kStaticStatusWords = kMaxTeamsPerLaunch;
+static __device__ __align__(256) int scratch[kStaticStatusWords];
+
 enum WgMove { MOVE_ALLTOALL, MOVE_BROADCAST, MOVE_FCOLLECT };
 
 template <typename T, int kMove>
@@ -621,6 +633,56 @@ int rocshmem_amd_wg_reduce_teams(int dtype, int op, const rocshmem_amd_team_t *t
     for (int t = 0; t < n_teams; ++t) status = seen[t] > status ? seen[t] : status;
   }
   DRV_CHECK_HIP(hipFree(d_status));
+  return status;
+}
+
+// The address of `scratch` on the current device, looked up once per device.
+static int *static_status_words() {
+  constexpr int kMaxDevices = 64;
+  static std::mutex lock;
+  static int *words[kMaxDevices] = {};
+  int dev = 0;
+  DRV_CHECK_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= kMaxDevices) return nullptr;
+  std::lock_guard<std::mutex> guard(lock);
+  if (!words[dev]) {
+    void *p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+      fprintf(stderr, "rocshmem: hipGetSymbolAddress(scratch) failed on device %d: %s\n", dev,
+              hipGetErrorString(e));
+      return nullptr;
+    }
+    words[dev] = static_cast<int *>(p);
+  }
+  return words[dev];
+}
+
+int rocshmem_amd_wg_reduce_teams_static(int dtype, int op, const rocshmem_amd_team_t *teams,
+                                        int n_teams, void *dest, const void *source, int nreduce,
+                                        int wg_size, int iters, rocshmem_amd_stream_t stream) {
+  if (n_teams > kStaticStatusWords) {
+    fprintf(stderr,
+            "rocshmem: rocshmem_amd_wg_reduce_teams_static takes at most %d teams per call "
+            "(its status words are a fixed array), %d asked for\n",
+            kStaticStatusWords, n_teams);
+    return -1;
+  }
+  if (n_teams < 1) return -1;
+  int *words = static_status_words();
+  if (!words) return -1;
+  hipStream_t s = as_stream(stream);
+  // The array keeps what the last call left: clear the words this call uses.
+  hipLaunchKernelGGL(clear_words_kernel, dim3(1), dim3(256), 0, s, words, n_teams);
+  DRV_CHECK_HIP(hipGetLastError());
+  int status = enqueue_reduce_teams(dtype, op, teams, n_teams, dest, source, nreduce, wg_size,
+                                    iters, words, s);
+  if (status == 0) {
+    int seen[kStaticStatusWords];
+    DRV_CHECK_HIP(hipStreamSynchronize(s));
+    DRV_CHECK_HIP(hipMemcpy(seen, words, sizeof(int) * n_teams, hipMemcpyDeviceToHost));
+    for (int t = 0; t < n_teams; ++t) status = seen[t] > status ? seen[t] : status;
+  }
   return status;
 }
 

@@ -91,6 +91,8 @@ SIGNATURES = {
     "rocshmem_amd_wf_coalesce": (_i, [_vp, _vp, _vp, _vp, _u64, _vp, _vp]),
     "rocshmem_amd_wg_reduce": (_i, [_i, _i, _vp, _vp, _vp, _i, _i, _vp]),
     "rocshmem_amd_wg_reduce_teams": (_i, [_i, _i, C.POINTER(_vp), _i, _vp, _vp, _i, _i, _i, _vp]),
+    "rocshmem_amd_wg_reduce_teams_static": (_i, [_i, _i, C.POINTER(_vp), _i, _vp, _vp, _i, _i, _i,
+                                                 _vp]),
     "rocshmem_amd_wg_alltoall": (_i, [_i, _vp, _vp, _vp, _i, _i, _vp]),
     "rocshmem_amd_wg_broadcast": (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "rocshmem_amd_wg_fcollect": (_i, [_i, _vp, _vp, _vp, _i, _i, _vp]),

@@ -38,7 +38,7 @@ def test_reduce_grid_that_cannot_be_resident_is_refused_and_launches_nothing(rt,
     for p in range(P):
         rt.put_bytes(l.pe_ptr(src, p), ones)
         l.fill(l.pe_ptr(dst, p), 0x5A, n * 4)
-    for entry in (l.wg_reduce_teams,):
+    for entry in (l.wg_reduce_teams, l.wg_reduce_teams_static):
         assert entry(L.INT, L.SUM, teams, n_teams, dst, src, n, 1024, 1, None) == -1
     l.stream_sync(None)
     for p in range(P):
