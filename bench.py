@@ -49,6 +49,10 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--quick", action="store_true", help="headline only, no CPU baseline")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--profile-kernels", action="store_true",
+                    help="a short run for rocprofv3: a few launches each of the headline put, the "
+                         "fp32 sum all-reduce, the alltoall and the dispatch, and three 256 MiB "
+                         "hipMemcpy calls to calibrate the byte counters; prints the launch counts")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run three 256 MiB device-to-device hipMemcpy calls (the HIP "
                          "runtime's copy kernel) for calibrating FETCH_SIZE / WRITE_SIZE")
@@ -486,8 +490,45 @@ def cpu_baseline():
             "pingpong_8B_us": round(pp, 3)}
 
 
+def profile_kernels():
+    """What rocprofv3 --pmc / --kernel-trace is pointed at: each dominant kernel
+    a few times on full-size inputs, and the HIP runtime's own copy kernel on
+    256 MiB as the yardstick of the byte counters."""
+    os.environ.setdefault("ROCSHMEM_EMU_SPREAD", "1")
+    from rocshmem_amd import lib as L
+    b = Bench(L)
+    b.quick = True
+    l = b.l
+    assert l.init(P, 8 << 30) == 0
+    disp = dispatch_config(b, 20)                      # 2 warm-up + 5 timed launches per context kind
+    n = 256 * MiB
+    cs, cd = l.malloc(n), l.malloc(n)
+    for _ in range(3):
+        l.copy_dev(cd, cs, n)
+    l.free(cs)
+    l.free(cd)
+    head = headline(b, 8, 2)                           # 10 launches of each of the put routes
+    m = 1 << 26
+    src, dst = l.malloc(m * 4), l.malloc(m * 4)
+    for p in range(P):
+        b.fill_random(l.pe_ptr(src, p), m * 4, p, 10 + p, "f32")
+    ms_red = b.time_ms(lambda: l.to_all(L.FLOAT, L.SUM, dst, src, m, 0, 0, P, None), 6, 2)
+    l.free(src)
+    l.free(dst)
+    a2a = alltoall_config(b, 6)
+    l.finalize()
+    print(json.dumps({"putmem_wg_nostore_gbs": round(head["gbs"], 1),
+                      "putmem_wg_default_gbs": round(head["default_ctx_gbs"], 1),
+                      "host_putmem_gbs": round(head["host_putmem_gbs"], 1),
+                      "to_all_fp32_sum_gbs": round(2 * P * m * 4 / ms_red / 1e6, 1),
+                      "alltoall_gbs": a2a["gbs"], "dispatch": disp}))
+
+
 def main():
     a = parse()
+    if a.profile_kernels:
+        profile_kernels()
+        return
     if a.gpus != 1:
         print("bench.py measures one GPU: every PE is a slice of one symmetric heap on a single "
               "MI355X; --gpus %d is not supported (use --gpus 1)." % a.gpus, file=sys.stderr)

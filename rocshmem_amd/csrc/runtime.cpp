@@ -186,6 +186,73 @@ void Runtime::write_team(int pool_index, int pe, const detail::TeamInfo &world,
                          sizeof(t), hipMemcpyHostToDevice));
 }
 
+// ---- the device allocation behind the symmetric heap ---------------------------
+// The heap is UNCACHED device memory (hipDeviceMallocUncached), as the
+// reference's is (src/memory/hip_allocator.hpp:58-65, heap_type.hpp:50).  The
+// L2 of an XCD then never holds a line of it, clean or dirty, and that is what
+// makes ordering cheap on this part: an agent-scope release is an L2 write-back
+// (buffer_wbl2), which on MI355X occupies the XCD's L2 for about 0.3 us
+// whenever the L2 holds lines that loads brought in — dirty or not — and for a
+// few ns when it holds none.  Measured, 256 MiB copied in 16 KiB tiles by 1024
+// work-groups of 256 with one release per tile: 760 us with a cached heap
+// (hipMalloc, or fine-grained), 156 us with an uncached one, 87 us without
+// releases; the copy itself runs at the same rate on either.  Stores to the
+// heap never sit dirty either, plain ones included, so quiet / fence / barriers
+// on a default context publish them at once.
+//
+// Uncached memory is never given back while the process lives: on this class
+// of machines memory allocated after such a release has shown wrong values.
+// rocshmem_finalize marks the block idle, and a later rocshmem_init reuses
+// the smallest idle block that is large enough before it allocates another.
+// ROCSHMEM_EMU_HEAP_CACHED=1 selects plain hipMalloc / hipFree instead
+// (measurements).
+namespace {
+struct HeapBlock {
+  char *base;
+  size_t bytes;
+  bool in_use;
+};
+std::mutex g_heap_lock;
+std::vector<HeapBlock> g_heap_blocks;  // uncached blocks of this process, never freed
+
+bool heap_cached_mode() { return env_size("ROCSHMEM_EMU_HEAP_CACHED", 0) != 0; }
+
+// An idle uncached block of at least `bytes`, or nullptr.
+char *reuse_heap_block(size_t bytes, size_t *block_bytes) {
+  std::lock_guard<std::mutex> guard(g_heap_lock);
+  HeapBlock *best = nullptr;
+  for (HeapBlock &b : g_heap_blocks)
+    if (!b.in_use && b.bytes >= bytes && (!best || b.bytes < best->bytes)) best = &b;
+  if (!best) return nullptr;
+  best->in_use = true;
+  *block_bytes = best->bytes;
+  return best->base;
+}
+
+hipError_t new_heap_block(char **base, size_t bytes) {
+  if (heap_cached_mode()) return hipMalloc(reinterpret_cast<void **>(base), bytes);
+  const hipError_t e =
+      hipExtMallocWithFlags(reinterpret_cast<void **>(base), bytes, hipDeviceMallocUncached);
+  if (e == hipSuccess) {
+    std::lock_guard<std::mutex> guard(g_heap_lock);
+    g_heap_blocks.push_back(HeapBlock{*base, bytes, true});
+  }
+  return e;
+}
+
+void release_heap_block(char *base) {
+  {
+    std::lock_guard<std::mutex> guard(g_heap_lock);
+    for (HeapBlock &b : g_heap_blocks)
+      if (b.base == base) {
+        b.in_use = false;
+        return;
+      }
+  }
+  RT_CHECK_HIP(hipFree(base));  // a cached-mode block
+}
+}  // namespace
+
 int Runtime::init(int want_npes, size_t want_heap) {
   if (live) return 0;
   int ndev = 0;
@@ -224,10 +291,10 @@ int Runtime::init(int want_npes, size_t want_heap) {
   const size_t min_stride = round_up(heap_size, two_mib);
   const bool spread = env_size("ROCSHMEM_EMU_SPREAD", 0) != 0;
   size_t want = env_size("ROCSHMEM_EMU_PE_STRIDE", 0);
+  size_t free_b = 0, total_b = 0;
+  RT_CHECK_HIP(hipMemGetInfo(&free_b, &total_b));
   if (!want && spread) {
-    size_t free_b = 0, total_b = 0;
-    RT_CHECK_HIP(hipMemGetInfo(&free_b, &total_b));
-    const size_t budget = std::min(total_b / 2, free_b / 4 * 3);
+    const size_t budget = total_b / 2;
     const size_t grid = size_t{4} << 30;
     want = npes <= 2 ? size_t{16} << 30 : budget / npes;
     if (want >= grid) want = want / grid * grid;
@@ -237,38 +304,55 @@ int Runtime::init(int want_npes, size_t want_heap) {
   acting_pe = 0;
   driver_ctx_options = 0;
 
-  size_t alloc_bytes = pe_stride * npes;
+  // Three tries: the spread block placed in the upper half of the memory, the
+  // spread block, the packed slices.  Each first looks for an idle block from
+  // an earlier rocshmem_init of this process.
+  const size_t anchor = total_b / 2 + (size_t{1} << 30);
+  const bool want_anchor = spread && env_size("ROCSHMEM_EMU_HEAP_ANCHOR", 1) != 0 &&
+                           pe_stride * npes >= total_b / 4 && pe_stride * npes < anchor;
   bool anchored = false;
-  if (spread && env_size("ROCSHMEM_EMU_HEAP_ANCHOR", 1) != 0) {
-    size_t free_b = 0, total_b = 0;
-    RT_CHECK_HIP(hipMemGetInfo(&free_b, &total_b));
-    const size_t anchor = total_b / 2 + (size_t{1} << 30);
-    if (alloc_bytes >= total_b / 4 && alloc_bytes < anchor && free_b > anchor + (size_t{16} << 30)) {
-      alloc_bytes = anchor;
+  heap_base = nullptr;
+  size_t alloc_bytes = 0;
+  auto try_block = [&](size_t bytes) {
+    size_t had = 0;
+    if (!heap_cached_mode() && (heap_base = reuse_heap_block(bytes, &had))) {
+      alloc_bytes = had;
+      return true;
+    }
+    if (new_heap_block(&heap_base, bytes) == hipSuccess) {
+      alloc_bytes = bytes;
+      return true;
+    }
+    (void)hipGetLastError();
+    heap_base = nullptr;
+    return false;
+  };
+  if (want_anchor) {
+    size_t had = 0;
+    if (!heap_cached_mode() && (heap_base = reuse_heap_block(anchor, &had))) {
+      alloc_bytes = had;
       anchored = true;
+    } else if (free_b > anchor + (size_t{16} << 30)) {
+      anchored = try_block(anchor);
     }
   }
-  hipError_t got = hipMalloc(reinterpret_cast<void **>(&heap_base), alloc_bytes);
-  if (got != hipSuccess && anchored) {
-    (void)hipGetLastError();  // no room for the larger block: just the slices
-    anchored = false;
-    alloc_bytes = pe_stride * npes;
-    got = hipMalloc(reinterpret_cast<void **>(&heap_base), alloc_bytes);
-  }
-  if (got != hipSuccess && pe_stride != min_stride) {
-    (void)hipGetLastError();
+  if (!heap_base && !try_block(pe_stride * npes) && pe_stride != min_stride) {
     fprintf(stderr,
             "rocshmem: no room for %d slices %zu bytes apart; packing them (stride = heap size)\n",
             npes, pe_stride);
     pe_stride = min_stride;
-    alloc_bytes = pe_stride * npes;
-    got = hipMalloc(reinterpret_cast<void **>(&heap_base), alloc_bytes);
+    try_block(pe_stride * npes);
   }
-  RT_CHECK_HIP(got);
+  if (!heap_base) {
+    fprintf(stderr, "rocshmem: cannot allocate %zu bytes of device memory for the symmetric heap\n",
+            pe_stride * npes);
+    exit(EXIT_FAILURE);
+  }
   heap_alloc_bytes = alloc_bytes;
   if (env_size("ROCSHMEM_EMU_VERBOSE", 0) != 0)
-    fprintf(stderr, "rocshmem: %d PEs, heap %zu B per PE, slices %zu B apart, %zu B allocated%s\n",
-            npes, heap_size, pe_stride, alloc_bytes, anchored ? " (placed)" : "");
+    fprintf(stderr, "rocshmem: %d PEs, heap %zu B per PE, slices %zu B apart, %zu B allocated%s%s\n",
+            npes, heap_size, pe_stride, alloc_bytes, anchored ? " (placed)" : "",
+            heap_cached_mode() ? " (cached)" : " (uncached)");
   allocator.reset(reinterpret_cast<uint64_t>(heap_base), heap_size);
 
   ws_stride = ws_bytes_per_pe();
@@ -378,7 +462,7 @@ void Runtime::finalize() {
   RT_CHECK_HIP(hipFree(d_default_ctx));
   RT_CHECK_HIP(hipFree(d_teams));
   RT_CHECK_HIP(hipFree(d_ws));
-  RT_CHECK_HIP(hipFree(heap_base));
+  release_heap_block(heap_base);
   heap_base = nullptr;
   d_ws = nullptr;
   d_teams = nullptr;

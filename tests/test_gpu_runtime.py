@@ -1,9 +1,14 @@
 """H1-H3, X2: bring-up, symmetric allocation on the device heap, PE
 addressing and teams through the C entry points."""
 import ctypes
+import os
+import subprocess
+import sys
 
 import numpy as np
 import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 pytestmark = pytest.mark.gpu
 
@@ -140,32 +145,36 @@ def test_default_layout_allocates_what_the_slices_need(rt, L, monkeypatch):
     2 MiB, one allocation of P strides.  A default rocshmem_init with 8 PEs and
     the default 1 GiB per PE leaves the rest of the device memory to the user:
     free memory afterwards is within 1 GiB of what was free before minus the
-    8 GiB of slices."""
-    monkeypatch.delenv("ROCSHMEM_EMU_PE_STRIDE", raising=False)
-    monkeypatch.delenv("ROCSHMEM_EMU_SPREAD", raising=False)
-    monkeypatch.delenv("ROCSHMEM_HEAP_SIZE", raising=False)
+    8 GiB of slices.  (In a process of its own: the heap is uncached memory,
+    which a process keeps and reuses once it has it.)"""
     rt.down()
-    l = L.load()
-    free0, free1, total = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()
-    assert l.dev_mem_info(ctypes.byref(free0), ctypes.byref(total)) == 0
-    assert l.init(8, 0) == 0
-    try:
-        assert l.heap_size() == 1 << 30 and l.pe_stride() == 1 << 30
-        assert l.heap_alloc_bytes() == 8 << 30
-        assert l.dev_mem_info(ctypes.byref(free1), ctypes.byref(total)) == 0
-        taken = free0.value - free1.value  # slices + work/sync area + contexts and teams
-        assert (8 << 30) - (64 << 20) <= taken <= (9 << 30), taken
-        # and the user can still allocate most of the device
-        big = l.dev_alloc(free1.value // 2)
-        assert big
-        l.dev_free(big)
-    finally:
-        l.finalize()
-    for npes, heap in ((3, (1 << 24) + 5), (5, 3 << 20)):
-        assert l.init(npes, heap) == 0
-        want = (heap + (2 << 20) - 1) // (2 << 20) * (2 << 20)
-        assert l.pe_stride() == want and l.heap_alloc_bytes() == want * npes
-        l.finalize()
+    code = (
+        "import ctypes, sys\n"
+        "sys.path.insert(0, %r)\n"
+        "from rocshmem_amd import lib as L\n"
+        "l = L.load()\n"
+        "f0, f1, tot = ctypes.c_size_t(), ctypes.c_size_t(), ctypes.c_size_t()\n"
+        "assert l.dev_mem_info(ctypes.byref(f0), ctypes.byref(tot)) == 0\n"
+        "assert l.init(8, 0) == 0\n"
+        "assert l.heap_size() == 1 << 30 and l.pe_stride() == 1 << 30\n"
+        "assert l.heap_alloc_bytes() == 8 << 30\n"
+        "assert l.dev_mem_info(ctypes.byref(f1), ctypes.byref(tot)) == 0\n"
+        "taken = f0.value - f1.value\n"
+        "assert (8 << 30) - (64 << 20) <= taken <= (9 << 30), taken\n"
+        "big = l.dev_alloc(f1.value // 2)\n"
+        "assert big\n"
+        "l.dev_free(big)\n"
+        "l.finalize()\n"
+        "for npes, heap in ((3, (1 << 24) + 5), (5, 3 << 20)):\n"
+        "    assert l.init(npes, heap) == 0\n"
+        "    want = (heap + (2 << 20) - 1) // (2 << 20) * (2 << 20)\n"
+        "    assert l.pe_stride() == want\n"
+        "    l.finalize()\n"
+        "print('ok')\n" % ROOT)
+    env = {k: v for k, v in os.environ.items()
+           if k not in ("ROCSHMEM_EMU_PE_STRIDE", "ROCSHMEM_EMU_SPREAD", "ROCSHMEM_HEAP_SIZE")}
+    r = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0 and "ok" in r.stdout, (r.stdout[-400:], r.stderr[-800:])
 
 
 def test_spread_layout_is_opt_in(rt, L, monkeypatch):
