@@ -30,9 +30,8 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X, published
 # HBM bytes one launch of the headline kernel moves, from FETCH_SIZE + WRITE_SIZE
-# under rocprofv3 --pmc (profiles/putmem_wg_tiled_256MiB_hbm_traffic.txt); None
-# until that profile has been taken for the current kernel.
-PUT_TRAFFIC_BYTES = None
+# under rocprofv3 --pmc (profiles/putmem_wg_tiled_256MiB_hbm_traffic.txt).
+PUT_TRAFFIC_BYTES = 536948703
 P = 8
 MiB = 1 << 20
 

@@ -133,6 +133,47 @@ __device__ __forceinline__ T from_lane(T v, int lane) {
   }
 }
 
+// One step of a wavefront-wide inclusive sum over all 64 lanes with DPP moves:
+// every lane adds the value `ctrl` brings it (0 where there is no source lane).
+template <typename T, int kCtrl, int kRowMask>
+__device__ __forceinline__ T dpp_add_step(T x) {
+  if constexpr (sizeof(T) == 8) {
+    unsigned long long b;
+    __builtin_memcpy(&b, &x, 8);
+    const unsigned lo = static_cast<unsigned>(__builtin_amdgcn_update_dpp(
+        0, static_cast<int>(static_cast<unsigned>(b)), kCtrl, kRowMask, 0xf, false));
+    const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_update_dpp(
+        0, static_cast<int>(static_cast<unsigned>(b >> 32)), kCtrl, kRowMask, 0xf, false));
+    const unsigned long long moved = (static_cast<unsigned long long>(hi) << 32) | lo;
+    T add;
+    __builtin_memcpy(&add, &moved, 8);
+    return static_cast<T>(x + add);
+  } else {
+    unsigned b;
+    __builtin_memcpy(&b, &x, 4);
+    const unsigned moved =
+        static_cast<unsigned>(__builtin_amdgcn_update_dpp(0, static_cast<int>(b), kCtrl, kRowMask, 0xf, false));
+    T add;
+    __builtin_memcpy(&add, &moved, 4);
+    return static_cast<T>(x + add);
+  }
+}
+// Inclusive prefix sum of x over lanes 0..63 in six DPP steps (shifts by 1, 2,
+// 4, 8 within rows of 16 lanes, then the last lane of row 0/2 and of rows 0-1
+// broadcast to the rows after them).  Every lane of the wavefront must be
+// active: a partial sum travels through the lanes between its source and its
+// destination.
+template <typename T>
+__device__ __forceinline__ T wave_inclusive_sum(T x) {
+  x = dpp_add_step<T, 0x111, 0xf>(x);  // row_shr:1
+  x = dpp_add_step<T, 0x112, 0xf>(x);  // row_shr:2
+  x = dpp_add_step<T, 0x114, 0xf>(x);  // row_shr:4
+  x = dpp_add_step<T, 0x118, 0xf>(x);  // row_shr:8
+  x = dpp_add_step<T, 0x142, 0xa>(x);  // row_bcast:15 into rows 1 and 3
+  x = dpp_add_step<T, 0x143, 0xc>(x);  // row_bcast:31 into rows 2 and 3
+  return x;
+}
+
 // Wavefront-aggregated add.  Lanes of the calling wavefront that target the
 // same word are merged: the lowest such lane issues ONE RMW with the sum, and
 // every lane of the group receives base + (sum of the group's lower lanes) —
@@ -140,38 +181,63 @@ __device__ __forceinline__ T from_lane(T v, int lane) {
 // back in lane order, so the fetched values remain a valid serialisation.
 // A hot word (skewed address streams) then costs one memory-side atomic per
 // wavefront instead of one per lane.  Groups are found by peeling: take the
-// first unassigned lane, ballot for its address, repeat; the search stops
-// early once kMissBudget lanes in a row turned out to be alone, which keeps
-// the cost flat for address streams without collisions.
+// first unassigned lane, ballot for its address, repeat; the search stops once
+// a number of lanes in a row turned out to be alone (six, plus four for every
+// group found so far: a stream that has shown one hot word tends to have
+// more), which keeps the cost flat for address streams without collisions.
+// The lower-lane sums of a group come from the lane count when all its addends
+// are equal (fetch_inc, add of a constant), from a six-step DPP prefix sum over
+// the wavefront when the group is large and the wavefront full, and from a walk
+// over the group's lanes otherwise.
 template <typename T, bool kFetch>
 __device__ __forceinline__ T amo_add_wave(T *p, T v, bool relaxed) {
-  constexpr int kMissBudget = 6;
+  constexpr int kMissBudget = 6, kMissBudgetPerGroup = 4, kScanFrom = 5;
   const unsigned lane = lane_index();
   const unsigned long long addr = reinterpret_cast<unsigned long long>(p);
-  unsigned long long rem = __ballot(1);
+  const unsigned long long active = __ballot(1);
+  unsigned long long rem = active;
   int leader = static_cast<int>(lane);
   T prefix = static_cast<T>(0);
   T total = v;
-  int misses = 0;
-  while (rem && misses < kMissBudget) {
+  int misses = 0, budget = kMissBudget;
+  while (rem && misses < budget) {
     const int l = __ffsll(static_cast<long long>(rem)) - 1;
     const unsigned long long a = read_lane(addr, l);
     const bool mine = addr == a;
     const unsigned long long same = __ballot(mine);
     if (same & (same - 1)) {  // two or more lanes share this word
       misses = 0;
-      T run = static_cast<T>(0);
-      unsigned long long m = same;
-      while (m) {
-        const int j = __ffsll(static_cast<long long>(m)) - 1;
-        const T vj = read_lane(v, j);
-        if (static_cast<int>(lane) == j) prefix = run;
-        run = static_cast<T>(run + vj);
-        m &= m - 1;
+      budget += kMissBudgetPerGroup;
+      const int members = __popcll(same);
+      const T v_first = read_lane(v, l);
+      T before, sum;  // of this lane's group: addends of its lower lanes, all addends
+      if (__ballot(mine && v != v_first) == 0) {
+        const unsigned below = __builtin_amdgcn_mbcnt_hi(
+            static_cast<unsigned>(same >> 32), __builtin_amdgcn_mbcnt_lo(static_cast<unsigned>(same), 0u));
+        before = static_cast<T>(v_first * static_cast<T>(below));
+        sum = static_cast<T>(v_first * static_cast<T>(members));
+      } else if (members >= kScanFrom && active == ~0ull) {
+        const T mine_v = mine ? v : static_cast<T>(0);
+        const T upto = wave_inclusive_sum<T>(mine_v);
+        before = static_cast<T>(upto - mine_v);
+        sum = read_lane(upto, 63);
+      } else {
+        T run = static_cast<T>(0);
+        before = run;
+        unsigned long long m = same;
+        while (m) {
+          const int j = __ffsll(static_cast<long long>(m)) - 1;
+          const T vj = read_lane(v, j);
+          if (static_cast<int>(lane) == j) before = run;
+          run = static_cast<T>(run + vj);
+          m &= m - 1;
+        }
+        sum = run;
       }
       if (mine) {
         leader = l;
-        total = run;
+        prefix = before;
+        total = sum;
       }
     } else {
       ++misses;

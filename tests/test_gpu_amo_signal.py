@@ -101,6 +101,33 @@ def test_int64_fetch_add_histogram(rt, L, orc, dist):
     ctr.free()
 
 
+@pytest.mark.parametrize("dtype_name", ["INT", "UINT", "LONG", "ULONGLONG"])
+@pytest.mark.parametrize("K,n,wg", [(8, 64 * 257, 256), (3, 1000, 64), (64, 64 * 64 + 17, 192)])
+def test_fetch_add_lanes_that_share_a_word_are_merged_correctly(rt, L, orc, dtype_name, K, n, wg):
+    """Few counters, so most lanes of a wavefront share their word with many
+    others: the merged add must hand every lane base + the sum of its group's
+    lower lanes whether that sum comes from the lane count (equal addends), the
+    DPP prefix sum (large groups in full wavefronts) or the walk (small groups,
+    partly filled wavefronts: n is not a multiple of 64).  Final counters exact,
+    fetched values a valid serialisation, for 32- and 64-bit types."""
+    l = rt.up(P, HEAP)
+    np_t = NP[dtype_name]
+    ids = (orc.fill_u64(n, 7, K) % K).astype(np.uint32) * (P * 16 // K)  # spread over the PEs
+    ctr = Counters(rt, l, 16, np_t)
+    for vals in ((orc.fill_u64(n, 8, 1) % 5 + 1).astype(np_t), np.full(n, 3, np_t)):
+        ctr.set_all(np.zeros(P * 16, np_t))
+        fetched = run_amo(rt, l, L, L.AMO_FETCH_ADD, dtype_name, ctr, ids, values=vals, n_wgs=7, wg=wg)
+        want = np.zeros(P * 16, np.int64)
+        np.add.at(want, ids, vals.astype(np.int64))
+        assert np.array_equal(ctr.read_all().astype(np.int64), want)
+        check_fetch_chain(ids, fetched.astype(np.int64), vals.astype(np.int64), 0)
+        # the non-fetching form lands the same totals
+        ctr.set_all(np.zeros(P * 16, np_t))
+        run_amo(rt, l, L, L.AMO_ADD, dtype_name, ctr, ids, values=vals, fetch=False, n_wgs=7, wg=wg)
+        assert np.array_equal(ctr.read_all().astype(np.int64), want)
+    ctr.free()
+
+
 @pytest.mark.parametrize("dtype_name", ["INT", "LONG", "LONGLONG", "UINT", "ULONG", "ULONGLONG"])
 def test_standard_amos_known_answers(rt, L, orc, dtype_name):
     """tests/functional_tests/amo_standard_tester.cpp:77-117,131-160: m calls on
