@@ -149,6 +149,13 @@ def headline(b, steps, warmup):
         rotating(lambda me, pe: l.putmem(dsts[me], srcs[me], n, me, pe, None)), steps, warmup) / 1e6
     out["host_getmem_gbs"] = 2 * n / b.time_ms(
         rotating(lambda me, pe: l.getmem(dsts[me], srcs[me], n, me, pe, None)), steps, warmup) / 1e6
+    # rocshmem_ctx_getmem_wg from every CU, the shape of the headline put
+    l.set_ctx_options(1)
+    wg, tile, _ = PUT_SHAPES["nostore_ctx"]
+    out["getmem_wg_gbs"] = 2 * n / b.time_ms(
+        rotating(lambda me, pe: l.rma(L.GET, L.WG, dsts[me], srcs[me], n, tile, me, pe, n // tile, wg, 1,
+                                      None)), steps, warmup) / 1e6
+    l.set_ctx_options(0)
     if b.quick:
         l.free(src)
         l.free(dst)
@@ -582,7 +589,9 @@ def main():
             "putmem_wg_all_cus_frac": frac(head["default_ctx_gbs"]),
             "host_putmem_gbs": round(head["host_putmem_gbs"], 1),
             "host_putmem_frac": frac(head["host_putmem_gbs"]),
-            "host_getmem_gbs": round(head["host_getmem_gbs"], 1)}
+            "host_getmem_gbs": round(head["host_getmem_gbs"], 1),
+            "getmem_wg_all_cus_gbs_nostore": round(head["getmem_wg_gbs"], 1),
+            "getmem_wg_all_cus_frac_nostore": frac(head["getmem_wg_gbs"])}
     if not a.quick:
         ta, a2a = allc["to_all_P8_64Mi"], allc["alltoall_512x7168_bf16"]
         dp, amo, pp = allc["dispatch_put_signal"], allc["atomic_fetch_add_16Mi"], allc["pingpong"]
