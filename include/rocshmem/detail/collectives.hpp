@@ -22,7 +22,7 @@ namespace detail {
 // ROCSHMEM_CTX_NOSTORE (include/rocshmem/rocshmem_common.hpp; the reference
 // switches its flush off for that option, src/fence_policy.hpp:45-63).
 __device__ __forceinline__ int publish_of(const Context *c) {
-  return (c->options & static_cast<unsigned>(ROCSHMEM_CTX_NOSTORE)) ? PUBLISH_LIBRARY : PUBLISH_ALL;
+  return (ctx_view(c)->options & static_cast<unsigned>(ROCSHMEM_CTX_NOSTORE)) ? PUBLISH_LIBRARY : PUBLISH_ALL;
 }
 
 __device__ __forceinline__ void team_pad_sync(const Context *c, Team *t, int kind, int publish) {
@@ -32,7 +32,7 @@ __device__ __forceinline__ void team_pad_sync(const Context *c, Team *t, int kin
 
 // src/ipc/context_ipc_device_coll.cpp:101-123
 __device__ __forceinline__ void sync_all(Context *c) {
-  sync_pes(c, c->world_sync, 0, 1, c->num_pes, c->my_pe, publish_of(c));
+  sync_pes(c, ctx_view(c)->world_sync, 0, 1, ctx_view(c)->num_pes, ctx_view(c)->my_pe, publish_of(c));
 }
 __device__ __forceinline__ void barrier_all(Context *c) {
   // quiet() of the calling PE is the release half of the barrier's first step.
@@ -61,10 +61,10 @@ __device__ __forceinline__ int wg_reduce(Context *c, Team *t,
   team_pad_sync(c, t, SYNC_REDUCE, publish_of(c));
 
   const size_t n = static_cast<size_t>(nreduce);
-  const int64_t to_first = static_cast<int64_t>(t->wrt_world.pe_start - c->my_pe) *
-                           static_cast<int64_t>(c->pe_stride);
+  const int64_t to_first = static_cast<int64_t>(t->wrt_world.pe_start - ctx_view(c)->my_pe) *
+                           static_cast<int64_t>(ctx_view(c)->pe_stride);
   const int64_t hop = static_cast<int64_t>(t->wrt_world.stride) *
-                      static_cast<int64_t>(c->pe_stride);
+                      static_cast<int64_t>(ctx_view(c)->pe_stride);
   S *dst0 = reinterpret_cast<S *>(reinterpret_cast<char *>(dest) + to_first);
   const S *src0 = reinterpret_cast<const S *>(reinterpret_cast<const char *>(source) + to_first);
   // The members share the whole range block by block (see fold_window).  Arrays

@@ -78,82 +78,138 @@ __device__ __forceinline__ u32x4 load16(const char *p) {
     return *reinterpret_cast<const u32x4_any *>(p);
   }
 }
+// The same from a pointer known to name device (global) memory, split into a
+// wave-uniform base and a 32-bit byte offset per lane: a global_load with the
+// base in scalar registers and one address register.  A load through a
+// generic pointer is a flat instruction, which the hardware may also route to
+// LDS or scratch; the compiler then has to wait for all outstanding memory
+// operations before it uses the result, and the pipelining below is lost.
+typedef const __attribute__((address_space(1))) char *GlobalBytes;
+typedef const __attribute__((address_space(1))) u32x4_any *GlobalVec;
+template <bool kNonTemporal>
+__device__ __forceinline__ u32x4 load16(GlobalBytes base, uint32_t off) {
+  if constexpr (kNonTemporal) {
+    return __builtin_nontemporal_load((GlobalVec)(base + off));  // NOLINT
+  } else {
+    return *(GlobalVec)(base + off);  // NOLINT
+  }
+}
+__device__ __forceinline__ GlobalBytes wave_uniform_global(const char *p) {
+  const uint64_t a = reinterpret_cast<uint64_t>(p);
+  const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(a));
+  const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(a >> 32));
+  return (GlobalBytes)((static_cast<uint64_t>(hi) << 32) | lo);  // NOLINT
+}
+// True when a generic pointer names LDS or private (scratch) memory.
+__device__ __forceinline__ bool in_lds_or_scratch(const void *p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __builtin_amdgcn_is_shared(p) || __builtin_amdgcn_is_private(p);
+#else
+  (void)p;  // the host pass only parses device functions
+  return false;
+#endif
+}
+
+// The local side of a put or get may be a __shared__ array or a stack
+// variable (the reference copies through generic pointers, so it accepts
+// them).  Buffer stores and global loads cannot reach those, so such a copy
+// goes through flat accesses, 16 bytes per lane per step and bytes at the end.
+__device__ __forceinline__ void copy_generic(char *dst, const char *src, size_t n, size_t lane,
+                                          size_t nlanes) {
+  const size_t nvec = n >> 4;
+  for (size_t i = lane; i < nvec; i += nlanes)
+    *reinterpret_cast<u32x4_any *>(dst + (i << 4)) =
+        *reinterpret_cast<const u32x4_any *>(src + (i << 4));
+  for (size_t k = (nvec << 4) + lane; k < n; k += nlanes) dst[k] = src[k];
+}
 
 // Copy n <= kWindowBytes bytes with `nlanes` cooperating lanes; this lane is
 // number `lane` (0-based, dense).  Lanes need not belong to one wavefront or
-// work-group: a whole grid can call this with global thread ids.
+// work-group: a whole grid can call this with global thread ids.  dst, src
+// and n are the same in every lane of a wavefront.
 template <int kUnroll, bool kNonTemporal>
-__device__ __forceinline__ void copy_window(char *dst, const char *src, size_t n, size_t lane,
+__device__ __forceinline__ void copy_window(char *dst, const char *src_any, size_t n, size_t lane,
                                             size_t nlanes) {
+  if (__builtin_expect(in_lds_or_scratch(dst) || in_lds_or_scratch(src_any), 0)) {
+    copy_generic(dst, src_any, n, lane, nlanes);
+    return;
+  }
   const __amdgpu_buffer_rsrc_t w = window_of(dst, n);
   size_t head = (16u - (reinterpret_cast<uintptr_t>(dst) & 15u)) & 15u;
   if (head > n) head = n;
-  for (size_t k = lane; k < head; k += nlanes) store1(w, static_cast<uint32_t>(k), src[k]);
-  src += head;
+  for (size_t k = lane; k < head; k += nlanes) store1(w, static_cast<uint32_t>(k), src_any[k]);
+  const GlobalBytes src = wave_uniform_global(src_any + head);
   const size_t body = n - head;
   const uint32_t base = static_cast<uint32_t>(head);
 
   const size_t nvec = body >> 4;
-  size_t i = lane;
+  const size_t span = static_cast<size_t>(kUnroll) * nlanes;
+  auto load_batch = [&](u32x4 (&v)[kUnroll], size_t first) {
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+      v[u] = load16<kNonTemporal>(src, static_cast<uint32_t>((first + lane + u * nlanes) << 4));
+  };
+  auto store_batch = [&](const u32x4 (&v)[kUnroll], size_t first) {
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+      store16<kNonTemporal>(w, base + static_cast<uint32_t>((first + lane + u * nlanes) << 4), v[u]);
+  };
+  // Whole batches of kUnroll vectors per lane: all loads of a batch, then all
+  // its stores; the stores are not waited for, so they overlap the next
+  // batch's loads.  Measured on MI355X with 256 work-groups of 1024 lanes
+  // streaming 900 KB messages each: batches of 8 give 6.15 TB/s, of 4 6.0, of 2
+  // 5.4; keeping a second batch loading while the first is stored (two
+  // register sets taking turns) loses 2-7 % against the plain alternation.
+  size_t done_vec = 0;  // vectors [0, done_vec) are on their way; uniform
   if constexpr (kUnroll > 1) {
-    // Two batches of kUnroll vectors: the loads of the next batch are issued
-    // before the stores of the current one, so a lane always has loads in
-    // flight while it waits.
-    const size_t span = static_cast<size_t>(kUnroll) * nlanes;
-    if (i + span - nlanes < nvec) {
-      u32x4 v[kUnroll];
-#pragma unroll
-      for (int u = 0; u < kUnroll; ++u)
-        v[u] = load16<kNonTemporal>(src + ((i + u * nlanes) << 4));
-      for (i += span; i + span - nlanes < nvec; i += span) {
-        u32x4 next[kUnroll];
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u)
-          next[u] = load16<kNonTemporal>(src + ((i + u * nlanes) << 4));
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u)
-          store16<kNonTemporal>(w, base + static_cast<uint32_t>((i - span + u * nlanes) << 4), v[u]);
-#pragma unroll
-        for (int u = 0; u < kUnroll; ++u) v[u] = next[u];
-      }
-#pragma unroll
-      for (int u = 0; u < kUnroll; ++u)
-        store16<kNonTemporal>(w, base + static_cast<uint32_t>((i - span + u * nlanes) << 4), v[u]);
+    u32x4 v[kUnroll];
+    for (; done_vec + span <= nvec; done_vec += span) {
+      load_batch(v, done_vec);
+      store_batch(v, done_vec);
     }
   }
-  for (; i < nvec; i += nlanes)
-    store16<kNonTemporal>(w, base + static_cast<uint32_t>(i << 4),
-                          load16<kNonTemporal>(src + (i << 4)));
+  // Fewer than kUnroll vectors per lane are left (any number when kUnroll is
+  // 1): all of a lane's are loaded before the first is stored, so a message of
+  // up to kUnroll vectors per lane costs one memory round trip, not one per
+  // vector.
+  for (size_t i = done_vec + lane; i < nvec; i += span) {
+    u32x4 v[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+      if (i + u * nlanes < nvec)
+        v[u] = load16<kNonTemporal>(src, static_cast<uint32_t>((i + u * nlanes) << 4));
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u)
+      if (i + u * nlanes < nvec)
+        store16<kNonTemporal>(w, base + static_cast<uint32_t>((i + u * nlanes) << 4), v[u]);
+  }
 
-  const size_t done = nvec << 4;
+  const uint32_t done = static_cast<uint32_t>(nvec << 4);
   const size_t tail = body - done;
   for (size_t k = lane; k < tail; k += nlanes)
-    store1(w, base + static_cast<uint32_t>(done + k), src[done + k]);
+    store1(w, base + done + static_cast<uint32_t>(k), src[done + k]);
 }
 
 // Any size: 1 GiB windows, one buffer resource each.
 template <int kUnroll, bool kNonTemporal>
 __device__ __forceinline__ void copy_lanes_impl(char *dst, const char *src, size_t n, size_t lane,
                                                 size_t nlanes) {
-  while (n > kWindowBytes) {
-    copy_window<kUnroll, kNonTemporal>(dst, src, kWindowBytes, lane, nlanes);
-    dst += kWindowBytes;
-    src += kWindowBytes;
-    n -= kWindowBytes;
-  }
-  copy_window<kUnroll, kNonTemporal>(dst, src, n, lane, nlanes);
+  do {
+    const size_t chunk = n < kWindowBytes ? n : kWindowBytes;
+    copy_window<kUnroll, kNonTemporal>(dst, src, chunk, lane, nlanes);
+    dst += chunk;
+    src += chunk;
+    n -= chunk;
+  } while (n);
 }
 
-// kLoads: 16-byte vectors per batch; the loop keeps two batches per lane (the
-// next one loading while the current one is stored), which measured 3 % more
-// for a put_signal dispatch of 900 KB messages and 17 % more for a lone
-// wavefront than one batch at a time.  Batches of 4 saturate a CU when a full
-// work-group copies (batches of 2 lose 10-40 %); a lone wavefront needs 8 to
-// cover the memory latency.  The register count of a kernel is that of its
-// widest path (about 100 VGPRs with batches of 4, the limit of 128 for a
-// 1024-lane work-group with batches of 8), so the deeper variant is chosen
-// per call site, not at run time.
-template <int kLoads = 4>
+// kLoads: 16-byte vectors a lane loads before it stores them.  A message of up
+// to kLoads vectors per lane costs one memory round trip; longer ones alternate
+// bursts of kLoads loads and kLoads stores.  Eight covers the memory latency
+// for a lone wavefront and is the best burst length for full work-groups that
+// stream long messages (see copy_window); the loop needs 4 * kLoads data
+// registers.
+template <int kLoads = 8>
 __device__ __forceinline__ void copy_lanes(void *dst, const void *src, size_t n, size_t lane,
                                            size_t nlanes,
                                            size_t nt_bytes = kNonTemporalBytes) {
@@ -217,7 +273,7 @@ __device__ __forceinline__ void copy_wave(void *dst, const void *src, size_t n,
                                           size_t nt_bytes = kNonTemporalBytes) {
   unsigned count;
   const unsigned rank = active_lane_rank(&count);
-  copy_lanes<8>(dst, src, n, rank, count, nt_bytes);
+  copy_lanes(dst, src, n, rank, count, nt_bytes);
 }
 
 }  // namespace detail

@@ -28,7 +28,7 @@ __device__ __forceinline__ int translate_pe(rocshmem_ctx_t ctx, int pe) {
 // after another, about 60 ns each when idle and a memory round trip each while
 // stores are in flight.
 __device__ __forceinline__ bool no_store_order(const Context *c) {
-  return (c->options & static_cast<unsigned>(ROCSHMEM_CTX_NOSTORE)) != 0;
+  return (ctx_view(c)->options & static_cast<unsigned>(ROCSHMEM_CTX_NOSTORE)) != 0;
 }
 // quiet / fence on context c.
 __device__ __forceinline__ void ctx_release(const Context *c) {
@@ -198,21 +198,21 @@ __device__ __forceinline__ Context *pool_claim(CtxPool *pool) {
   return nullptr;
 }
 __device__ __forceinline__ void pool_release(CtxPool *pool, Context *c) {
-  const int s = c->pool_slot;
+  const int s = ctx_view(c)->pool_slot;
   __hip_atomic_fetch_or(&pool->free_mask[s >> 6], 1ull << (s & 63), __ATOMIC_RELEASE,
                         __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Thread 0 claims a context of PE `pe` bound to `tinfo`; every thread learns
-// the outcome through *ctx (which lives in the caller's shared memory).
+// the outcome through *ctx (which lives in the caller's shared memory).  Each
+// pool slot holds one prebuilt object per ordering option, so nothing is
+// written into a context here; the team travels in the handle.
 __device__ __forceinline__ int wg_ctx_create_for(int pe, TeamInfo *tinfo, long options,
                                                  rocshmem_ctx_t *ctx) {
   if (is_block_leader()) {
-    Context *c = pool_claim(g_state.ctx_pool + pe);
-    if (c) {
-      c->tinfo = tinfo;
-      c->options = static_cast<unsigned>(options);
-    }
+    CtxPool *pool = g_state.ctx_pool + pe;
+    Context *c = pool_claim(pool);
+    if (c && (options & ROCSHMEM_CTX_NOSTORE)) c += pool->capacity;
     ctx->ctx_opaque = c;
     ctx->team_opaque = tinfo;
   }
@@ -223,7 +223,7 @@ __device__ __forceinline__ int wg_ctx_create_for(int pe, TeamInfo *tinfo, long o
 __device__ __forceinline__ void wg_ctx_destroy(rocshmem_ctx_t *ctx) {
   if (is_block_leader()) {
     Context *c = reinterpret_cast<Context *>(ctx->ctx_opaque);
-    if (c && c->pool_slot >= 0) pool_release(g_state.ctx_pool + c->my_pe, c);
+    if (c && ctx_view(c)->pool_slot >= 0) pool_release(g_state.ctx_pool + ctx_view(c)->my_pe, c);
   }
 }
 

@@ -92,16 +92,18 @@ struct Team {
   void *pWrk;          // ROCSHMEM_REDUCE_MIN_WRKDATA_SIZE * 8 bytes
 };
 
-// Per-PE communication context (device memory, pooled).
+// Per-PE communication context (device memory, pooled).  Kernels never write
+// a context: the host fills them all in at initialisation, so device code
+// reads them through the scalar data path (see ctx_view).
 struct Context {
   char *heap_base;      // base of PE 0's slice
   uint64_t pe_stride;   // bytes between consecutive slices
   uint64_t ws_stride;   // bytes between consecutive PEs' work/sync areas
   int my_pe;
   int num_pes;
-  TeamInfo *tinfo;      // team this context translates PE numbers with
+  TeamInfo *tinfo;      // world team of this PE
   SyncPad *world_sync;  // this PE's pad for barrier_all / sync_all
-  unsigned options;
+  unsigned options;     // ROCSHMEM_CTX_* bits, fixed per object
   int pool_slot;        // index in the context pool, -1 for default contexts
 };
 
@@ -109,12 +111,15 @@ struct Context {
 // slot; claiming is a fetch-and that clears the bit, releasing a fetch-or, so
 // work-groups never hold a lock (the reference guards a free list with a
 // ticket mutex, src/containers/free_list_impl.hpp:76-137).
+// Slot s stands for two prebuilt objects, slots[s] with no option and
+// slots[capacity + s] with ROCSHMEM_CTX_NOSTORE, so that claiming a context
+// with either option writes nothing into it.
 struct CtxPool {
   static constexpr int kMaxWords = 64;  // up to 4096 contexts per PE
   unsigned long long free_mask[kMaxWords];
   int capacity;
   int pad_;
-  Context *slots;       // [capacity]
+  Context *slots;       // [2 * capacity]
 };
 
 struct DeviceState {
@@ -148,18 +153,16 @@ __device__ __forceinline__ unsigned long long dispatch_queue_id() {
 }
 
 __device__ __forceinline__ int acting_pe() {
-  const int n = g_state.n_pes;
-  switch (g_state.pe_rule) {
-    case PE_RULE_BLOCK_X: return static_cast<int>(blockIdx.x % n);
-    case PE_RULE_BLOCK_Y: return static_cast<int>(blockIdx.y % n);
-    case PE_RULE_BLOCK_Z: return static_cast<int>(blockIdx.z % n);
-    case PE_RULE_QUEUE: {
-      const unsigned long long id = dispatch_queue_id();
-      const QueueBinding b = g_state.queue_table[id % kQueueTableSize];
-      return b.queue_id == id ? b.pe : g_state.fixed_pe;
-    }
-    default: return g_state.fixed_pe;
+  const int rule = g_state.pe_rule;
+  if (rule == PE_RULE_FIXED) return g_state.fixed_pe;
+  if (rule == PE_RULE_QUEUE) {
+    const unsigned long long id = dispatch_queue_id();
+    const QueueBinding b = g_state.queue_table[id % kQueueTableSize];
+    return b.queue_id == id ? b.pe : g_state.fixed_pe;
   }
+  const unsigned block = rule == PE_RULE_BLOCK_X ? blockIdx.x
+                         : rule == PE_RULE_BLOCK_Y ? blockIdx.y : blockIdx.z;
+  return static_cast<int>(block % static_cast<unsigned>(g_state.n_pes));
 }
 
 // A null ctx_opaque denotes the default context of the acting PE.
@@ -182,11 +185,22 @@ __device__ __forceinline__ Team *team_of(rocshmem_team_t team) {
   return t->my_pe < 0 ? nullptr : t;
 }
 
+// A context as read-only data in the constant address space.  The address of a
+// context is the same in every lane of a wavefront, and nothing writes a
+// context while kernels run, so its fields can come through the scalar data
+// cache (one s_load shared by the wavefront, a fraction of the latency of a
+// vector load that queues behind the wavefront's bulk traffic).  The compiler
+// only chooses that path for memory it knows to be constant.
+typedef const __attribute__((address_space(4))) Context ContextView;
+__device__ __forceinline__ ContextView *ctx_view(const Context *c) {
+  return (ContextView *)c;  // NOLINT: address-space cast
+}
+
 // Address of the same symmetric object on PE `pe`.
 template <typename T>
 __device__ __forceinline__ T *remote_addr(const Context *c, T *local, int pe) {
-  const int64_t hop = static_cast<int64_t>(pe - c->my_pe) *
-                      static_cast<int64_t>(c->pe_stride);
+  const int64_t hop = static_cast<int64_t>(pe - ctx_view(c)->my_pe) *
+                      static_cast<int64_t>(ctx_view(c)->pe_stride);
   return reinterpret_cast<T *>(
       reinterpret_cast<char *>(const_cast<typename std::remove_const<T>::type *>(local)) + hop);
 }
@@ -194,17 +208,33 @@ __device__ __forceinline__ T *remote_addr(const Context *c, T *local, int pe) {
 // Address of the same work/sync object on PE `pe`.
 template <typename T>
 __device__ __forceinline__ T *remote_ws(const Context *c, T *local, int pe) {
-  const int64_t hop = static_cast<int64_t>(pe - c->my_pe) *
-                      static_cast<int64_t>(c->ws_stride);
+  const int64_t hop = static_cast<int64_t>(pe - ctx_view(c)->my_pe) *
+                      static_cast<int64_t>(ctx_view(c)->ws_stride);
   return reinterpret_cast<T *>(reinterpret_cast<char *>(local) + hop);
 }
 
+// Work-group extents.  The three 16-bit sizes sit at bytes 12, 14 and 16 of
+// the implicit kernel arguments (code object version 5 and later, hipcc's
+// default; earlier versions are not supported); read as
+// the two aligned words that hold them they come through scalar loads, where
+// blockDim.y and .z read one by one get merged into a misaligned word that
+// only the vector memory path can fetch.
+struct BlockExtent {
+  unsigned x, y, z;
+};
+__device__ __forceinline__ BlockExtent block_extent() {
+  typedef const __attribute__((address_space(4))) uint32_t const_u32;
+  const_u32 *ia = (const_u32 *)__builtin_amdgcn_implicitarg_ptr();  // NOLINT
+  const uint32_t xy = ia[3], z = ia[4];
+  return BlockExtent{xy & 0xffffu, xy >> 16, z & 0xffffu};
+}
 __device__ __forceinline__ unsigned flat_thread_id() {
-  return threadIdx.x + threadIdx.y * blockDim.x +
-         threadIdx.z * blockDim.x * blockDim.y;
+  const BlockExtent b = block_extent();
+  return threadIdx.x + (threadIdx.y + threadIdx.z * b.y) * b.x;
 }
 __device__ __forceinline__ unsigned flat_block_size() {
-  return blockDim.x * blockDim.y * blockDim.z;
+  const BlockExtent b = block_extent();
+  return b.x * b.y * b.z;
 }
 __device__ __forceinline__ bool is_block_leader() { return flat_thread_id() == 0; }
 __device__ __forceinline__ bool is_wave_leader() {

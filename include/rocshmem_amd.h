@@ -258,6 +258,24 @@ int rocshmem_amd_timer_destroy(void *timer);
 int rocshmem_amd_rma(int rma_op, int gran, void *dest, const void *source, size_t nbytes,
                      size_t tile_bytes, int my_pe, int pe, int n_wgs, int wg_size,
                      int iters, rocshmem_amd_stream_t stream);
+
+/* The same calls with the local buffer in LDS: one work-group stages `nbytes`
+ * of `source` (a device buffer) in a __shared__ array, puts from there to
+ * `dest` on `pe` (rocshmem_ctx_putmem[_wave|_wg] + quiet), gets the bytes back
+ * from `pe` into a second __shared__ array at an odd offset, and copies that
+ * array to `back` (a device buffer).  The reference copies through generic
+ * pointers, so it accepts __shared__ and stack buffers on the local side
+ * (src/util.hpp:170-262); nbytes <= ROCSHMEM_AMD_STAGED_MAX_BYTES. */
+#define ROCSHMEM_AMD_STAGED_MAX_BYTES 24576
+int rocshmem_amd_rma_staged(int gran, void *dest, const void *source, void *back, size_t nbytes,
+                            int my_pe, int pe, int wg_size, rocshmem_amd_stream_t stream);
+
+/* Work-group rank and size as the _wg calls compute them (the flat thread id
+ * of the reference's get_flat_block_id / get_flat_block_size, src/util.hpp:100-118),
+ * for a block of bx x by x bz threads: out_host[0] = the size seen by rank 0,
+ * out_host[1 + r] = how many threads computed rank r, for r < 1024
+ * (out_host holds 1026 words). */
+int rocshmem_amd_flat_ids(int bx, int by, int bz, unsigned *out_host);
 /* Host-initiated bulk copy between PEs over the whole GPU: the host-side
  * rocshmem_putmem / rocshmem_getmem (rocshmem_RMA.hpp; reference forwards them
  * to MPI_Put / MPI_Get, src/host/host_helpers.hpp:52-88). */

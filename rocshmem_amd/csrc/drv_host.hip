@@ -111,8 +111,8 @@ int rocshmem_amd_ctx_pe(const void *ctx_opaque) {
   const auto *c = static_cast<const detail::Context *>(ctx_opaque);
   if (c >= r.d_default_ctx && c < r.d_default_ctx + 2 * r.npes)
     return static_cast<int>((c - r.d_default_ctx) % r.npes);
-  if (c >= r.d_ctx_slots && c < r.d_ctx_slots + static_cast<size_t>(r.npes) * r.max_ctxs)
-    return static_cast<int>((c - r.d_ctx_slots) / r.max_ctxs);
+  if (c >= r.d_ctx_slots && c < r.d_ctx_slots + static_cast<size_t>(r.npes) * 2 * r.max_ctxs)
+    return static_cast<int>((c - r.d_ctx_slots) / (2 * r.max_ctxs));
   return -1;
 }
 

@@ -36,10 +36,9 @@ __global__ void rma_kernel(RmaArgs a) {
     group = blockIdx.x * bs + tid;
     groups = gridDim.x * bs;
   }
-  const size_t ntiles = (a.nbytes + a.tile - 1) / a.tile;
+  const size_t stride = groups * a.tile;
   for (int it = 0; it < a.iters; ++it) {
-    for (size_t t = group; t < ntiles; t += groups) {
-      const size_t off = t * a.tile;
+    for (size_t off = group * a.tile; off < a.nbytes; off += stride) {
       const size_t len = a.nbytes - off < a.tile ? a.nbytes - off : a.tile;
       if constexpr (kOp == ROCSHMEM_AMD_PUT) {
         if constexpr (kGran == ROCSHMEM_AMD_WG)
@@ -74,6 +73,57 @@ __global__ void rma_kernel(RmaArgs a) {
   }
   // One quiet per group, as a kernel that batches its puts would issue it.
   if (kGran != ROCSHMEM_AMD_WG || threadIdx.x == 0) rocshmem_ctx_quiet(a.ctx);
+}
+
+// A put whose source is a __shared__ array, then a get whose destination is
+// one: the local side of either call may be LDS (the reference copies through
+// generic pointers), which the buffer stores and global loads of the
+// cooperative copy cannot reach.
+struct StagedArgs {
+  char *dest;
+  const char *source;
+  char *back;
+  size_t nbytes;
+  rocshmem_ctx_t ctx;
+  int pe;
+  int gran;
+};
+__global__ void staged_kernel(StagedArgs a) {
+  extern __shared__ __attribute__((aligned(16))) char staged_lds[];
+  char *out = staged_lds;
+  char *in = staged_lds + ((a.nbytes + 15) & ~size_t{15}) + 3;  // odd offset on purpose
+  for (size_t i = threadIdx.x; i < a.nbytes; i += blockDim.x) {
+    out[i] = a.source[i];
+    in[i] = 0;
+  }
+  __syncthreads();
+  if (a.gran == ROCSHMEM_AMD_WG) {
+    rocshmem_ctx_putmem_wg(a.ctx, a.dest, out, a.nbytes, a.pe);
+    rocshmem_ctx_quiet(a.ctx);
+    __syncthreads();
+    rocshmem_ctx_getmem_wg(a.ctx, in, a.dest, a.nbytes, a.pe);
+  } else if (a.gran == ROCSHMEM_AMD_WAVE) {
+    if (threadIdx.x < 64) {
+      rocshmem_ctx_putmem_wave(a.ctx, a.dest, out, a.nbytes, a.pe);
+      rocshmem_ctx_quiet(a.ctx);
+      rocshmem_ctx_getmem_wave(a.ctx, in, a.dest, a.nbytes, a.pe);
+    }
+  } else if (threadIdx.x == 0) {
+    rocshmem_ctx_putmem(a.ctx, a.dest, out, a.nbytes, a.pe);
+    rocshmem_ctx_quiet(a.ctx);
+    rocshmem_ctx_getmem(a.ctx, in, a.dest, a.nbytes, a.pe);
+  }
+  __syncthreads();
+  for (size_t i = threadIdx.x; i < a.nbytes; i += blockDim.x) a.back[i] = in[i];
+}
+
+// The library's own view of a thread's rank in its work-group and of the
+// work-group's size, for any block shape: out[0] = size, out[1 + r] = number
+// of threads that believe their rank is r (each must be 1).
+__global__ void flat_ids_kernel(unsigned *out) {
+  const unsigned r = detail::flat_thread_id();
+  if (r == 0) out[0] = detail::flat_block_size();
+  atomicAdd(&out[1 + (r < 1024 ? r : 1024)], 1u);
 }
 
 // Whole-GPU copy: every thread of the grid is one lane of a single
@@ -250,6 +300,41 @@ int rocshmem_amd_rma(int rma_op, int gran, void *dest, const void *source, size_
   RMA_CASE(ROCSHMEM_AMD_GET_NBI, ROCSHMEM_AMD_WG)
 #undef RMA_CASE
   DRV_CHECK_HIP(hipGetLastError());
+  return 0;
+}
+
+int rocshmem_amd_rma_staged(int gran, void *dest, const void *source, void *back, size_t nbytes,
+                            int my_pe, int pe, int wg_size, rocshmem_amd_stream_t stream) {
+  if (!valid_pe(my_pe) || !valid_pe(pe) || !valid_launch(1, wg_size)) return -1;
+  if (gran < ROCSHMEM_AMD_THREAD || gran > ROCSHMEM_AMD_WG) return -1;
+  if (!nbytes || nbytes > ROCSHMEM_AMD_STAGED_MAX_BYTES) return -1;
+  if (!sym_ok_on(dest, nbytes, my_pe) || !local_ok(source, nbytes) || !local_ok(back, nbytes))
+    return -1;
+  StagedArgs a;
+  a.dest = static_cast<char *>(dest);
+  a.source = static_cast<const char *>(source);
+  a.back = static_cast<char *>(back);
+  a.nbytes = nbytes;
+  a.ctx = runtime::rt().driver_ctx_handle(my_pe);
+  a.pe = pe;
+  a.gran = gran;
+  const size_t lds = 2 * ((nbytes + 15) & ~size_t{15}) + 16;
+  hipLaunchKernelGGL(staged_kernel, dim3(1), dim3(wg_size), lds, as_stream(stream), a);
+  DRV_CHECK_HIP(hipGetLastError());
+  return 0;
+}
+
+int rocshmem_amd_flat_ids(int bx, int by, int bz, unsigned *out_host) {
+  if (!runtime::rt().live || !out_host || bx < 1 || by < 1 || bz < 1) return -1;
+  if (static_cast<long>(bx) * by * bz > 1024 || bz > 64) return -1;
+  unsigned *d;
+  const size_t bytes = 1026 * sizeof(unsigned);
+  DRV_CHECK_HIP(hipMalloc(&d, bytes));
+  DRV_CHECK_HIP(hipMemset(d, 0, bytes));
+  hipLaunchKernelGGL(flat_ids_kernel, dim3(1), dim3(bx, by, bz), 0, 0, d);
+  DRV_CHECK_HIP(hipGetLastError());
+  DRV_CHECK_HIP(hipMemcpy(out_host, d, bytes, hipMemcpyDeviceToHost));
+  DRV_CHECK_HIP(hipFree(d));
   return 0;
 }
 

@@ -396,17 +396,24 @@ int Runtime::init(int want_npes, size_t want_heap) {
                          hipMemcpyHostToDevice));
 
   RT_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&d_ctx_slots),
-                         sizeof(detail::Context) * max_ctxs * npes));
+                         sizeof(detail::Context) * 2 * max_ctxs * npes));
   RT_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&d_pools), sizeof(detail::CtxPool) * npes));
-  std::vector<detail::Context> slots(static_cast<size_t>(max_ctxs) * npes);
+  // Two objects per pool slot: [0, max_ctxs) without an option, [max_ctxs,
+  // 2 * max_ctxs) with ROCSHMEM_CTX_NOSTORE; kernels only read them.
+  std::vector<detail::Context> slots(static_cast<size_t>(max_ctxs) * 2 * npes);
   std::vector<detail::CtxPool> pools(npes);
   for (int pe = 0; pe < npes; ++pe) {
-    for (int s = 0; s < max_ctxs; ++s) fill_ctx(slots[static_cast<size_t>(pe) * max_ctxs + s], pe, s);
+    detail::Context *row = slots.data() + static_cast<size_t>(pe) * 2 * max_ctxs;
+    for (int s = 0; s < max_ctxs; ++s) {
+      fill_ctx(row[s], pe, s);
+      fill_ctx(row[max_ctxs + s], pe, s);
+      row[max_ctxs + s].options = static_cast<unsigned>(ROCSHMEM_CTX_NOSTORE);
+    }
     detail::CtxPool &p = pools[pe];
     memset(&p, 0, sizeof(p));
     for (int s = 0; s < max_ctxs; ++s) p.free_mask[s >> 6] |= 1ull << (s & 63);
     p.capacity = max_ctxs;
-    p.slots = d_ctx_slots + static_cast<size_t>(pe) * max_ctxs;
+    p.slots = d_ctx_slots + static_cast<size_t>(pe) * 2 * max_ctxs;
   }
   RT_CHECK_HIP(hipMemcpy(d_ctx_slots, slots.data(), sizeof(detail::Context) * slots.size(),
                          hipMemcpyHostToDevice));

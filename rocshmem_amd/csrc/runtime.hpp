@@ -35,7 +35,7 @@ struct Runtime {
   char *d_ws = nullptr;
   detail::Team *d_teams = nullptr;         // [max_teams][npes]
   detail::Context *d_default_ctx = nullptr;  // [2*npes]: default, then NOSTORE
-  detail::Context *d_ctx_slots = nullptr;  // [npes][max_ctxs]
+  detail::Context *d_ctx_slots = nullptr;  // [npes][2 * max_ctxs]: per slot one object per ordering option
   detail::CtxPool *d_pools = nullptr;      // [npes]
   detail::QueueBinding *d_queue_table = nullptr;  // [kQueueTableSize]
   int *h_bind_problem = nullptr;  // pinned, [kQueueTableSize]: what each stream binding reported

@@ -76,6 +76,8 @@ SIGNATURES = {
     "rocshmem_amd_timer_elapsed_ms": (C.c_float, [_vp]),
     "rocshmem_amd_timer_destroy": (_i, [_vp]),
     "rocshmem_amd_rma": (_i, [_i, _i, _vp, _vp, _sz, _sz, _i, _i, _i, _i, _i, _vp]),
+    "rocshmem_amd_rma_staged": (_i, [_i, _vp, _vp, _vp, _sz, _i, _i, _i, _vp]),
+    "rocshmem_amd_flat_ids": (_i, [_i, _i, _i, _vp]),
     "rocshmem_amd_ctx_pe": (_i, [_vp]),
     "rocshmem_amd_host_putmem": (_i, [_vp, _vp, _sz, _i, _i]),
     "rocshmem_amd_host_getmem": (_i, [_vp, _vp, _sz, _i, _i]),

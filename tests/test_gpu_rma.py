@@ -252,3 +252,49 @@ def test_argument_errors_launch_nothing(rt, L, env):
     assert l.rma(L.PUT, L.WG, l.pe_ptr(dst, 1), src, 16, 0, 0, 1, 1, 64, 1, None) == -1  # not my_pe's address
     assert l.putmem(dst, src, HEAP, 0, 1, None) == -1
     assert l.rma(7, L.WG, dst, src, 16, 0, 0, 1, 1, 64, 1, None) == -1
+
+
+@pytest.mark.parametrize("ctx_options", [0, 1])
+@pytest.mark.parametrize("gran_name,wg_size", [("WG", 256), ("WG", 1024), ("WG", 192), ("WAVE", 128),
+                                               ("THREAD", 64)])
+@pytest.mark.parametrize("n", [1, 15, 16, 17, 4096, 4099, 24576])
+def test_local_buffer_in_lds(rt, L, orc, env, gran_name, wg_size, n, ctx_options):
+    """The local side of a put and of a get may be a __shared__ array, as with
+    the reference's generic-pointer copy (src/util.hpp:170-262): put from LDS,
+    get back into LDS at an odd offset, both byte-exact."""
+    l = env["l"]
+    src, dst, host = env["src"], env["dst"], env["host"]
+    my_pe, pe, soff, doff = 2, 5, 5, GUARD + 3
+    rt.put_bytes(l.pe_ptr(src, my_pe), host[:soff + n])
+    landing = l.pe_ptr(dst, pe) + doff
+    l.fill(landing - GUARD, 0xA5, n + 2 * GUARD)
+    back = l.dev_alloc(n)
+    l.fill(back, 0x5A, n)
+    before = l.set_ctx_options(ctx_options)
+    rc = l.rma_staged(getattr(L, gran_name), l.pe_ptr(dst, my_pe) + doff, l.pe_ptr(src, my_pe) + soff,
+                      back, n, my_pe, pe, wg_size, None)
+    l.set_ctx_options(before)
+    assert rc == 0
+    l.stream_sync(None)
+    want = np.full(n + 2 * GUARD, 0xA5, np.uint8)
+    exp = np.empty(n, np.uint8)
+    orc.lib.orc_copy(exp.ctypes.data, host[soff:soff + n].ctypes.data, n)
+    want[GUARD:GUARD + n] = exp
+    assert np.array_equal(rt.get_bytes(landing - GUARD, n + 2 * GUARD), want)
+    assert np.array_equal(rt.get_bytes(back, n), exp)
+    l.dev_free(back)
+    assert l.rma_staged(L.WG, l.pe_ptr(dst, my_pe), l.pe_ptr(src, my_pe), back, 24577, my_pe, pe, 256,
+                        None) == -1
+
+
+@pytest.mark.parametrize("shape", [(64, 1, 1), (256, 1, 1), (1024, 1, 1), (32, 8, 1), (16, 4, 4),
+                                   (7, 5, 3), (1, 1, 64), (3, 1, 1), (1, 1000, 1)])
+def test_work_group_rank_and_size_for_any_block_shape(env, shape):
+    """Every thread of a 1-, 2- or 3-D block gets a distinct rank
+    x + y*X + z*X*Y below X*Y*Z (src/util.hpp:100-118)."""
+    l = env["l"]
+    out = np.zeros(1026, np.uint32)
+    assert l.flat_ids(shape[0], shape[1], shape[2], out.ctypes.data) == 0
+    n = shape[0] * shape[1] * shape[2]
+    assert out[0] == n
+    assert (out[1:1 + n] == 1).all() and (out[1 + n:] == 0).all()
