@@ -189,20 +189,29 @@ __device__ __forceinline__ void fold_window(
   const size_t vlo = lo + head;
   const size_t nvec = (hi - vlo) / V;
   const size_t step = nparts * nlanes;
-  auto load_vec = [&](int p, size_t i) -> r_u32x4 {
-    if constexpr (kNonTemporal)
-      return __builtin_nontemporal_load(reinterpret_cast<const r_u32x4_any *>(src_at(p, i)));
-    else
-      return *reinterpret_cast<const r_u32x4_any *>(src_at(p, i));
+  // Vector v of the window sits 16 * v bytes after element vlo in every source
+  // and destination.  Each source is a global-memory base in scalar registers
+  // plus that one 32-bit offset, each destination a buffer resource built once.
+  const char *const first_src = reinterpret_cast<const char *>(src0 + vlo);
+  char *const first_dst = reinterpret_cast<char *>(dst0 + vlo);
+  const size_t vec_bytes = nvec << 4;
+  auto load_vec = [&](GlobalBytes base, uint32_t off) -> r_u32x4 {
+    return load16<kNonTemporal>(base, off);
   };
 
-  for (size_t v = part * nlanes + lane; v < nvec; v += step) {
-    const size_t i = vlo + v * V;
-    Pack<S> out;
-    if constexpr (kP != 0) {
-      Pack<S> in[kP ? kP : 1];
+  if constexpr (kP != 0) {
+    GlobalBytes from[kP];
+    __amdgpu_buffer_rsrc_t to[kP];
 #pragma unroll
-      for (int p = 0; p < kP; ++p) in[p].raw = load_vec(p, i);
+    for (int p = 0; p < kP; ++p) {
+      from[p] = wave_uniform_global(first_src + p * hop);
+      to[p] = window_of(first_dst + p * hop, vec_bytes);
+    }
+    for (size_t v = part * nlanes + lane; v < nvec; v += step) {
+      const uint32_t off = static_cast<uint32_t>(v << 4);
+      Pack<S> in[kP], out;
+#pragma unroll
+      for (int p = 0; p < kP; ++p) in[p].raw = load_vec(from[p], off);
 #pragma unroll
       for (int e = 0; e < V; ++e) {
         A acc = Tr::widen(in[0].e[e]);
@@ -210,26 +219,26 @@ __device__ __forceinline__ void fold_window(
         for (int p = 1; p < kP; ++p) acc = combine<A, Op>(acc, Tr::widen(in[p].e[e]));
         out.e[e] = Tr::narrow(acc);
       }
-    } else {
+#pragma unroll
+      for (int p = 0; p < kP; ++p) store16<kNonTemporal>(to[p], off, out.raw);
+    }
+  } else {
+    for (size_t v = part * nlanes + lane; v < nvec; v += step) {
+      const uint32_t off = static_cast<uint32_t>(v << 4);
       A acc[V];
-      Pack<S> in;
-      in.raw = load_vec(0, i);
+      Pack<S> in, out;
+      in.raw = load_vec(wave_uniform_global(first_src), off);
 #pragma unroll
       for (int e = 0; e < V; ++e) acc[e] = Tr::widen(in.e[e]);
       for (int p = 1; p < P; ++p) {
-        in.raw = load_vec(p, i);
+        in.raw = load_vec(wave_uniform_global(first_src + p * hop), off);
 #pragma unroll
         for (int e = 0; e < V; ++e) acc[e] = combine<A, Op>(acc[e], Tr::widen(in.e[e]));
       }
 #pragma unroll
       for (int e = 0; e < V; ++e) out.e[e] = Tr::narrow(acc[e]);
-    }
-    const uint32_t off = static_cast<uint32_t>((i - lo) * sizeof(S));
-    if constexpr (kP != 0) {
-#pragma unroll
-      for (int p = 0; p < kP; ++p) store16<kNonTemporal>(dst_window(p), off, out.raw);
-    } else {
-      for (int p = 0; p < P; ++p) store16<kNonTemporal>(dst_window(p), off, out.raw);
+      for (int p = 0; p < P; ++p)
+        store16<kNonTemporal>(window_of(first_dst + p * hop, vec_bytes), off, out.raw);
     }
   }
 

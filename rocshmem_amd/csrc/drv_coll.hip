@@ -246,19 +246,27 @@ void launch_grid_reduce(void *dst0, const void *src0, int64_t hop, int np, size_
   a.hop = hop;
   a.np = np;
   a.n = n;
-  // Shape from a sweep on MI355X (P = 8, fp32, 64 Mi elements): one 16-byte
-  // vector per lane, 128 lanes, one span per work-group, non-temporal loads and
-  // stores: 5.8 TB/s; 256 lanes x 4 vectors on a 2048-group grid gave 5.4.
-  const int wg = 128;
+  // Shape from sweeps on MI355X (P = 8, fp32, 64 Mi elements): one wavefront
+  // per work-group, one 16-byte vector per lane and source, non-temporal loads
+  // and stores.  A wavefront then has P KiB of loads in flight, and the rate
+  // peaks when a CU holds about 48 KiB of them: 6 wavefronts per CU for P = 8
+  // give 6.58 TB/s, 8 give 6.54, 16 or the full 32 give 6.46, 4 give 6.35.  The
+  // residency is set by asking for LDS the kernel never touches.
+  const int wg = 64;
+  size_t lds = 0;
+  if (np == 2 || np == 4 || np == 8) {
+    const size_t waves_per_cu = (48 * 1024) / (static_cast<size_t>(np) * 1024);
+    if (waves_per_cu < 32) lds = (160 * 1024) / waves_per_cu - 512;
+  }
   a.span = static_cast<size_t>(wg) * (16 / sizeof(S));
   const size_t nspans = (n + a.span - 1) / a.span;
   const size_t max_wgs = size_t{1} << 20;
   const int grid = static_cast<int>(nspans < max_wgs ? (nspans ? nspans : 1) : max_wgs);
   const bool nt = n * sizeof(S) >= runtime::rt().state.nt_bytes;
   if (nt)
-    hipLaunchKernelGGL((grid_reduce_kernel<E, Op, true>), dim3(grid), dim3(wg), 0, stream, a);
+    hipLaunchKernelGGL((grid_reduce_kernel<E, Op, true>), dim3(grid), dim3(wg), lds, stream, a);
   else
-    hipLaunchKernelGGL((grid_reduce_kernel<E, Op, false>), dim3(grid), dim3(wg), 0, stream, a);
+    hipLaunchKernelGGL((grid_reduce_kernel<E, Op, false>), dim3(grid), dim3(wg), lds, stream, a);
   DRV_CHECK_HIP(hipGetLastError());
 }
 
@@ -284,7 +292,7 @@ __global__ void grid_alltoall_kernel(GridMoveArgs a) {
   const char *src = a.src0 + i * a.hop + static_cast<size_t>(j) * a.nbytes;
   for (size_t off = blockIdx.x * a.span; off < a.nbytes; off += gridDim.x * a.span) {
     const size_t len = a.nbytes - off < a.span ? a.nbytes - off : a.span;
-    detail::copy_lanes_impl<2, kNonTemporal>(d + off, src + off, len, threadIdx.x, blockDim.x);
+    detail::copy_lanes_impl<1, kNonTemporal>(d + off, src + off, len, threadIdx.x, blockDim.x);
   }
 }
 

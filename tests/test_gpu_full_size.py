@@ -58,10 +58,13 @@ def test_dispatch_put_signal_full_size(rt, L, orc, ctx_kind):
     assert l.fill_every_pe(sig, 0, 8 * P, None) == 0
     tabs = [np.ascontiguousarray(a, np.uint32) for a in (counts, send_row, recv_row)]
     before = l.set_ctx_options(ctx_kind)
+    # (rows per call, work-group size): the shape bench.py times, and a second one
+    rows_per_call, wg_size = (8, 1024) if ctx_kind else (16, 256)
     try:
         for _ in range(2):
             assert l.dispatch_put_signal(recv, send, sig, tabs[0].ctypes.data, tabs[1].ctypes.data,
-                                         tabs[2].ctypes.data, row, 16, 256, expect, None) == 0
+                                         tabs[2].ctypes.data, row, rows_per_call, wg_size, expect,
+                                         None) == 0
         l.stream_sync(None)
     finally:
         l.set_ctx_options(max(before, 0))
