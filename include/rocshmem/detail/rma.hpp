@@ -67,10 +67,15 @@ __device__ __forceinline__ void getmem_nbi(Context *c, void *dest, const void *s
 }
 
 // ---- wavefront granularity (context_ipc_device.cpp:137-164) ---------------
+// The ordering option is looked at before the copy although it is only needed
+// after it: the context's hot fields share one scalar load, and a call then
+// waits for the scalar data path once, not once per field (a scalar load that
+// hits costs about 100 ns, which a small message feels).
 __device__ __forceinline__ void putmem_wave(Context *c, void *dest, const void *source,
                                             size_t n, int pe) {
+  const bool relaxed = no_store_order(c);
   copy_wave(remote_addr(c, static_cast<char *>(dest), pe), source, n, g_state.nt_bytes);
-  if (no_store_order(c)) drain_own_stores();
+  if (relaxed) drain_own_stores();
   else fence_full();
 }
 __device__ __forceinline__ void getmem_wave(Context *c, void *dest, const void *source,
@@ -93,11 +98,12 @@ __device__ __forceinline__ void getmem_nbi_wave(Context *c, void *dest, const vo
 // ---- work-group granularity: copy, then __syncthreads (:109-125) ----------
 __device__ __forceinline__ void putmem_wg(Context *c, void *dest, const void *source,
                                           size_t n, int pe) {
+  const bool relaxed = no_store_order(c);
   copy_lanes(remote_addr(c, static_cast<char *>(dest), pe), source, n,
              flat_thread_id(), flat_block_size(), g_state.nt_bytes);
   // Each wavefront completes its own share, so that after the barrier a quiet
   // by any one thread covers the whole work-group's put.
-  if (no_store_order(c)) drain_own_stores();
+  if (relaxed) drain_own_stores();
   __syncthreads();
 }
 __device__ __forceinline__ void getmem_wg(Context *c, void *dest, const void *source,

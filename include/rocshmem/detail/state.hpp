@@ -96,15 +96,17 @@ struct Team {
 // a context: the host fills them all in at initialisation, so device code
 // reads them through the scalar data path (see ctx_view).
 struct Context {
-  char *heap_base;      // base of PE 0's slice
+  // What every put, get and atomic reads, side by side: one 16-byte scalar
+  // load brings all three.
   uint64_t pe_stride;   // bytes between consecutive slices
-  uint64_t ws_stride;   // bytes between consecutive PEs' work/sync areas
   int my_pe;
+  unsigned options;     // ROCSHMEM_CTX_* bits, fixed per object
+  char *heap_base;      // base of PE 0's slice
+  uint64_t ws_stride;   // bytes between consecutive PEs' work/sync areas
   int num_pes;
+  int pool_slot;        // index in the context pool, -1 for default contexts
   TeamInfo *tinfo;      // world team of this PE
   SyncPad *world_sync;  // this PE's pad for barrier_all / sync_all
-  unsigned options;     // ROCSHMEM_CTX_* bits, fixed per object
-  int pool_slot;        // index in the context pool, -1 for default contexts
 };
 
 // Pool of pre-built contexts for one PE.  A set bit in free_mask marks a free
