@@ -298,3 +298,21 @@ def test_work_group_rank_and_size_for_any_block_shape(env, shape):
     n = shape[0] * shape[1] * shape[2]
     assert out[0] == n
     assert (out[1:1 + n] == 1).all() and (out[1 + n:] == 0).all()
+
+
+@pytest.mark.parametrize("lanes,gran_name", [(64, "WG"), (192, "WG"), (256, "WG"), (1024, "WG"),
+                                             (64, "WAVE"), (37, "WAVE")])
+def test_sizes_around_the_burst_boundaries(rt, L, orc, env, lanes, gran_name):
+    """A lane moves bursts of eight 16-byte vectors: message sizes either side
+    of 1, 7, 8, 9 and 16 vectors per lane, of the 64-byte single-wavefront
+    path and of the non-temporal threshold, with misaligned ends."""
+    g = getattr(L, gran_name)
+    per = lanes * 16
+    sizes = set()
+    for k in (1, 7, 8, 9, 16):
+        for d in (-17, -16, -1, 0, 1, 16, 33):
+            sizes.add(k * per + d)
+    sizes.update((63, 64, 65, 4095, 4096, 4097))
+    for i, n in enumerate(sorted(s for s in sizes if 0 < s <= (4 << 20))):
+        run_case(rt, L, orc, env, L.PUT, g, n, i % 16, (3 * i) % 16, 1, lanes, ctx_options=i & 1)
+        run_case(rt, L, orc, env, L.GET, g, n, (5 * i) % 16, i % 16, 1, lanes)
