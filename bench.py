@@ -6,7 +6,7 @@
 Prints ONE JSON line.  The headline (`metric`/`value`) is the bulk putmem
 workload of BASELINE.json's configs[1]: one 256 MiB message between two of
 P=8 PE slices of one symmetric heap, moved by all CUs through the device API
-(rocshmem_ctx_putmem_wg, one 16 KiB tile per work-group of 256, on a context
+(rocshmem_ctx_putmem_wg, one 4 KiB tile per work-group of 128, on a context
 created with ROCSHMEM_CTX_NOSTORE); a step is one such message and `value`
 counts algorithmic bytes (N read + N written).  The same workload through a
 default context and through the host-side rocshmem_putmem, and every other
@@ -31,7 +31,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0  # MI355X, published
 # HBM bytes one launch of the headline kernel moves, from FETCH_SIZE + WRITE_SIZE
 # under rocprofv3 --pmc (profiles/putmem_wg_tiled_256MiB_hbm_traffic.txt).
-PUT_TRAFFIC_BYTES = 536948703
+PUT_TRAFFIC_BYTES = 536932764
 P = 8
 MiB = 1 << 20
 
@@ -647,7 +647,8 @@ def main():
         "data": "synthetic",
         "config": {"workload": "bulk putmem through the device API: one 256 MiB message per step from PE "
                                "k%8 to PE (k+1)%8 of P=8 slices in one symmetric heap, every CU calling "
-                               "rocshmem_ctx_putmem_wg on 16 KiB tiles (one tile per work-group of 256) "
+                               "rocshmem_ctx_putmem_wg on " + "%d-byte tiles (one tile per work-group of %d) " % (
+                                   PUT_SHAPES["nostore_ctx"][1], PUT_SHAPES["nostore_ctx"][0]) +
                                "through a ROCSHMEM_CTX_NOSTORE context, one quiet per work-group "
                                "(BASELINE configs[1], largest size; buffers rotate so no step re-reads "
                                "cached data)",
