@@ -246,16 +246,17 @@ void launch_grid_reduce(void *dst0, const void *src0, int64_t hop, int np, size_
   a.hop = hop;
   a.np = np;
   a.n = n;
-  // Shape from sweeps on MI355X (P = 8, fp32, 64 Mi elements): one wavefront
-  // per work-group, one 16-byte vector per lane and source, non-temporal loads
-  // and stores.  A wavefront then has P KiB of loads in flight, and the rate
-  // peaks when a CU holds about 48 KiB of them: 6 wavefronts per CU for P = 8
-  // give 6.58 TB/s, 8 give 6.54, 16 or the full 32 give 6.46, 4 give 6.35.  The
-  // residency is set by asking for LDS the kernel never touches.
+  // Shape from sweeps on MI355X (P = 8, 64 Mi elements): one wavefront per
+  // work-group, one 16-byte vector per lane and source, non-temporal loads and
+  // stores.  A wavefront then has P KiB of loads in flight, and the rate peaks
+  // when a CU holds 48-64 KiB of them: for P = 8, 6 or 8 wavefronts per CU give
+  // 6.55 TB/s (fp32, bf16 and int64 alike), 12 give 6.51, 16 or the full 32
+  // 6.46-6.49, and 5 only 6.25 - so 8, the side of the optimum away from the
+  // drop.  The residency is set by asking for LDS the kernel never touches.
   const int wg = 64;
   size_t lds = 0;
   if (np == 2 || np == 4 || np == 8) {
-    const size_t waves_per_cu = (48 * 1024) / (static_cast<size_t>(np) * 1024);
+    const size_t waves_per_cu = (64 * 1024) / (static_cast<size_t>(np) * 1024);
     if (waves_per_cu < 32) lds = (160 * 1024) / waves_per_cu - 512;
   }
   a.span = static_cast<size_t>(wg) * (16 / sizeof(S));
