@@ -72,3 +72,30 @@ def test_reference_examples_compile_unchanged(example, tmp_path):
     r = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
     assert r.returncode == 0, r.stderr[-3000:]
     assert out.exists()
+
+
+@pytest.mark.skipif(not os.path.isdir(REFERENCE) or not shutil.which("hipcc"),
+                    reason="needs the reference tree and hipcc (build container only)")
+def test_every_function_name_of_the_reference_headers_is_declared(tmp_path):
+    """Every rocshmem_* function the reference's public headers declare
+    (include/rocshmem/*.hpp, over a thousand once the type tables are stamped
+    out) exists under the same name in these headers: the preprocessed device
+    pass of <rocshmem/rocshmem.hpp> is searched for each of them."""
+    def function_names(text):
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        text = re.sub(r"//.*", "", text)
+        return set(re.findall(r"\b(rocshmem_\w+)\s*\(", text))
+
+    wanted = set()
+    for path in glob.glob(os.path.join(REFERENCE, "include", "rocshmem", "*.hpp")):
+        wanted |= function_names(open(path, errors="ignore").read())
+    assert len(wanted) > 1000
+    src = tmp_path / "api.hip"
+    src.write_text("#include <rocshmem/rocshmem.hpp>\n")
+    out = tmp_path / "api.i"
+    cmd = ["hipcc", "--offload-arch=gfx950", "-std=c++17", "-DROCSHMEM_AMD_NO_MPI_HEADER", "-I",
+           os.path.join(ROOT, "include"), "-E", "--cuda-device-only", str(src), "-o", str(out)]
+    r = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-3000:]
+    have = function_names(out.read_text(errors="ignore"))
+    assert not sorted(wanted - have), sorted(wanted - have)[:40]
