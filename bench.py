@@ -304,7 +304,7 @@ def zipf_table(K, s):
     return np.cumsum(w / w.sum())
 
 
-def dispatch_config(b, steps, shapes=((8, 1024),)):
+def dispatch_config(b, steps, shapes=((7, 1024),)):
     """configs[4] part 2: put_signal dispatch, 4096 tokens/PE, top-8 of 256
     experts by Zipf(1.1), rows of 7168 bf16.  shapes: (rows per
     putmem_signal_wg call, work-group size)."""

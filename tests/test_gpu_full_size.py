@@ -59,7 +59,7 @@ def test_dispatch_put_signal_full_size(rt, L, orc, ctx_kind):
     tabs = [np.ascontiguousarray(a, np.uint32) for a in (counts, send_row, recv_row)]
     before = l.set_ctx_options(ctx_kind)
     # (rows per call, work-group size): the shape bench.py times, and a second one
-    rows_per_call, wg_size = (8, 1024) if ctx_kind else (16, 256)
+    rows_per_call, wg_size = (7, 1024) if ctx_kind else (16, 256)
     try:
         for _ in range(2):
             assert l.dispatch_put_signal(recv, send, sig, tabs[0].ctypes.data, tabs[1].ctypes.data,
