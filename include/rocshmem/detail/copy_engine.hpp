@@ -137,9 +137,9 @@ __device__ __forceinline__ void copy_window(char *dst, const char *src_any, size
   const __amdgpu_buffer_rsrc_t w = window_of(dst, n);
   if (n <= 64 && n <= nlanes) {
     // A byte per lane of the first wavefront (flags, counters, small control
-    // messages): no peeling and no loops.  A lone wavefront issues an instruction every few
-    // cycles, so what a small message pays for beyond its one load and one
-    // store is the number of instructions on its path.
+    // messages): no peeling and no loops.  A lone wavefront issues an
+    // instruction every few cycles, so what a small message pays for beyond
+    // its one load and one store is the number of instructions on its path.
     if (lane < n) store1(w, static_cast<uint32_t>(lane), wave_uniform_global(src_any)[lane]);
     return;
   }
