@@ -31,7 +31,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0  # MI355X, published
 # HBM bytes one launch of the headline kernel moves, from FETCH_SIZE + WRITE_SIZE
 # under rocprofv3 --pmc (profiles/putmem_wg_tiled_256MiB_hbm_traffic.txt).
-PUT_TRAFFIC_BYTES = 536951062
+PUT_TRAFFIC_BYTES = 536951306
 P = 8
 MiB = 1 << 20
 
