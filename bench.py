@@ -11,8 +11,19 @@ created with ROCSHMEM_CTX_NOSTORE); a step is one such message and `value`
 counts algorithmic bytes (N read + N written).  The same workload through a
 default context and through the host-side rocshmem_putmem, and every other
 configuration (all-reduce, alltoall, put_signal dispatch, atomics, ping-pong),
-are carried as scalar keys of `roofline` (and in full under `all_configs`),
-beside a CPU baseline (the oracle's threaded routines on the host cores).
+are carried as scalar keys of `roofline` — one figure per configuration first,
+then the same in the packed default layout and on a cached heap, then the rest
+— and in full under `all_configs`, beside a CPU baseline (the oracle's
+threaded routines on the host cores).  After the timed loops the last
+destination of the headline put is compared with its source on the device
+(`roofline.verified`).
+
+The run has three bring-ups of the library: slices spread over half of the
+device memory (ROCSHMEM_EMU_SPREAD=1, 8 GiB per PE: every configuration), the
+default packed layout (1 GiB per PE: the layout a plain rocshmem_init gives),
+and a cached heap (ROCSHMEM_EMU_HEAP_CACHED=1: what a consumer that re-reads
+symmetric data gains, and what ordering then costs).  The CPU baseline's legs
+run between them.
 
 Inputs are resident in HBM before any timed region starts.
 """
@@ -62,6 +73,7 @@ class Bench:
     def __init__(self, L):
         self.L = L
         self.l = L.load()
+        self.probes = L.load_probes()
         self.timer = self.l.timer_create()
 
     def time_ms(self, fn, steps, warmup):
@@ -141,6 +153,18 @@ def headline(b, steps, warmup):
                                              1, None))
 
     out = {"bytes_per_step": 2 * n}
+
+    def moves_every_byte(step):
+        """What a timed loop moved: every destination is cleared, one more step
+        runs, and its destination is compared with its source on the device."""
+        for p in range(P):
+            l.fill(dsts[p], 0, n)
+        step()
+        me = (k[0] - 1) % P
+        bad = C.c_uint64(1)
+        assert l.compare(dsts[(me + 1) % P], srcs[me], n, C.byref(bad), None) == 0
+        return bad.value == 0
+
     # The host-side rocshmem_putmem / getmem (one whole-GPU kernel per message).
     # Measured first: whatever runs first in the process comes out about 3 %
     # low (the GPU's first milliseconds of work run below its sustained rate,
@@ -155,8 +179,10 @@ def headline(b, steps, warmup):
     l.set_ctx_options(1)
     out["ms"] = b.time_ms(tiled_put("nostore_ctx"), steps, warmup)
     out["gbs"] = 2 * n / out["ms"] / 1e6
+    out["verified"] = moves_every_byte(tiled_put("nostore_ctx"))
     l.set_ctx_options(0)
     out["default_ctx_gbs"] = 2 * n / b.time_ms(tiled_put("default_ctx"), steps, warmup) / 1e6
+    out["verified"] = moves_every_byte(tiled_put("default_ctx")) and out["verified"]
     # rocshmem_ctx_getmem_wg from every CU, the shape of the headline put
     l.set_ctx_options(1)
     wg, tile, _ = PUT_SHAPES["nostore_ctx"]
@@ -164,7 +190,7 @@ def headline(b, steps, warmup):
         rotating(lambda me, pe: l.rma(L.GET, L.WG, dsts[me], srcs[me], n, tile, me, pe, n // tile, wg, 1,
                                       None)), steps, warmup) / 1e6
     l.set_ctx_options(0)
-    if b.quick:
+    if b.quick or b.short:
         l.free(src)
         l.free(dst)
         return out
@@ -194,8 +220,8 @@ def headline(b, steps, warmup):
     out["curve"] = curve
     # One-directional ceilings of the memory system, same buffers and rotation:
     # a copy that reads N and writes N cannot beat 2 / (1/read + 1/write).
-    t_rd = b.time_ms(rotating(lambda me, pe: l.hbm_probe(0, srcs[me], n, None)), steps, warmup)
-    t_wr = b.time_ms(rotating(lambda me, pe: l.hbm_probe(1, dsts[pe], n, None)), steps, warmup)
+    t_rd = b.time_ms(rotating(lambda me, pe: b.probes.hbm_probe(0, srcs[me], n, None)), steps, warmup)
+    t_wr = b.time_ms(rotating(lambda me, pe: b.probes.hbm_probe(1, dsts[pe], n, None)), steps, warmup)
     rd, wr = n / t_rd / 1e6, n / t_wr / 1e6
     out["ceilings"] = {"read_only_gbs": round(rd, 1), "write_only_gbs": round(wr, 1),
                        "copy_bound_gbs": round(2 / (1 / rd + 1 / wr), 1)}
@@ -203,7 +229,7 @@ def headline(b, steps, warmup):
     # costs while the copy runs: 1024 work-groups of 256, 16 KiB tiles.
     rp = {}
     for mode in (0, 1, 2):
-        rp[mode] = b.time_ms(rotating(lambda me, pe: l.release_probe(mode, dsts[pe], srcs[me], n, 16384,
+        rp[mode] = b.time_ms(rotating(lambda me, pe: b.probes.release_probe(mode, dsts[pe], srcs[me], n, 16384,
                                                                      1024, 256, None)), 5, 2)
     out["release_ns_each_per_tile"] = round((rp[2] - rp[0]) * 1e6 / (n // 16384), 1)
     out["release_ns_each_at_end"] = round((rp[1] - rp[0]) * 1e6 / 1024, 1)
@@ -223,14 +249,23 @@ def headline(b, steps, warmup):
     return out
 
 
-def to_all_configs(b, steps, warmup):
-    """configs[2]: all-reduce over P=8 slices x 64 Mi elements."""
+# Launch shape of the many-teams device all-reduce (teams, lanes per work-group,
+# elements per call; 0 = one contiguous slice per team), from sweeps on MI355X.
+TEAM_SHAPE = (32, 256, 0)
+
+
+def to_all_configs(b, steps, warmup, which=("int64_xor", "fp32_sum", "fp32_max", "bf16_sum"), device_api=True):
+    """configs[2]: all-reduce over P=8 slices x 64 Mi elements; and configs[0],
+    the int32 sum over P=2 x 1 Mi, as the same host call on an active set of
+    two PEs."""
     l, L = b.l, b.L
     n = 1 << 26
     res = {}
+    table = {"int64_xor": (L.LONG, L.XOR, 8), "fp32_sum": (L.FLOAT, L.SUM, 4),
+             "fp32_max": (L.FLOAT, L.MAX, 4), "bf16_sum": (L.BF16, L.SUM, 2)}
     # largest buffers first: freed blocks are never merged by the allocator
-    for name, dt, op, es in (("int64_xor", L.LONG, L.XOR, 8), ("fp32_sum", L.FLOAT, L.SUM, 4),
-                             ("fp32_max", L.FLOAT, L.MAX, 4), ("bf16_sum", L.BF16, L.SUM, 2)):
+    for name in which:
+        dt, op, es = table[name]
         src, dst = l.malloc(n * es), l.malloc(n * es)
         assert src and dst, name
         kind = {L.FLOAT: "f32", L.BF16: "bf16"}.get(dt, "u8")
@@ -240,16 +275,23 @@ def to_all_configs(b, steps, warmup):
         alg = 2 * P * n * es
         res[name] = {"ms": round(ms, 4), "gbs": round(alg / ms / 1e6, 1),
                      "frac": round(alg / ms / 1e6 / HBM_PEAK_GBS, 4)}
-        if name == "fp32_sum":
+        if name == "fp32_sum" and device_api:
+            # configs[0]: int32 sum, P=2 x 1 Mi elements (the reference's CPU-runnable
+            # case, src/rocshmem.cpp:974-980), through the same host call
+            m = 1 << 20
+            ms1 = b.time_ms(lambda: l.to_all(L.INT, L.SUM, dst, src, m, 0, 0, 2, None), 200, 20)
+            res["int32_sum_P2_1Mi"] = {"ms": round(ms1, 5), "gbs": round(2 * 2 * m * 4 / ms1 / 1e6, 1)}
             # The device call rocshmem_ctx_float_sum_wg_reduce: by its contract ONE
             # work-group per PE takes part, so 8 of the 256 CUs do all the work.
             ms = b.time_ms(lambda: l.wg_reduce(dt, op, l.team_world(), dst, src, n, 1024, None), 3, 1)
             res["fp32_sum_wg_reduce_one_wg_per_pe"] = {"ms": round(ms, 4),
                                                        "gbs": round(alg / ms / 1e6, 1)}
             # ... and the way the reference's testers scale it: one team per
-            # work-group, 32 teams x 8 PEs at once (one work-group of 256 per CU),
-            # the call repeated four times inside the kernel.
-            NT, inner = 32, 4
+            # work-group, many teams x 8 PEs at once, the call repeated four
+            # times inside the kernel.  Through the entry point that allocates
+            # nothing, so no hipMalloc sits inside the timed call.
+            NT, wg, chunk = TEAM_SHAPE
+            inner = 4
             teams = (C.c_void_p * NT)()
             for t in range(NT):
                 h = C.c_void_p()
@@ -257,16 +299,68 @@ def to_all_configs(b, steps, warmup):
                 teams[t] = h.value
             for cname, opt in CTX_KINDS:
                 l.set_ctx_options(opt)
-                ms = b.time_ms(lambda: l.wg_reduce_teams(dt, op, teams, NT, dst, src, n, 256, inner, None),
-                               3, 1) / inner
-                res["fp32_sum_wg_reduce_32_teams_" + cname] = {
+                ms = b.time_ms(lambda: l.wg_reduce_teams_static(dt, op, teams, NT, dst, src, n, chunk, wg,
+                                                                inner, None), 3, 1) / inner
+                res["fp32_sum_wg_reduce_teams_" + cname] = {
                     "ms": round(ms, 4), "gbs": round(alg / ms / 1e6, 1),
-                    "frac": round(alg / ms / 1e6 / HBM_PEAK_GBS, 4)}
+                    "frac": round(alg / ms / 1e6 / HBM_PEAK_GBS, 4), "teams": NT, "wg": wg,
+                    "chunk_elems": chunk}
             l.set_ctx_options(0)
             for t in range(NT):
                 l.team_destroy(teams[t])
         l.free(src)
         l.free(dst)
+    return res
+
+
+def message_rates(b, steps):
+    """Two thirds of the reference's test matrix is thread- and
+    wavefront-granularity traffic (scripts/functional_tests/driver.sh:142-218;
+    src/ipc/context_ipc_device.cpp:62-88,137-164): rocshmem_putmem of 8 B, 64 B
+    and 4 KiB per lane and rocshmem_putmem_wave of 512 B and 4 KiB per
+    wavefront from every CU, with lanes (wavefronts) that continue one another
+    and with their messages scattered, on both kinds of context."""
+    l, L = b.l, b.L
+    cap = 1 << 30
+    src, dst = l.malloc(cap), l.malloc(cap)
+    assert src and dst
+    b.fill_random(l.pe_ptr(src, 0), cap, 0, 77)
+    res = {}
+    for gran, gname, msg in ((L.THREAD, "putmem", 8), (L.THREAD, "putmem", 64), (L.THREAD, "putmem", 4096),
+                             (L.WAVE, "putmem_wave", 512), (L.WAVE, "putmem_wave", 4096)):
+        count = min(1 << 24, cap // msg)
+        groups_per_wg = 256 if gran == L.THREAD else 4
+        n_wgs = max(256, min(8192, count // groups_per_wg))
+        for scattered in (0, 1):
+            for cname, opt in CTX_KINDS:
+                l.set_ctx_options(opt)
+                ms = b.time_ms(lambda: l.rma_messages(L.PUT, gran, l.pe_ptr(dst, 0), l.pe_ptr(src, 0),
+                                                      count * msg, msg, scattered, 0, 1, n_wgs, 256, 1, None),
+                               max(3, steps // 10), 1)
+                key = "%s_%dB_%s_%s" % (gname, msg, "scattered" if scattered else "contiguous", cname)
+                res[key] = {"ms": round(ms, 4), "msgs": count, "mmsg_per_s": round(count / ms / 1e3, 1),
+                            "gbs": round(2 * count * msg / ms / 1e6, 1)}
+    l.set_ctx_options(0)
+    l.free(src)
+    l.free(dst)
+    return res
+
+
+def reuse_config(b, steps):
+    """What a consumer that re-reads symmetric data gets from the caches: a
+    256 MiB symmetric buffer read four times, tile by tile (256 KiB tiles, each
+    read four times in a row by its work-group), against one pass."""
+    l = b.l
+    n = 256 * MiB
+    buf = l.malloc(n)
+    assert buf
+    b.fill_random(buf, n, 0, 91)
+    res = {}
+    for passes in (1, 4):
+        ms = b.time_ms(lambda: b.probes.reuse_probe(buf, n, 256 << 10, passes, 1024, 256, None),
+                       max(5, steps // 4), 2)
+        res["read_x%d_gbs" % passes] = round(passes * n / ms / 1e6, 1)
+    l.free(buf)
     return res
 
 
@@ -452,13 +546,17 @@ def barrier_config(b):
     return res
 
 
-def cpu_baseline():
-    """The oracle's threaded routines on this host's cores, bounded samples of
-    the same workloads.  (The only place outside tests/ and smoke() that
-    touches oracle/.)"""
-    from oracle import pyoracle as orc
+# ---- CPU baseline: the oracle's threaded routines on this host's cores, bounded
+# samples of the same workloads.  (The only place outside tests/ and smoke()
+# that touches oracle/.)  Three legs, run between the GPU bring-ups.
+def cpu_threads(orc):
     # a one-GPU box gives a job 16 cores, whatever the machine has
-    threads = max(1, min(16, orc.lib.orc_hardware_threads()))
+    return max(1, min(16, orc.lib.orc_hardware_threads()))
+
+
+def cpu_copy_leg():
+    from oracle import pyoracle as orc
+    threads = cpu_threads(orc)
     # bulk copy: 256 MiB messages, as the headline
     n = 256 * MiB
     src = np.random.default_rng(0).integers(0, 256, n, dtype=np.uint8)
@@ -474,8 +572,23 @@ def cpu_baseline():
         k = reps % P
         orc.lib.orc_copy_threaded(dsts[(k + 1) % P].ctypes.data, srcs[k].ctypes.data, n, threads)
         reps += 1
-    copy_gbs = 2 * n * reps / (time.perf_counter() - t0) / 1e9
-    del srcs, dsts, src
+    return {"cores": threads, "putmem_256MiB_gbs": round(2 * n * reps / (time.perf_counter() - t0) / 1e9, 2)}
+
+
+def cpu_reduce_leg():
+    from oracle import pyoracle as orc
+    threads = cpu_threads(orc)
+    # configs[0] as BASELINE.json states it: int32 sum, P=2 x 1 Mi elements, values
+    # uniform in [-1000, 1000] from seed 0, both destinations written
+    rng = np.random.default_rng(0)
+    small = [rng.integers(-1000, 1001, 1 << 20, dtype=np.int32) for _ in range(2)]
+    orc.to_all(orc.INT, orc.SUM, small, ndst=2, nthreads=threads)
+    t0 = time.perf_counter()
+    reps = 0
+    while time.perf_counter() - t0 < 1.0:
+        orc.to_all(orc.INT, orc.SUM, small, ndst=2, nthreads=threads)
+        reps += 1
+    small_gbs = 2 * 2 * (1 << 20) * 4 * reps / (time.perf_counter() - t0) / 1e9
     # fp32 sum all-reduce at the GPU's size: P=8 x 64 Mi elements, result written to
     # all 8 destinations (4 GiB of host memory), at least two passes
     m = 1 << 26
@@ -488,7 +601,12 @@ def cpu_baseline():
         orc.to_all(orc.FLOAT, orc.SUM, srcs, ndst=P, nthreads=threads)
         reps += 1
     red_gbs = 2 * P * m * 4 * reps / (time.perf_counter() - t0) / 1e9
-    del srcs
+    return {"to_all_int32_P2_1Mi_gbs": round(small_gbs, 2), "to_all_fp32_sum_gbs": round(red_gbs, 2)}
+
+
+def cpu_amo_leg():
+    from oracle import pyoracle as orc
+    threads = cpu_threads(orc)
     # atomics at the GPU's size: 16 Mi seq_cst fetch_adds onto 4096 counters
     k = 1 << 24
     ids = np.random.default_rng(1).integers(0, 4096, k, dtype=np.uint32)
@@ -497,15 +615,21 @@ def cpu_baseline():
     sec = orc.lib.orc_amo_fetch_add_threaded(counters.ctypes.data, ids.ctypes.data, None,
                                              fetched.ctypes.data, k, threads)
     pp = orc.lib.orc_pingpong_threaded(8, 200000) / 200000 / 2 * 1e6
-    return {"value": round(copy_gbs, 2), "unit": "GB/s", "cores": threads, "kind": "port",
+    return {"amo_fetch_add_mops": round(k / sec / 1e6, 1), "pingpong_8B_us": round(pp, 3)}
+
+
+def cpu_baseline_record(legs):
+    return {"value": legs["putmem_256MiB_gbs"], "unit": "GB/s", "cores": legs["cores"], "kind": "port",
             "sample": "threaded memcpy of 256 MiB messages for 4 s, eight buffer pairs in turn "
-                      "(2N bytes per message); all-reduce: P=8 x 64 Mi fp32, ascending fold, all 8 "
-                      "destinations written, >= 2 passes; atomics: 16 Mi seq_cst fetch_add on 4096 "
-                      "counters, uniform; ping-pong: 200000 round trips of 8 B between two threads",
-            "putmem_256MiB_gbs": round(copy_gbs, 2),
-            "to_all_fp32_sum_gbs": round(red_gbs, 2),
-            "amo_fetch_add_mops": round(k / sec / 1e6, 1),
-            "pingpong_8B_us": round(pp, 3)}
+                      "(2N bytes per message); config 1: int32 sum P=2 x 1 Mi for 1 s; all-reduce: P=8 "
+                      "x 64 Mi fp32, ascending fold, all 8 destinations written, >= 2 passes; atomics: "
+                      "16 Mi seq_cst fetch_add on 4096 counters, uniform; ping-pong: 200000 round trips "
+                      "of 8 B between two threads",
+            "to_all_int32_P2_1Mi_gbs": legs["to_all_int32_P2_1Mi_gbs"],
+            "to_all_fp32_sum_gbs": legs["to_all_fp32_sum_gbs"],
+            "amo_fetch_add_mops": legs["amo_fetch_add_mops"],
+            "pingpong_8B_us": legs["pingpong_8B_us"],
+            "putmem_256MiB_gbs": legs["putmem_256MiB_gbs"]}
 
 
 def profile_kernels():
@@ -516,6 +640,7 @@ def profile_kernels():
     from rocshmem_amd import lib as L
     b = Bench(L)
     b.quick = True
+    b.short = False
     l = b.l
     assert l.init(P, 8 << 30) == 0
     disp = dispatch_config(b, 10)                      # 10 warm-up + 5 timed launches per context kind
@@ -542,6 +667,20 @@ def profile_kernels():
                       "alltoall_gbs": a2a["gbs"], "dispatch": disp}))
 
 
+def bring_up(L, heap_bytes, **env):
+    """rocshmem_init with the given layout / heap switches in the environment
+    (a value of None removes the variable)."""
+    for name, value in env.items():
+        if value is None:
+            os.environ.pop(name, None)
+        else:
+            os.environ[name] = value
+    l = L.load()
+    assert l.init(P, heap_bytes) == 0
+    return {"pe_stride_bytes": l.pe_stride(), "heap_alloc_bytes": l.heap_alloc_bytes(),
+            "heap_uncached": l.heap_is_uncached()}
+
+
 def main():
     a = parse()
     if a.profile_kernels:
@@ -551,20 +690,24 @@ def main():
         print("bench.py measures one GPU: every PE is a slice of one symmetric heap on a single "
               "MI355X; --gpus %d is not supported (use --gpus 1)." % a.gpus, file=sys.stderr)
         sys.exit(2)
-    # The slices spread over half of the device memory (16 GiB apart): kernels that
-    # write to all 8 slices at once sustain about 10 % more than with packed slices.
-    os.environ.setdefault("ROCSHMEM_EMU_SPREAD", "1")
-    os.environ.setdefault("ROCSHMEM_MAX_NUM_TEAMS", "40")
+    os.environ.setdefault("ROCSHMEM_MAX_NUM_TEAMS", "140")
     from rocshmem_amd import lib as L
     b = Bench(L)
     b.quick = a.quick
-    # 8 slices of 8 GiB: with Zipf(1.1) routing the busiest PE receives 2.3 GiB
-    # of rows, a 4 GiB block of the power-of-two allocator.  That request goes
-    # first because the allocator never merges freed blocks.
-    assert b.l.init(P, 8 << 30) == 0
-    layout = {"pe_stride_bytes": b.l.pe_stride(), "heap_alloc_bytes": b.l.heap_alloc_bytes()}
+    b.short = False
+    full = not a.quick
+    with_cpu = full and not a.no_cpu
+    legs = {}
     allc = {}
-    if not a.quick:
+
+    # ---- first bring-up: the slices spread over half of the device memory (16 GiB
+    # apart): kernels that write to all 8 slices at once sustain about 10 % more
+    # than with packed slices.  8 slices of 8 GiB: with Zipf(1.1) routing the
+    # busiest PE receives 2.3 GiB of rows, a 4 GiB block of the power-of-two
+    # allocator.  That request goes first because the allocator never merges
+    # freed blocks.
+    layout = bring_up(L, 8 << 30, ROCSHMEM_EMU_SPREAD="1", ROCSHMEM_EMU_HEAP_CACHED=None)
+    if full:
         allc["dispatch_put_signal"] = dispatch_config(b, a.steps)
     if a.calibrate:
         cs, cd = b.l.malloc(256 * MiB), b.l.malloc(256 * MiB)
@@ -573,69 +716,142 @@ def main():
         b.l.free(cs)
         b.l.free(cd)
     head = headline(b, a.steps, a.warmup)
-    if not a.quick:
+    if full:
         allc["to_all_P8_64Mi"] = to_all_configs(b, a.steps, a.warmup)
         allc["alltoall_512x7168_bf16"] = alltoall_config(b, a.steps)
         allc["atomic_fetch_add_16Mi"] = amo_config(b, a.steps)
         allc["pingpong"] = pingpong_config(b)
         allc["barrier_P8"] = barrier_config(b)
+        allc["message_rates"] = message_rates(b, a.steps)
+        allc["reuse_256MiB"] = {"uncached_heap": reuse_config(b, a.steps)}
         allc["putmem_curve"] = head["curve"]
         allc["hbm_one_direction_256MiB"] = head["ceilings"]
         allc["putmem_wg_tiled_256MiB"] = head["tiled"]
     b.l.finalize()
-    cpu = None if (a.quick or a.no_cpu) else cpu_baseline()
+    if with_cpu:
+        legs.update(cpu_copy_leg())
+
+    # ---- second bring-up: the default layout, slices packed (stride = heap size),
+    # 1 GiB per PE — what a plain rocshmem_init gives, and the layout BASELINE.json
+    # names ("one 8 GiB symmetric heap").
+    packed = {}
+    if full:
+        b.short = True
+        packed["layout"] = bring_up(L, 1 << 30, ROCSHMEM_EMU_SPREAD=None)
+        packed["putmem_wg"] = headline(b, a.steps, a.warmup)
+        packed["to_all"] = to_all_configs(b, a.steps, a.warmup, which=("fp32_sum",), device_api=False)
+        packed["alltoall"] = alltoall_config(b, a.steps)
+        b.l.finalize()
+        allc["packed_layout_1GiB_per_pe"] = {
+            "layout": packed["layout"],
+            "putmem_wg_nostore_gbs": round(packed["putmem_wg"]["gbs"], 1),
+            "putmem_wg_default_ctx_gbs": round(packed["putmem_wg"]["default_ctx_gbs"], 1),
+            "host_putmem_gbs": round(packed["putmem_wg"]["host_putmem_gbs"], 1),
+            "to_all_fp32_sum": packed["to_all"]["fp32_sum"], "alltoall": packed["alltoall"]}
+    if with_cpu:
+        legs.update(cpu_reduce_leg())
+
+    # ---- third bring-up: a cached heap (plain hipMalloc, what the reference's IPC
+    # build uses), packed, 8 GiB per PE for the dispatch: what a consumer that
+    # re-reads symmetric data gains, and what ordering costs there.
+    cached = {}
+    if full:
+        cached["layout"] = bring_up(L, 8 << 30, ROCSHMEM_EMU_HEAP_CACHED="1")
+        cached["dispatch"] = dispatch_config(b, a.steps)
+        cached["putmem_wg"] = headline(b, a.steps, a.warmup)
+        cached["reuse"] = reuse_config(b, a.steps)
+        b.l.finalize()
+        os.environ.pop("ROCSHMEM_EMU_HEAP_CACHED", None)
+        allc["reuse_256MiB"]["cached_heap"] = cached["reuse"]
+        allc["cached_heap_8GiB_per_pe"] = {
+            "layout": cached["layout"],
+            "putmem_wg_nostore_gbs": round(cached["putmem_wg"]["gbs"], 1),
+            "putmem_wg_default_ctx_gbs": round(cached["putmem_wg"]["default_ctx_gbs"], 1),
+            "host_putmem_gbs": round(cached["putmem_wg"]["host_putmem_gbs"], 1),
+            "dispatch_put_signal": cached["dispatch"]}
+        b.short = False
+    if with_cpu:
+        legs.update(cpu_amo_leg())
+    cpu = cpu_baseline_record(legs) if with_cpu else None
 
     def frac(gbs):
         return round(gbs / HBM_PEAK_GBS, 4)
 
+    verified = bool(head["verified"])
+    # One figure per configuration first (a record that keeps only the leading
+    # keys still carries every configuration), then the rest.
     roof = {"bound": "hbm", "achieved": round(head["gbs"], 1), "peak": HBM_PEAK_GBS,
             "unit": "GB/s", "frac": frac(head["gbs"]),
             # FETCH_SIZE + WRITE_SIZE per launch under rocprofv3 --pmc, scaled by the
             # HIP runtime's own copy kernel (profiles/putmem_wg_tiled_256MiB_hbm_traffic.txt)
-            "traffic": PUT_TRAFFIC_BYTES, "kernel": "rma_kernel<PUT, WG> (rocshmem_ctx_putmem_wg)",
-            "algorithmic_bytes_per_launch": head["bytes_per_step"],
-            # the same message through the other two routes
-            "putmem_wg_all_cus_gbs_nostore": round(head["gbs"], 1),
-            "putmem_wg_all_cus_frac_nostore": frac(head["gbs"]),
-            "putmem_wg_all_cus_gbs": round(head["default_ctx_gbs"], 1),
-            "putmem_wg_all_cus_frac": frac(head["default_ctx_gbs"]),
-            "host_putmem_gbs": round(head["host_putmem_gbs"], 1),
-            "host_putmem_frac": frac(head["host_putmem_gbs"]),
-            "host_getmem_gbs": round(head["host_getmem_gbs"], 1),
-            "getmem_wg_all_cus_gbs_nostore": round(head["getmem_wg_gbs"], 1),
-            "getmem_wg_all_cus_frac_nostore": frac(head["getmem_wg_gbs"])}
-    if not a.quick:
+            "traffic": PUT_TRAFFIC_BYTES, "kernel": "rma_kernel<PUT, WG> (rocshmem_ctx_putmem_wg)"}
+    if full:
         ta, a2a = allc["to_all_P8_64Mi"], allc["alltoall_512x7168_bf16"]
         dp, amo, pp = allc["dispatch_put_signal"], allc["atomic_fetch_add_16Mi"], allc["pingpong"]
+        mr, ru = allc["message_rates"], allc["reuse_256MiB"]
+        verified = verified and bool(packed["putmem_wg"]["verified"]) and bool(cached["putmem_wg"]["verified"])
         roof.update({
+            # configs[1]: bulk putmem through the device API, both kinds of context
+            "verified": verified,
+            "putmem_wg_frac": frac(head["default_ctx_gbs"]),
+            "putmem_wg_frac_nostore": frac(head["gbs"]),
+            # configs[2]: all-reduce P=8 x 64 Mi, host call and device call
+            "to_all_fp32_sum_frac": ta["fp32_sum"]["frac"],
+            "to_all_bf16_sum_frac": ta["bf16_sum"]["frac"],
+            "to_all_int64_xor_frac": ta["int64_xor"]["frac"],
+            "wg_reduce_teams_frac": ta["fp32_sum_wg_reduce_teams_default_ctx"]["frac"],
+            # configs[3]: alltoall and put_signal dispatch
+            "alltoall_frac": a2a["frac"],
+            "dispatch_frac": dp["default_ctx"]["frac"],
+            "dispatch_frac_nostore": dp["nostore_ctx"]["frac"],
+            # configs[4]: atomics and ping-pong
+            "amo_uniform_mops": amo["uniform"]["default_ctx"]["mops"],
+            "amo_zipf_mops": amo["zipf"]["default_ctx"]["mops"],
+            "pingpong_8B_us": pp["8"]["default_ctx"]["latency_us"],
+            # the default (packed) layout, 1 GiB per PE
+            "to_all_fp32_sum_frac_packed": packed["to_all"]["fp32_sum"]["frac"],
+            "putmem_wg_frac_nostore_packed": frac(packed["putmem_wg"]["gbs"]),
+            # configs[0]: int32 sum, P=2 x 1 Mi
+            "to_all_int32_P2_1Mi_gbs": ta["int32_sum_P2_1Mi"]["gbs"],
+            "to_all_fp32_max_frac": ta["fp32_max"]["frac"],
+            # ---- beyond the leading keys
+            "wg_reduce_teams_frac_nostore": ta["fp32_sum_wg_reduce_teams_nostore_ctx"]["frac"],
+            "amo_uniform_mops_nostore": amo["uniform"]["nostore_ctx"]["mops"],
+            "amo_zipf_mops_nostore": amo["zipf"]["nostore_ctx"]["mops"],
+            "putmem_8B_per_lane_mmsg_per_s": mr["putmem_8B_contiguous_default_ctx"]["mmsg_per_s"],
+            "putmem_8B_per_lane_scattered_mmsg_per_s": mr["putmem_8B_scattered_default_ctx"]["mmsg_per_s"],
+            "putmem_64B_per_lane_gbs": mr["putmem_64B_contiguous_default_ctx"]["gbs"],
+            "putmem_4KiB_per_lane_gbs": mr["putmem_4096B_contiguous_default_ctx"]["gbs"],
+            "putmem_wave_512B_gbs": mr["putmem_wave_512B_contiguous_default_ctx"]["gbs"],
+            "putmem_wave_4KiB_gbs": mr["putmem_wave_4096B_contiguous_default_ctx"]["gbs"],
+            "putmem_wave_4KiB_gbs_nostore": mr["putmem_wave_4096B_contiguous_nostore_ctx"]["gbs"],
+            "reuse_read_x4_gbs_uncached_heap": ru["uncached_heap"]["read_x4_gbs"],
+            "reuse_read_x4_gbs_cached_heap": ru["cached_heap"]["read_x4_gbs"],
+            "putmem_wg_frac_cached_heap": frac(cached["putmem_wg"]["default_ctx_gbs"]),
+            "putmem_wg_frac_nostore_cached_heap": frac(cached["putmem_wg"]["gbs"]),
+            "dispatch_frac_cached_heap": cached["dispatch"]["default_ctx"]["frac"],
+            "dispatch_frac_nostore_cached_heap": cached["dispatch"]["nostore_ctx"]["frac"],
+            "alltoall_frac_packed": packed["alltoall"]["frac"],
+            "algorithmic_bytes_per_launch": head["bytes_per_step"],
+            "host_putmem_frac": frac(head["host_putmem_gbs"]),
+            "host_getmem_frac": frac(head["host_getmem_gbs"]),
+            "getmem_wg_frac_nostore": frac(head["getmem_wg_gbs"]),
             "hbm_read_only_gbs": head["ceilings"]["read_only_gbs"],
             "hbm_write_only_gbs": head["ceilings"]["write_only_gbs"],
             "l2_release_ns_each_per_tile": head["release_ns_each_per_tile"],
             "l2_release_ns_each_at_end": head["release_ns_each_at_end"],
-            "to_all_fp32_sum_gbs": ta["fp32_sum"]["gbs"], "to_all_fp32_sum_frac": ta["fp32_sum"]["frac"],
-            "to_all_fp32_max_gbs": ta["fp32_max"]["gbs"], "to_all_fp32_max_frac": ta["fp32_max"]["frac"],
-            "to_all_bf16_sum_gbs": ta["bf16_sum"]["gbs"], "to_all_bf16_sum_frac": ta["bf16_sum"]["frac"],
-            "to_all_int64_xor_gbs": ta["int64_xor"]["gbs"], "to_all_int64_xor_frac": ta["int64_xor"]["frac"],
-            "wg_reduce_fp32_sum_32_teams_gbs": ta["fp32_sum_wg_reduce_32_teams_default_ctx"]["gbs"],
-            "wg_reduce_fp32_sum_32_teams_frac": ta["fp32_sum_wg_reduce_32_teams_default_ctx"]["frac"],
-            "wg_reduce_fp32_sum_32_teams_gbs_nostore": ta["fp32_sum_wg_reduce_32_teams_nostore_ctx"]["gbs"],
-            "wg_reduce_fp32_sum_32_teams_frac_nostore": ta["fp32_sum_wg_reduce_32_teams_nostore_ctx"]["frac"],
             "wg_reduce_fp32_sum_one_wg_per_pe_gbs": ta["fp32_sum_wg_reduce_one_wg_per_pe"]["gbs"],
-            "alltoall_gbs": a2a["gbs"], "alltoall_frac": a2a["frac"],
             "fcollect_frac": a2a["fcollect_same_block"]["frac"],
             "broadcast_frac": a2a["broadcast_P_blocks_from_pe0"]["frac"],
-            "dispatch_gbs": dp["default_ctx"]["gbs"], "dispatch_frac": dp["default_ctx"]["frac"],
-            "dispatch_gbs_nostore": dp["nostore_ctx"]["gbs"], "dispatch_frac_nostore": dp["nostore_ctx"]["frac"],
-            "amo_uniform_mops": amo["uniform"]["default_ctx"]["mops"],
-            "amo_uniform_mops_nostore": amo["uniform"]["nostore_ctx"]["mops"],
-            "amo_zipf_mops": amo["zipf"]["default_ctx"]["mops"],
-            "amo_zipf_mops_nostore": amo["zipf"]["nostore_ctx"]["mops"],
-            "pingpong_8B_us": pp["8"]["default_ctx"]["latency_us"],
             "pingpong_8B_us_nostore": pp["8"]["nostore_ctx"]["latency_us"],
             "pingpong_64KiB_us": pp["65536"]["default_ctx"]["latency_us"],
             "pingpong_32pairs_msg_per_s": pp["8_x32pairs"]["nostore_ctx"]["msg_per_s"],
             "barrier_all_round_us": allc["barrier_P8"]["barrier_all_round_us"],
         })
+    else:
+        roof.update({"verified": verified, "putmem_wg_frac": frac(head["default_ctx_gbs"]),
+                     "putmem_wg_frac_nostore": frac(head["gbs"]),
+                     "host_putmem_frac": frac(head["host_putmem_gbs"])})
     line = {
         "metric": "HBM GB/s (% of MI355X peak) for to_all/alltoall/putmem; atomic Mops/s",
         "value": round(head["gbs"], 1),
@@ -649,17 +865,16 @@ def main():
         "vs_baseline": None,
         "dtype": "u8",
         "data": "synthetic",
-        "config": {"workload": "bulk putmem through the device API: one 256 MiB message per step from PE "
-                               "k%8 to PE (k+1)%8 of P=8 slices in one symmetric heap, every CU calling "
-                               "rocshmem_ctx_putmem_wg on " + "%d-byte tiles (one tile per work-group of %d) " % (
-                                   PUT_SHAPES["nostore_ctx"][1], PUT_SHAPES["nostore_ctx"][0]) +
-                               "through a ROCSHMEM_CTX_NOSTORE context, one quiet per work-group "
-                               "(BASELINE configs[1], largest size; buffers rotate so no step re-reads "
-                               "cached data)",
+        "config": {"workload": "configs[1] largest size: 256 MiB putmem per step, PE k%8 -> (k+1)%8 of P=8, "
+                               "every CU calling rocshmem_ctx_putmem_wg",
+                   "detail": "one %d-byte tile per work-group of %d, ROCSHMEM_CTX_NOSTORE context, one quiet "
+                             "per work-group; buffers rotate so no step re-reads cached data" % (
+                                 PUT_SHAPES["nostore_ctx"][1], PUT_SHAPES["nostore_ctx"][0]),
                    "n_pes": P, "message_bytes": 256 * MiB, "heap_bytes_per_pe": 8 << 30,
-                   "layout": "ROCSHMEM_EMU_SPREAD=%s" % os.environ.get("ROCSHMEM_EMU_SPREAD"),
+                   "layout": "ROCSHMEM_EMU_SPREAD=1",
                    "pe_stride_bytes": layout["pe_stride_bytes"],
-                   "heap_alloc_bytes": layout["heap_alloc_bytes"]},
+                   "heap_alloc_bytes": layout["heap_alloc_bytes"],
+                   "verified": verified},
         "roofline": roof,
         # the reference's own convention (tests/functional_tests/tester.cpp:505-508):
         # payload bytes per second in GiB/s, counting each byte once

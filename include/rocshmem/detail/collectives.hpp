@@ -43,10 +43,25 @@ __device__ __forceinline__ void barrier_all(Context *c) {
 // and its two algorithms (src/ipc/context_ipc_tmpl_device.hpp:166-418) by a
 // direct reduce-scatter + all-gather in one pass: after every member has
 // arrived, member k folds its share of the index range (every P-th block of
-// one vector per lane) from all P sources in ascending member order and stores
-// the result into all P destinations; a second barrier ends the operation.  Each element is computed once, so all
-// members hold bit-identical results.  Keeps the reference's refusal of teams
-// with 2*P > ROCSHMEM_REDUCE_SYNC_SIZE (:412-415).
+// kShareVectors vectors, whatever the size of its work-group) from all P
+// sources in ascending member order and stores the result into all P
+// destinations; a second barrier ends the operation.  Each element is computed
+// once, so all members hold bit-identical results.
+//
+// The reference's selector (:361-418) takes its direct path when P * nreduce
+// elements fit max(nreduce / 2 + 1, ROCSHMEM_REDUCE_MIN_WRKDATA_SIZE) and
+// P <= ROCSHMEM_REDUCE_SYNC_SIZE, otherwise its ring when
+// 2 * P <= ROCSHMEM_REDUCE_SYNC_SIZE, and otherwise returns ROCSHMEM_ERROR.
+// Nothing here needs those buffers, but the same calls are refused so that a
+// program sees the same status on either library.
+__device__ __forceinline__ bool reduce_accepted(int P, int nreduce) {
+  const size_t direct_wrk = static_cast<size_t>(P) * static_cast<size_t>(nreduce);
+  size_t provided_wrk = static_cast<size_t>(nreduce / 2 + 1);
+  if (provided_wrk < ROCSHMEM_REDUCE_MIN_WRKDATA_SIZE) provided_wrk = ROCSHMEM_REDUCE_MIN_WRKDATA_SIZE;
+  if (provided_wrk >= direct_wrk && static_cast<size_t>(P) <= ROCSHMEM_REDUCE_SYNC_SIZE) return true;
+  return static_cast<size_t>(2 * P) <= ROCSHMEM_REDUCE_SYNC_SIZE;
+}
+
 template <typename E, ROCSHMEM_OP Op>
 __device__ __forceinline__ int wg_reduce(Context *c, Team *t,
                                          typename ElemTraits<E>::storage *dest,
@@ -54,7 +69,7 @@ __device__ __forceinline__ int wg_reduce(Context *c, Team *t,
                                          int nreduce) {
   using S = typename ElemTraits<E>::storage;
   const int P = t->num_pes;
-  if (static_cast<size_t>(2 * P) > ROCSHMEM_REDUCE_SYNC_SIZE) return ROCSHMEM_ERROR;
+  if (!reduce_accepted(P, nreduce)) return ROCSHMEM_ERROR;
 
   // Entry: every member's source, which its caller may have written with plain
   // stores, is final.
@@ -72,11 +87,11 @@ __device__ __forceinline__ int wg_reduce(Context *c, Team *t,
   // the bulk copy does.
   const size_t part = static_cast<size_t>(t->my_pe), nparts = static_cast<size_t>(P);
   if (n * sizeof(S) >= g_state.nt_bytes)
-    fold_span_any<E, Op, true>(dst0, src0, hop, P, 0, n, flat_thread_id(), flat_block_size(), part,
-                               nparts);
+    fold_span_any<E, Op, true, true>(dst0, src0, hop, P, 0, n, flat_thread_id(), flat_block_size(),
+                                     part, nparts);
   else
-    fold_span_any<E, Op, false>(dst0, src0, hop, P, 0, n, flat_thread_id(), flat_block_size(), part,
-                                nparts);
+    fold_span_any<E, Op, false, true>(dst0, src0, hop, P, 0, n, flat_thread_id(),
+                                      flat_block_size(), part, nparts);
 
   // Exit: the results were written by the fold, through to memory.
   team_pad_sync(c, t, SYNC_REDUCE, PUBLISH_LIBRARY);

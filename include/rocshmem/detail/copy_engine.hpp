@@ -112,15 +112,32 @@ __device__ __forceinline__ bool in_lds_or_scratch(const void *p) {
 
 // The local side of a put or get may be a __shared__ array or a stack
 // variable (the reference copies through generic pointers, so it accepts
-// them).  Buffer stores and global loads cannot reach those, so such a copy
-// goes through flat accesses, 16 bytes per lane per step and bytes at the end.
+// them).  Global loads cannot reach those, so such a copy reads through flat
+// accesses, 16 bytes per lane per step and bytes at the end.  A destination in
+// device memory (a put from a local buffer) is still written with write-through
+// buffer stores, like every other store of a cooperative copy: completion on a
+// ROCSHMEM_CTX_NOSTORE context counts on that.  n <= kWindowBytes.
 __device__ __forceinline__ void copy_generic(char *dst, const char *src, size_t n, size_t lane,
-                                          size_t nlanes) {
+                                             size_t nlanes) {
   const size_t nvec = n >> 4;
-  for (size_t i = lane; i < nvec; i += nlanes)
-    *reinterpret_cast<u32x4_any *>(dst + (i << 4)) =
-        *reinterpret_cast<const u32x4_any *>(src + (i << 4));
-  for (size_t k = (nvec << 4) + lane; k < n; k += nlanes) dst[k] = src[k];
+  if (in_lds_or_scratch(dst)) {
+    for (size_t i = lane; i < nvec; i += nlanes)
+      *reinterpret_cast<u32x4_any *>(dst + (i << 4)) =
+          *reinterpret_cast<const u32x4_any *>(src + (i << 4));
+    for (size_t k = (nvec << 4) + lane; k < n; k += nlanes) dst[k] = src[k];
+    return;
+  }
+  const __amdgpu_buffer_rsrc_t w = window_of(dst, n);
+  size_t head = (16u - (reinterpret_cast<uintptr_t>(dst) & 15u)) & 15u;
+  if (head > n) head = n;
+  for (size_t k = lane; k < head; k += nlanes)
+    store1(w, static_cast<uint32_t>(k), static_cast<uint8_t>(src[k]));
+  const size_t body_vec = (n - head) >> 4;
+  for (size_t i = lane; i < body_vec; i += nlanes)
+    store16<false>(w, static_cast<uint32_t>(head + (i << 4)),
+                   *reinterpret_cast<const u32x4_any *>(src + head + (i << 4)));
+  for (size_t k = head + (body_vec << 4) + lane; k < n; k += nlanes)
+    store1(w, static_cast<uint32_t>(k), static_cast<uint8_t>(src[k]));
 }
 
 // Copy n <= kWindowBytes bytes with `nlanes` cooperating lanes; this lane is

@@ -137,6 +137,13 @@ __device__ __forceinline__ void store_elem(__amdgpu_buffer_rsrc_t w, uint32_t of
   }
 }
 
+// Vectors (16 bytes each) per block when several groups share one range: the
+// unit in which team members take turns through the arrays.  A constant, so
+// that the split does not depend on how many lanes each group brings (team
+// members may run work-groups of different sizes); 1024 keeps every lane of
+// the largest work-group busy.
+constexpr size_t kShareVectors = 1024;
+
 // Fold elements [lo, hi) across P team members and store the result on all P.
 //   src0 / dst0 : the buffers on team member 0
 //   hop         : bytes from one team member's buffer to the next member's
@@ -146,15 +153,16 @@ __device__ __forceinline__ void store_elem(__amdgpu_buffer_rsrc_t w, uint32_t of
 // (hi - lo) * sizeof(element) must not exceed kWindowBytes.  Results leave as
 // write-through buffer stores, one resource per destination.
 //
-// The range may be shared by `nparts` such groups of equal size (the members
-// of a team, one work-group each): group `part` takes the blocks part,
-// part + nparts, ... of nlanes vectors each, so the groups work side by side
-// through the arrays.  Group 0 also takes the unaligned head, the last group
-// the tail.  (Measured on MI355X, P = 8 x 64 Mi fp32, 256-1024 work-groups that
-// loop: 6.3-6.4 TB/s for this split and for contiguous chunks alike, against
-// 6.45 for one-vector work-groups; issuing a lane's next loads ahead of its
-// stores gained nothing and cost 20-40 registers.)
-template <typename E, ROCSHMEM_OP Op, int kP, bool kNonTemporal>
+// With kShared the range is shared by `nparts` such groups (the members of a
+// team, one work-group each, of any sizes): group `part` takes the blocks
+// part, part + nparts, ... of kShareVectors vectors each and strides through
+// a block with its own lanes, so the groups work side by side through the
+// arrays.  Group 0 also takes the unaligned head, the last group the tail.
+// (Measured on MI355X, P = 8 x 64 Mi fp32, 256-1024 work-groups that loop:
+// 6.3-6.4 TB/s for this split and for contiguous chunks alike, against 6.45
+// for one-vector work-groups; issuing a lane's next loads ahead of its stores
+// gained nothing and cost 20-40 registers.)
+template <typename E, ROCSHMEM_OP Op, int kP, bool kNonTemporal, bool kShared = false>
 __device__ __forceinline__ void fold_window(
     typename ElemTraits<E>::storage *dst0,
     const typename ElemTraits<E>::storage *src0, int64_t hop, int np,
@@ -188,7 +196,6 @@ __device__ __forceinline__ void fold_window(
     for (size_t k = lane; k < head; k += nlanes) scalar_one(lo + k);
   const size_t vlo = lo + head;
   const size_t nvec = (hi - vlo) / V;
-  const size_t step = nparts * nlanes;
   // Vector v of the window sits 16 * v bytes after element vlo in every source
   // and destination.  Each source is a global-memory base in scalar registers
   // plus that one 32-bit offset, each destination a buffer resource built once.
@@ -197,6 +204,17 @@ __device__ __forceinline__ void fold_window(
   const size_t vec_bytes = nvec << 4;
   auto load_vec = [&](GlobalBytes base, uint32_t off) -> r_u32x4 {
     return load16<kNonTemporal>(base, off);
+  };
+  // Calls body(v) for every vector index this lane owns.
+  auto for_my_vectors = [&](auto &&body) {
+    if constexpr (kShared) {
+      for (size_t b = part * kShareVectors; b < nvec; b += nparts * kShareVectors) {
+        const size_t bend = b + kShareVectors < nvec ? b + kShareVectors : nvec;
+        for (size_t v = b + lane; v < bend; v += nlanes) body(v);
+      }
+    } else {
+      for (size_t v = lane; v < nvec; v += nlanes) body(v);
+    }
   };
 
   if constexpr (kP != 0) {
@@ -207,7 +225,7 @@ __device__ __forceinline__ void fold_window(
       from[p] = wave_uniform_global(first_src + p * hop);
       to[p] = window_of(first_dst + p * hop, vec_bytes);
     }
-    for (size_t v = part * nlanes + lane; v < nvec; v += step) {
+    for_my_vectors([&](size_t v) {
       const uint32_t off = static_cast<uint32_t>(v << 4);
       Pack<S> in[kP], out;
 #pragma unroll
@@ -221,9 +239,9 @@ __device__ __forceinline__ void fold_window(
       }
 #pragma unroll
       for (int p = 0; p < kP; ++p) store16<kNonTemporal>(to[p], off, out.raw);
-    }
+    });
   } else {
-    for (size_t v = part * nlanes + lane; v < nvec; v += step) {
+    for_my_vectors([&](size_t v) {
       const uint32_t off = static_cast<uint32_t>(v << 4);
       A acc[V];
       Pack<S> in, out;
@@ -239,7 +257,7 @@ __device__ __forceinline__ void fold_window(
       for (int e = 0; e < V; ++e) out.e[e] = Tr::narrow(acc[e]);
       for (int p = 0; p < P; ++p)
         store16<kNonTemporal>(window_of(first_dst + p * hop, vec_bytes), off, out.raw);
-    }
+    });
   }
 
   const size_t tlo = vlo + nvec * V;
@@ -248,28 +266,29 @@ __device__ __forceinline__ void fold_window(
 }
 
 // Any range: windows of at most kWindowBytes.
-template <typename E, ROCSHMEM_OP Op, int kP, bool kNonTemporal>
+template <typename E, ROCSHMEM_OP Op, int kP, bool kNonTemporal, bool kShared = false>
 __device__ __forceinline__ void fold_span(
     typename ElemTraits<E>::storage *dst0,
     const typename ElemTraits<E>::storage *src0, int64_t hop, int np,
     size_t lo, size_t hi, size_t lane, size_t nlanes, size_t part = 0, size_t nparts = 1) {
   constexpr size_t kWin = kWindowBytes / sizeof(typename ElemTraits<E>::storage);
   while (hi - lo > kWin) {
-    fold_window<E, Op, kP, kNonTemporal>(dst0, src0, hop, np, lo, lo + kWin, lane, nlanes, part,
-                                         nparts);
+    fold_window<E, Op, kP, kNonTemporal, kShared>(dst0, src0, hop, np, lo, lo + kWin, lane, nlanes,
+                                                  part, nparts);
     lo += kWin;
   }
-  fold_window<E, Op, kP, kNonTemporal>(dst0, src0, hop, np, lo, hi, lane, nlanes, part, nparts);
+  fold_window<E, Op, kP, kNonTemporal, kShared>(dst0, src0, hop, np, lo, hi, lane, nlanes, part,
+                                                nparts);
 }
 
 // Dispatch on the team size so the common sizes get fully unrolled loads.
-template <typename E, ROCSHMEM_OP Op, bool kNonTemporal>
+template <typename E, ROCSHMEM_OP Op, bool kNonTemporal, bool kShared = false>
 __device__ __forceinline__ void fold_span_any(
     typename ElemTraits<E>::storage *dst0,
     const typename ElemTraits<E>::storage *src0, int64_t hop, int np,
     size_t lo, size_t hi, size_t lane, size_t nlanes, size_t part = 0, size_t nparts = 1) {
 #define ROCSHMEM_AMD_FOLD_CASE(KP) \
-  fold_span<E, Op, KP, kNonTemporal>(dst0, src0, hop, np, lo, hi, lane, nlanes, part, nparts)
+  fold_span<E, Op, KP, kNonTemporal, kShared>(dst0, src0, hop, np, lo, hi, lane, nlanes, part, nparts)
   switch (np) {
     case 2: ROCSHMEM_AMD_FOLD_CASE(2); break;
     case 4: ROCSHMEM_AMD_FOLD_CASE(4); break;

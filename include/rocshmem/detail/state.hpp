@@ -215,16 +215,24 @@ __device__ __forceinline__ T *remote_ws(const Context *c, T *local, int pe) {
   return reinterpret_cast<T *>(reinterpret_cast<char *>(local) + hop);
 }
 
-// Work-group extents.  The three 16-bit sizes sit at bytes 12, 14 and 16 of
-// the implicit kernel arguments (code object version 5 and later, hipcc's
-// default; earlier versions are not supported); read as
-// the two aligned words that hold them they come through scalar loads, where
-// blockDim.y and .z read one by one get merged into a misaligned word that
-// only the vector memory path can fetch.
+// Work-group extents.  From code object version 5 on (hipcc's default is
+// later still) the three 16-bit sizes sit at bytes 12, 14 and 16 of the
+// implicit kernel arguments; read as the two aligned words that hold them they
+// come through scalar loads, where blockDim.y and .z read one by one get
+// merged into a misaligned word that only the vector memory path can fetch.
+// A translation unit built for an older code object version
+// (-mcode-object-version=4) has another layout there and takes blockDim: the
+// version is a constant of the device libraries, so the test folds away.
 struct BlockExtent {
   unsigned x, y, z;
 };
+#if defined(__HIP_DEVICE_COMPILE__)
+extern "C" __device__ const int __oclc_ABI_version;
+#endif
 __device__ __forceinline__ BlockExtent block_extent() {
+#if defined(__HIP_DEVICE_COMPILE__)
+  if (__oclc_ABI_version < 500) return BlockExtent{blockDim.x, blockDim.y, blockDim.z};
+#endif
   typedef const __attribute__((address_space(4))) uint32_t const_u32;
   const_u32 *ia = (const_u32 *)__builtin_amdgcn_implicitarg_ptr();  // NOLINT
   const uint32_t xy = ia[3], z = ia[4];

@@ -11,10 +11,17 @@
 #include <cstddef>
 #include <cstdint>
 
+// The device API is defined in these headers.  A call that stays a call costs
+// a GPU kernel the callee's worst-case register budget, a stack frame in
+// scratch memory and spilled scalar registers around it (the many-teams
+// all-reduce driver: 120 vector registers and 88 bytes of scratch per lane
+// with the public function called, against 40 and none with it inlined), so
+// by default every public device function is inlined into its caller.
+// USE_FUNC_CALL keeps the reference's meaning: real calls.
 #ifdef USE_FUNC_CALL
 #define ATTR_NO_INLINE __attribute__((noinline))
 #else
-#define ATTR_NO_INLINE
+#define ATTR_NO_INLINE __attribute__((always_inline))
 #endif
 
 namespace rocshmem {

@@ -149,6 +149,17 @@ size_t rocshmem_amd_pe_stride(void);
  * pe_stride x P by default (stride = heap size rounded up to 2 MiB);
  * ROCSHMEM_EMU_SPREAD=1 spreads the slices over half of the device memory. */
 size_t rocshmem_amd_heap_alloc_bytes(void);
+/* 1 when the heap of the live runtime is uncached device memory (the default),
+ * 0 under ROCSHMEM_EMU_HEAP_CACHED=1 (plain hipMalloc, what the reference's
+ * IPC build uses: src/memory/heap_type.hpp:41-51), -1 before rocshmem_init. */
+int rocshmem_amd_heap_is_uncached(void);
+/* Uncached heap blocks are kept until the process ends (rocshmem_finalize
+ * marks them idle, a later rocshmem_init reuses the smallest idle block that
+ * is large enough).  total_bytes: all such blocks of this process; idle_bytes:
+ * those no live runtime uses.  A new block that would take the total beyond
+ * ROCSHMEM_EMU_HEAP_HELD_LIMIT (bytes, default: the device memory) is refused
+ * with a message.  No reference counterpart. */
+int rocshmem_amd_heap_held(size_t *total_bytes, size_t *idle_bytes);
 
 /* The allocator on its own, usable without a GPU (planning and host-side
  * tests): a model heap of heap_bytes whose base has the alignment of
@@ -211,23 +222,12 @@ int rocshmem_amd_dev_free(void *ptr);
 int rocshmem_amd_copy_in(void *dst_dev, const void *src_host, size_t n);
 int rocshmem_amd_copy_out(void *dst_host, const void *src_dev, size_t n);
 int rocshmem_amd_fill(void *dst_dev, int byte, size_t n);
-/* Measurement aid (no reference counterpart): reads (write == 0) or overwrites
- * (write != 0) nbytes (>= 1 MiB, 16-byte aligned) of device memory with the
- * whole GPU, with the load and store instructions of the bulk copy, and nothing
- * else — the one-directional rate of the memory system that a copy is judged
- * against. */
-int rocshmem_amd_hbm_probe(int write, void *buf, size_t nbytes, rocshmem_amd_stream_t stream);
-/* Measurement aid (no reference counterpart): what one agent-scope release —
- * the L2 write-back that rocshmem_ctx_quiet / fence and every barrier perform
- * on a default context — costs while a copy is running.  n_wgs work-groups of
- * wg_size threads copy nbytes from src to dst in tiles of tile_bytes (tile t
- * to work-group t mod n_wgs) with the cooperative copy of putmem_wg and issue a
- * release never (mode 0), once per work-group at its end (mode 1) or after
- * every tile (mode 2).  Time modes 1 / 2 against mode 0 and divide by the
- * number of releases. */
-int rocshmem_amd_release_probe(int mode, void *dst, const void *src, size_t nbytes,
-                               size_t tile_bytes, int n_wgs, int wg_size,
-                               rocshmem_amd_stream_t stream);
+/* Compares two device buffers on the device (after waiting for the stream):
+ * differing_out = the number of 16-byte vectors, plus tail bytes, in which they
+ * differ.  How the benchmark verifies what its timed loops moved without
+ * bringing 256 MiB back to the host.  No reference counterpart. */
+int rocshmem_amd_compare(const void *x, const void *y, size_t nbytes, uint64_t *differing_out,
+                         rocshmem_amd_stream_t stream);
 /* The symmetric object `sym` (address on PE 0) set to `byte` on every PE with
  * one launch on `stream` — e.g. signal words cleared between dispatches. */
 int rocshmem_amd_fill_every_pe(void *sym, int byte, size_t n, rocshmem_amd_stream_t stream);
@@ -258,6 +258,17 @@ int rocshmem_amd_timer_destroy(void *timer);
 int rocshmem_amd_rma(int rma_op, int gran, void *dest, const void *source, size_t nbytes,
                      size_t tile_bytes, int my_pe, int pe, int n_wgs, int wg_size,
                      int iters, rocshmem_amd_stream_t stream);
+/* The same with the tiles visited through a permutation when `scattered` is
+ * nonzero: group g's i-th call moves the tile at slot ((i * odd) mod n_tiles)
+ * of both buffers instead of slot i, so that the messages of neighbouring
+ * lanes (or wavefronts) are far apart — the access pattern of the reference's
+ * per-thread testers with random targets, as opposed to lanes that continue
+ * one another (scripts/functional_tests/driver.sh:142-218 runs both
+ * granularities over sizes from 1 B up).  Needs a power-of-two number of whole
+ * tiles, else -1. */
+int rocshmem_amd_rma_messages(int rma_op, int gran, void *dest, const void *source, size_t nbytes,
+                              size_t tile_bytes, int scattered, int my_pe, int pe, int n_wgs,
+                              int wg_size, int iters, rocshmem_amd_stream_t stream);
 
 /* The same calls with the local buffer in LDS: one work-group stages `nbytes`
  * of `source` (a device buffer) in a __shared__ array, puts from there to
@@ -304,29 +315,45 @@ int rocshmem_amd_wg_reduce(int dtype, int op, rocshmem_amd_team_t team, void *de
 /* The same call made by n_teams (<= 256) work-groups per PE at once, each with a
  * team of its own over the same PEs — how the reference's testers spread a
  * device collective over the GPU (one team per work-group,
- * tests/functional_tests/team_reduction_tester.cpp:60-110).  Team t reduces
- * the t-th slice of the arrays (equal slices, whole 16-byte vectors).  teams:
- * host array of handles of distinct teams with the same members.  Every
- * work-group makes the call `iters` (>= 1) times in a row inside the kernel, as
- * the reference's testers loop inside theirs.  Returns the largest device
- * status any team saw, after waiting for the kernel; -1 if nothing was
- * launched (bad argument, or the grid n_teams x P cannot be resident at once). */
+ * tests/functional_tests/team_reduction_tester.cpp:60-110).  The arrays are
+ * cut into equal slices of whole 16-byte vectors: with chunk_elems == 0 one
+ * slice per team (team t reduces the t-th), otherwise slices of chunk_elems
+ * elements dealt out in turn (team t reduces slices t, t + n_teams, ..., one
+ * call each, so that at any moment the teams work side by side in one narrow
+ * window of the arrays).  teams: host array of handles of distinct teams with
+ * the same members.  Every work-group makes its calls `iters` (>= 1) times in
+ * a row inside the kernel, as the reference's testers loop inside theirs.
+ * Returns the largest device status any team saw, after waiting for the
+ * kernel; -1 if nothing was launched (bad argument, or the grid n_teams x P
+ * cannot be resident at once). */
 int rocshmem_amd_wg_reduce_teams(int dtype, int op, const rocshmem_amd_team_t *teams, int n_teams,
-                                 void *dest, const void *source, int nreduce, int wg_size,
-                                 int iters, rocshmem_amd_stream_t stream);
+                                 void *dest, const void *source, int nreduce, int chunk_elems,
+                                 int wg_size, int iters, rocshmem_amd_stream_t stream);
 /* rocshmem_amd_wg_reduce_teams for callers that cannot allocate device memory
- * (code under HIP graph capture, tight serving loops, harnesses that forbid
- * hipMalloc).  It has no counterpart in the reference.  Same arguments, same
- * results; the per-team status words, which rocshmem_amd_wg_reduce_teams
- * allocates and frees on every call, live in a fixed array inside the library's
- * code object instead: 256 words (1 KiB) per GPU, held until the process ends.
- * The call makes no hipMalloc / hipFree.  n_teams beyond 256 is refused with a
- * message on stderr.  All calls on one GPU share the array: it is cleared on the
- * stream before each launch, and two calls that overlap in time on one GPU
- * race on it (run them one after the other). */
+ * (tight serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  Same arguments, same results; the per-team
+ * status words, which rocshmem_amd_wg_reduce_teams allocates and frees on
+ * every call, live in a fixed array inside the library's code object instead:
+ * 256 words (1 KiB) per GPU, held until the process ends.  The call makes no
+ * hipMalloc / hipFree; like its sibling it waits for the kernel and copies the
+ * status words back, so it is not for code under stream capture.  n_teams
+ * beyond 256 is refused with a message on stderr.  All calls on one GPU share
+ * the array: once the arguments have been accepted it is cleared on the stream
+ * before the launch, and two calls that overlap in time on one GPU race on it
+ * (run them one after the other). */
 int rocshmem_amd_wg_reduce_teams_static(int dtype, int op, const rocshmem_amd_team_t *teams,
                                         int n_teams, void *dest, const void *source, int nreduce,
-                                        int wg_size, int iters, rocshmem_amd_stream_t stream);
+                                        int chunk_elems, int wg_size, int iters,
+                                        rocshmem_amd_stream_t stream);
+/* The members' shares of one int32 sum all-reduce over the world team computed
+ * by work-groups of different sizes in one launch: block k stands for member k
+ * and works with lanes_per_member[k] (1..1024) lanes.  Runs the fold that
+ * rocshmem_ctx_<T>_<op>_wg_reduce performs between its two barriers
+ * (include/rocshmem/detail/reduce_engine.hpp); a test aid for the rule that a
+ * member's share of the index range does not depend on work-group sizes.
+ * dest / source: symmetric addresses on PE 0. */
+int rocshmem_amd_fold_shares(void *dest, const void *source, int nreduce,
+                             const int *lanes_per_member, rocshmem_amd_stream_t stream);
 /* rocshmem_ctx_<T>_wg_alltoall / _wg_broadcast / _wg_fcollect
  * (rocshmem_COLL.hpp:44-258; context_ipc_tmpl_device.hpp:420-531).
  * elem_size in {1,2,4,8} selects the typed entry point (char/short/int/long). */
@@ -461,7 +488,9 @@ int rocshmem_amd_signal_fetch(int gran, const uint64_t *sig_addr, int my_pe,
  * with_signal == 2 / 3: the message goes out as several
  * rocshmem_ctx_putmem_nbi_wave calls per wavefront / rocshmem_ctx_putmem_nbi
  * calls of 12 bytes per thread, every thread calls rocshmem_ctx_quiet, and
- * thread 0 sets the flag after a work-group barrier;
+ * thread 0 sets the flag after a work-group barrier; with_signal == 4 / 5: as
+ * 0 / 1 with the pattern staged in the producer's LDS (nbytes <= 64 KiB), so
+ * the put's local side is a __shared__ buffer;
  * the receiver waits for the flag, compares every word, and acknowledges.  data: pairs*nbytes symmetric bytes,
  * flags: 2*pairs symmetric uint64 (addresses on pe_a).  mismatches_out = words
  * that differed; timed_out_out = 1 if a bounded wait ran out (all work-groups

@@ -48,6 +48,12 @@ int rocshmem_amd_dev_mem_info(size_t *free_bytes, size_t *total_bytes) {
   return hipMemGetInfo(free_bytes, total_bytes) == hipSuccess ? 0 : -1;
 }
 size_t rocshmem_amd_heap_alloc_bytes(void) { return rt().live ? rt().heap_alloc_bytes : 0; }
+int rocshmem_amd_heap_is_uncached(void) { return rt().live ? (rt().heap_uncached ? 1 : 0) : -1; }
+int rocshmem_amd_heap_held(size_t *total_bytes, size_t *idle_bytes) {
+  if (!total_bytes || !idle_bytes) return -1;
+  rocshmem::runtime::heap_held(total_bytes, idle_bytes);
+  return 0;
+}
 int rocshmem_amd_pe_threads_enter(int PE_start, int PE_stride, int PE_size) {
   return rocshmem::runtime::pe_threads_enter(PE_start, PE_stride, PE_size, nullptr) ? 1 : 0;
 }

@@ -47,8 +47,8 @@ struct PublicReduce;
   template <>                                                                      \
   struct PublicReduce<T, OP> {                                                     \
     using storage = T;                                                             \
-    __device__ static int call(rocshmem_ctx_t c, rocshmem_team_t t, T *d, const T *s, \
-                               int n) {                                            \
+    __device__ __forceinline__ static int call(rocshmem_ctx_t c, rocshmem_team_t t, T *d, \
+                                              const T *s, int n) {                             \
       return rocshmem_ctx_##TN##_##OPN##_wg_reduce(c, t, d, s, n);                 \
     }                                                                              \
   };
@@ -71,7 +71,7 @@ DRV_PUBLIC_ARITH(double, double)
 template <>
 struct PublicReduce<rocshmem_bf16, ROCSHMEM_SUM> {
   using storage = rocshmem_bf16;
-  __device__ static int call(rocshmem_ctx_t c, rocshmem_team_t t, rocshmem_bf16 *d,
+  __device__ __forceinline__ static int call(rocshmem_ctx_t c, rocshmem_team_t t, rocshmem_bf16 *d,
                              const rocshmem_bf16 *s, int n) {
     return rocshmem_ctx_bf16_sum_wg_reduce(c, t, d, s, n);
   }
@@ -99,8 +99,8 @@ struct WgTeamsArgs {
   int pe_start;
   int stride;
   int nelems;       // all slices together
-  int slice_elems;  // per team
-  int iters;        // calls per work-group, one after the other
+  int slice_elems;  // per call: team y reduces slices y, y + teams, ... one call each
+  int iters;        // passes over the whole range, one after the other
   int *status;      // [teams] largest return code each team saw
 };
 
@@ -110,16 +110,38 @@ __global__ void wg_reduce_teams_kernel(WgTeamsArgs a) {
   detail::Team *row = a.rows[blockIdx.y];
   const rocshmem_ctx_t ctx{a.ctx_row + pe, &row[pe].wrt_world};
   const rocshmem_team_t team = reinterpret_cast<rocshmem_team_t>(row + pe);
-  const long lo = static_cast<long>(blockIdx.y) * a.slice_elems;
-  long cnt = a.nelems - lo;
-  if (cnt > a.slice_elems) cnt = a.slice_elems;
-  if (cnt < 0) cnt = 0;
-  T *dest = reinterpret_cast<T *>(a.dest0 + static_cast<uint64_t>(pe) * a.pe_stride) + lo;
-  const T *source = reinterpret_cast<const T *>(a.src0 + static_cast<uint64_t>(pe) * a.pe_stride) + lo;
+  T *dest = reinterpret_cast<T *>(a.dest0 + static_cast<uint64_t>(pe) * a.pe_stride);
+  const T *source = reinterpret_cast<const T *>(a.src0 + static_cast<uint64_t>(pe) * a.pe_stride);
+  const long step = static_cast<long>(gridDim.y) * a.slice_elems;
   for (int it = 0; it < a.iters; ++it) {
-    const int rc = PublicReduce<T, Op>::call(ctx, team, dest, source, static_cast<int>(cnt));
-    if (threadIdx.x == 0 && rc != ROCSHMEM_SUCCESS) atomicMax(a.status + blockIdx.y, rc);
+    for (long lo = static_cast<long>(blockIdx.y) * a.slice_elems; lo < a.nelems; lo += step) {
+      const long left = a.nelems - lo;
+      const int cnt = static_cast<int>(left < a.slice_elems ? left : a.slice_elems);
+      const int rc = PublicReduce<T, Op>::call(ctx, team, dest + lo, source + lo, cnt);
+      if (threadIdx.x == 0 && rc != ROCSHMEM_SUCCESS) atomicMax(a.status + blockIdx.y, rc);
+    }
   }
+}
+
+// The members' shares of one all-reduce computed by work-groups of DIFFERENT
+// sizes: block k stands for team member k and brings lanes[k] lanes (its other
+// threads leave at once).  One launch has one block size, so this calls the
+// fold that wg_reduce runs between its barriers directly; a member's share
+// must not depend on how many lanes any member brings.
+struct FoldSharesArgs {
+  int *dst0;
+  const int *src0;
+  int64_t hop;
+  int np;
+  int nelems;
+  int lanes[detail::SyncPad::kMaxPes];
+};
+__global__ void fold_shares_kernel(FoldSharesArgs a) {
+  const int mine = a.lanes[blockIdx.x];
+  if (static_cast<int>(threadIdx.x) >= mine) return;
+  detail::fold_span_any<int, ROCSHMEM_SUM, false, true>(a.dst0, a.src0, a.hop, a.np, 0,
+                                                        static_cast<size_t>(a.nelems), threadIdx.x,
+                                                        mine, blockIdx.x, a.np);
 }
 
 // Sets n words to zero from the stream (a plain kernel: safe to record in a
@@ -257,7 +279,20 @@ void launch_grid_reduce(void *dst0, const void *src0, int64_t hop, int np, size_
   size_t lds = 0;
   if (np == 2 || np == 4 || np == 8) {
     const size_t waves_per_cu = (64 * 1024) / (static_cast<size_t>(np) * 1024);
-    if (waves_per_cu < 32) lds = (160 * 1024) / waves_per_cu - 512;
+    // An equal share of the CU's LDS per wavefront, whatever the part has
+    // (160 KiB on MI355X), less the 512 bytes the allocation granule may add.
+    static const size_t lds_per_cu = [] {
+      int dev = 0, bytes = 0;
+      if (hipGetDevice(&dev) != hipSuccess ||
+          hipDeviceGetAttribute(&bytes, hipDeviceAttributeMaxSharedMemoryPerMultiprocessor, dev) !=
+              hipSuccess || bytes <= 0) {
+        (void)hipGetLastError();
+        return size_t{0};
+      }
+      return static_cast<size_t>(bytes);
+    }();
+    if (waves_per_cu < 32 && lds_per_cu / waves_per_cu > 1024) lds = lds_per_cu / waves_per_cu - 512;
+    if (lds > (size_t{64} << 10)) lds = size_t{64} << 10;
   }
   a.span = static_cast<size_t>(wg) * (16 / sizeof(S));
   const size_t nspans = (n + a.span - 1) / a.span;
@@ -569,13 +604,16 @@ int rocshmem_amd_wg_reduce(int dtype, int op, rocshmem_amd_team_t team, void *de
   return status;
 }
 
-// Validates and enqueues the many-teams reduce; d_status: n_teams zeroed device
-// words.  0 = enqueued, -1 = refused (nothing enqueued).
+// Validates and enqueues the many-teams reduce; d_status: n_teams device words,
+// zeroed by the caller or, with clear_status, by a small kernel enqueued here
+// once every argument has been accepted.  0 = enqueued, -1 = refused (nothing
+// enqueued).
 static int enqueue_reduce_teams(int dtype, int op, const rocshmem_amd_team_t *teams, int n_teams,
-                                void *dest, const void *source, int nreduce, int wg_size,
-                                int iters, int *d_status, hipStream_t s) {
+                                void *dest, const void *source, int nreduce, int chunk_elems,
+                                int wg_size, int iters, int *d_status, bool clear_status,
+                                hipStream_t s) {
   if (!teams || n_teams < 1 || n_teams > kMaxTeamsPerLaunch || !valid_launch(1, wg_size) ||
-      nreduce < 0 || iters < 1)
+      nreduce < 0 || chunk_elems < 0 || iters < 1)
     return -1;
   TeamView first;
   if (!view_team(teams[0], &first)) return -1;
@@ -603,11 +641,13 @@ static int enqueue_reduce_teams(int dtype, int op, const rocshmem_amd_team_t *te
   a.pe_start = first.host->wrt_world.pe_start;
   a.stride = first.host->wrt_world.stride;
   a.nelems = nreduce;
-  // Equal slices, a whole number of 16-byte vectors each.
+  // Equal slices, a whole number of 16-byte vectors each: one per team, or of
+  // the size the caller asks for and then dealt out to the teams in turn.
   const int per_vec = static_cast<int>(16 / es);
-  int slice = (nreduce + n_teams - 1) / n_teams;
+  long slice = chunk_elems ? chunk_elems : (static_cast<long>(nreduce) + n_teams - 1) / n_teams;
   slice = (slice + per_vec - 1) / per_vec * per_vec;
-  a.slice_elems = slice > 0 ? slice : per_vec;
+  if (slice > nreduce) slice = (static_cast<long>(nreduce) + per_vec - 1) / per_vec * per_vec;
+  a.slice_elems = static_cast<int>(slice > 0 ? slice : per_vec);
   a.iters = iters;
   a.status = d_status;
   const dim3 grid(first.host->num_pes, n_teams), block(wg_size);
@@ -617,6 +657,8 @@ static int enqueue_reduce_teams(int dtype, int op, const rocshmem_amd_team_t *te
     if (!grid_fits(wg_reduce_teams_kernel<T, decltype(opc)::value>,
                    static_cast<long>(grid.x) * grid.y, wg_size))
       return;
+    // Everything has been checked: only now is anything put on the stream.
+    if (clear_status) hipLaunchKernelGGL(clear_words_kernel, dim3(1), dim3(256), 0, s, d_status, n_teams);
     hipLaunchKernelGGL((wg_reduce_teams_kernel<T, decltype(opc)::value>), grid, block, 0, s, a);
     launched = true;
   });
@@ -626,15 +668,15 @@ static int enqueue_reduce_teams(int dtype, int op, const rocshmem_amd_team_t *te
 }
 
 int rocshmem_amd_wg_reduce_teams(int dtype, int op, const rocshmem_amd_team_t *teams, int n_teams,
-                                 void *dest, const void *source, int nreduce, int wg_size,
-                                 int iters, rocshmem_amd_stream_t stream) {
+                                 void *dest, const void *source, int nreduce, int chunk_elems,
+                                 int wg_size, int iters, rocshmem_amd_stream_t stream) {
   if (n_teams < 1 || n_teams > kMaxTeamsPerLaunch) return -1;
   hipStream_t s = as_stream(stream);
   int *d_status;
   DRV_CHECK_HIP(hipMalloc(&d_status, sizeof(int) * n_teams));
   DRV_CHECK_HIP(hipMemsetAsync(d_status, 0, sizeof(int) * n_teams, s));
-  int status = enqueue_reduce_teams(dtype, op, teams, n_teams, dest, source, nreduce, wg_size,
-                                    iters, d_status, s);
+  int status = enqueue_reduce_teams(dtype, op, teams, n_teams, dest, source, nreduce, chunk_elems,
+                                    wg_size, iters, d_status, false, s);
   if (status == 0) {
     int seen[kMaxTeamsPerLaunch];
     DRV_CHECK_HIP(hipStreamSynchronize(s));
@@ -669,7 +711,8 @@ static int *static_status_words() {
 
 int rocshmem_amd_wg_reduce_teams_static(int dtype, int op, const rocshmem_amd_team_t *teams,
                                         int n_teams, void *dest, const void *source, int nreduce,
-                                        int wg_size, int iters, rocshmem_amd_stream_t stream) {
+                                        int chunk_elems, int wg_size, int iters,
+                                        rocshmem_amd_stream_t stream) {
   if (n_teams > kStaticStatusWords) {
     fprintf(stderr,
             "rocshmem: rocshmem_amd_wg_reduce_teams_static takes at most %d teams per call "
@@ -681,11 +724,10 @@ int rocshmem_amd_wg_reduce_teams_static(int dtype, int op, const rocshmem_amd_te
   int *words = static_status_words();
   if (!words) return -1;
   hipStream_t s = as_stream(stream);
-  // The array keeps what the last call left: clear the words this call uses.
-  hipLaunchKernelGGL(clear_words_kernel, dim3(1), dim3(256), 0, s, words, n_teams);
-  DRV_CHECK_HIP(hipGetLastError());
-  int status = enqueue_reduce_teams(dtype, op, teams, n_teams, dest, source, nreduce, wg_size,
-                                    iters, words, s);
+  // The array keeps what the last call left: the words this call uses are
+  // cleared on the stream, after the arguments have been checked.
+  int status = enqueue_reduce_teams(dtype, op, teams, n_teams, dest, source, nreduce, chunk_elems,
+                                    wg_size, iters, words, true, s);
   if (status == 0) {
     int seen[kStaticStatusWords];
     DRV_CHECK_HIP(hipStreamSynchronize(s));
@@ -693,6 +735,29 @@ int rocshmem_amd_wg_reduce_teams_static(int dtype, int op, const rocshmem_amd_te
     for (int t = 0; t < n_teams; ++t) status = seen[t] > status ? seen[t] : status;
   }
   return status;
+}
+
+int rocshmem_amd_fold_shares(void *dest, const void *source, int nreduce,
+                             const int *lanes_per_member, rocshmem_amd_stream_t stream) {
+  auto &r = runtime::rt();
+  if (!r.live || !lanes_per_member || nreduce < 0 || r.npes > detail::SyncPad::kMaxPes) return -1;
+  const size_t bytes = static_cast<size_t>(nreduce) * sizeof(int);
+  if (!sym_ok_on(dest, bytes, 0) || !sym_ok_on(source, bytes, 0)) return -1;
+  FoldSharesArgs a;
+  a.dst0 = static_cast<int *>(dest);
+  a.src0 = static_cast<const int *>(source);
+  a.hop = static_cast<int64_t>(r.pe_stride);
+  a.np = r.npes;
+  a.nelems = nreduce;
+  int widest = 0;
+  for (int k = 0; k < r.npes; ++k) {
+    if (lanes_per_member[k] < 1 || lanes_per_member[k] > 1024) return -1;
+    a.lanes[k] = lanes_per_member[k];
+    widest = lanes_per_member[k] > widest ? lanes_per_member[k] : widest;
+  }
+  hipLaunchKernelGGL(fold_shares_kernel, dim3(r.npes), dim3(widest), 0, as_stream(stream), a);
+  DRV_CHECK_HIP(hipGetLastError());
+  return 0;
 }
 
 int rocshmem_amd_wg_alltoall(int elem_size, rocshmem_amd_team_t team, void *dest,

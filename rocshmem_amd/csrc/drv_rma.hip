@@ -18,7 +18,14 @@ struct RmaArgs {
   rocshmem_ctx_t ctx;
   int pe;
   int iters;
+  uint32_t scatter_mask;  // 0: tile i sits at i * tile; else at ((i * odd) & mask) * tile
 };
+
+// Where message i of a scattered run lives: an odd multiplier is a bijection
+// on [0, 2^k), and neighbouring lanes land far apart.
+__device__ __forceinline__ size_t tile_slot(size_t i, uint32_t scatter_mask) {
+  return scatter_mask ? ((i * 0x9E3779B1ull) & scatter_mask) : i;
+}
 
 // One API call per tile; group g takes tiles g, g+G, ...
 template <int kOp, int kGran>
@@ -36,9 +43,10 @@ __global__ void rma_kernel(RmaArgs a) {
     group = blockIdx.x * bs + tid;
     groups = gridDim.x * bs;
   }
-  const size_t stride = groups * a.tile;
+  const size_t ntiles = (a.nbytes + a.tile - 1) / a.tile;
   for (int it = 0; it < a.iters; ++it) {
-    for (size_t off = group * a.tile; off < a.nbytes; off += stride) {
+    for (size_t i = group; i < ntiles; i += groups) {
+      const size_t off = tile_slot(i, a.scatter_mask) * a.tile;
       const size_t len = a.nbytes - off < a.tile ? a.nbytes - off : a.tile;
       if constexpr (kOp == ROCSHMEM_AMD_PUT) {
         if constexpr (kGran == ROCSHMEM_AMD_WG)
@@ -183,50 +191,19 @@ void launch_bulk(char *dst, const char *src, size_t nbytes, hipStream_t stream) 
   DRV_CHECK_HIP(hipGetLastError());
 }
 
-// What the memory system sustains in one direction only, with the copy
-// kernel's instructions (one 16-byte vector per lane, non-temporal load,
-// write-through streaming store): the yardstick the copy is read against.
-// 128 lanes per work-group is where both directions peak (6.9 TB/s each); at
-// 64 lanes a one-direction kernel is bound by work-group dispatch (4.7 TB/s).
-constexpr int kProbeThreads = 128;
-__global__ void probe_read_kernel(const char *src, size_t nvec, unsigned *sink) {
-  const size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (i >= nvec) return;
-  const detail::u32x4 a = detail::load16<true>(src + (i << 4));
-  const unsigned x = a.x ^ a.y ^ a.z ^ a.w;
-  if (x == 0x9e3779b9u && a.y == 0x7f4a7c15u) *sink = x;  // keeps the load alive; practically never taken
-}
-__global__ void probe_write_kernel(char *dst, size_t nvec) {
-  const size_t first = static_cast<size_t>(blockIdx.x) * blockDim.x;
-  const size_t i = first + threadIdx.x;
-  const size_t left = nvec - first;
-  const __amdgpu_buffer_rsrc_t w =
-      detail::window_of(dst + (first << 4), (left < blockDim.x ? left : blockDim.x) << 4);
-  const detail::u32x4 v = {1u, 2u, 3u, static_cast<unsigned>(i)};
-  if (i < nvec) detail::store16<true>(w, static_cast<uint32_t>(threadIdx.x << 4), v);
-}
-
-// What an agent-scope release (the L2 write-back behind quiet and fence on a
-// default context) costs in the middle of a copy: work-groups loop over tiles
-// with the cooperative copy and release never (mode 0), once at their end
-// (mode 1) or after every tile (mode 2).  The difference to mode 0, divided by
-// the number of releases, is the cost of one.
-template <int kMode>
-__global__ void release_probe_kernel(char *dst, const char *src, size_t n, size_t tile) {
-  const size_t ntiles = (n + tile - 1) / tile;
-  for (size_t t = blockIdx.x; t < ntiles; t += gridDim.x) {
-    const size_t off = t * tile;
-    const size_t len = n - off < tile ? n - off : tile;
-    detail::copy_lanes(dst + off, src + off, len, threadIdx.x, blockDim.x, 0);
-    if constexpr (kMode == 2) {
-      __syncthreads();
-      if (threadIdx.x == 0) detail::fence_release();
-    }
+// Number of 16-byte vectors (and tail bytes) in which two device buffers differ.
+__global__ void compare_kernel(const char *x, const char *y, size_t nbytes,
+                               unsigned long long *differing) {
+  const size_t nvec = nbytes >> 4;
+  const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+  unsigned long long bad = 0;
+  for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < nvec; i += stride) {
+    const detail::u32x4 a = detail::load16<false>(x + (i << 4)), b = detail::load16<false>(y + (i << 4));
+    bad += (a.x != b.x) | (a.y != b.y) | (a.z != b.z) | (a.w != b.w);
   }
-  if constexpr (kMode == 1) {
-    __syncthreads();
-    if (threadIdx.x == 0) detail::fence_release();
-  }
+  if (blockIdx.x == 0)
+    for (size_t k = (nvec << 4) + threadIdx.x; k < nbytes; k += blockDim.x) bad += x[k] != y[k];
+  if (bad) atomicAdd(differing, bad);
 }
 
 // The same byte range of every PE's slice set to one value: blockIdx.y is the PE.
@@ -260,6 +237,13 @@ extern "C" {
 int rocshmem_amd_rma(int rma_op, int gran, void *dest, const void *source, size_t nbytes,
                      size_t tile_bytes, int my_pe, int pe, int n_wgs, int wg_size,
                      int iters, rocshmem_amd_stream_t stream) {
+  return rocshmem_amd_rma_messages(rma_op, gran, dest, source, nbytes, tile_bytes, 0, my_pe, pe,
+                                   n_wgs, wg_size, iters, stream);
+}
+
+int rocshmem_amd_rma_messages(int rma_op, int gran, void *dest, const void *source, size_t nbytes,
+                              size_t tile_bytes, int scattered, int my_pe, int pe, int n_wgs,
+                              int wg_size, int iters, rocshmem_amd_stream_t stream) {
   if (!valid_pe(my_pe) || !valid_pe(pe) || !valid_launch(n_wgs, wg_size) || iters < 0)
     return -1;
   if (rma_op < ROCSHMEM_AMD_PUT || rma_op > ROCSHMEM_AMD_GET_NBI) return -1;
@@ -282,6 +266,16 @@ int rocshmem_amd_rma(int rma_op, int gran, void *dest, const void *source, size_
   a.ctx = runtime::rt().driver_ctx_handle(my_pe);
   a.pe = pe;
   a.iters = iters;
+  a.scatter_mask = 0;
+  if (scattered) {
+    // A permutation of the tiles: their number must be a power of two (up to
+    // 2^32) and the last tile whole.
+    const size_t ntiles = nbytes / a.tile;
+    if (!ntiles || ntiles * a.tile != nbytes || (ntiles & (ntiles - 1)) || ntiles > (size_t{1} << 32))
+      return -1;
+    a.scatter_mask = static_cast<uint32_t>(ntiles - 1);
+    if (ntiles == 1) a.scatter_mask = 0;
+  }
   hipStream_t s = as_stream(stream);
   const dim3 g(n_wgs), b(wg_size);
 #define RMA_CASE(OP, GR)                                                          \
@@ -338,40 +332,25 @@ int rocshmem_amd_flat_ids(int bx, int by, int bz, unsigned *out_host) {
   return 0;
 }
 
-int rocshmem_amd_hbm_probe(int write, void *buf, size_t nbytes, rocshmem_amd_stream_t stream) {
-  if (!runtime::rt().live || !buf || nbytes < (1u << 20) || (reinterpret_cast<uintptr_t>(buf) & 15u))
-    return -1;
-  if (!local_ok(buf, nbytes)) return -1;
-  static unsigned *sink = nullptr;  // never written in practice; allocated once
-  static std::once_flag sink_once;
-  std::call_once(sink_once, [] { DRV_CHECK_HIP(hipMalloc(&sink, sizeof(unsigned))); });
-  const size_t nvec = nbytes / 16;
-  const unsigned grid = static_cast<unsigned>((nvec + kProbeThreads - 1) / kProbeThreads);
-  if (write)
-    hipLaunchKernelGGL(probe_write_kernel, dim3(grid), dim3(kProbeThreads), 0, as_stream(stream),
-                       static_cast<char *>(buf), nvec);
-  else
-    hipLaunchKernelGGL(probe_read_kernel, dim3(grid), dim3(kProbeThreads), 0, as_stream(stream),
-                       static_cast<const char *>(buf), nvec, sink);
-  DRV_CHECK_HIP(hipGetLastError());
-  return 0;
-}
-
-int rocshmem_amd_release_probe(int mode, void *dst, const void *src, size_t nbytes,
-                               size_t tile_bytes, int n_wgs, int wg_size,
-                               rocshmem_amd_stream_t stream) {
-  if (!runtime::rt().live || !dst || !src || !nbytes || tile_bytes < 16 || mode < 0 || mode > 2 ||
-      !valid_launch(n_wgs, wg_size))
-    return -1;
-  if (!local_ok(dst, nbytes) || !local_ok(src, nbytes)) return -1;
-  const dim3 g(n_wgs), b(wg_size);
+int rocshmem_amd_compare(const void *x, const void *y, size_t nbytes, uint64_t *differing_out,
+                         rocshmem_amd_stream_t stream) {
+  if (!runtime::rt().live || !differing_out || !local_ok(x, nbytes) || !local_ok(y, nbytes)) return -1;
+  *differing_out = 0;
+  if (!nbytes) return 0;
+  static unsigned long long *d_count = nullptr;  // allocated once
+  static std::once_flag once;
+  std::call_once(once, [] { DRV_CHECK_HIP(hipMalloc(&d_count, sizeof(unsigned long long))); });
   hipStream_t s = as_stream(stream);
-  char *d = static_cast<char *>(dst);
-  const char *c = static_cast<const char *>(src);
-  if (mode == 0) hipLaunchKernelGGL(release_probe_kernel<0>, g, b, 0, s, d, c, nbytes, tile_bytes);
-  else if (mode == 1) hipLaunchKernelGGL(release_probe_kernel<1>, g, b, 0, s, d, c, nbytes, tile_bytes);
-  else hipLaunchKernelGGL(release_probe_kernel<2>, g, b, 0, s, d, c, nbytes, tile_bytes);
+  DRV_CHECK_HIP(hipMemsetAsync(d_count, 0, sizeof(unsigned long long), s));
+  const size_t want = (nbytes / 16 + 255) / 256;
+  hipLaunchKernelGGL(compare_kernel, dim3(static_cast<unsigned>(want < 8192 ? (want ? want : 1) : 8192)),
+                     dim3(256), 0, s, static_cast<const char *>(x), static_cast<const char *>(y),
+                     nbytes, d_count);
   DRV_CHECK_HIP(hipGetLastError());
+  DRV_CHECK_HIP(hipStreamSynchronize(s));
+  unsigned long long bad = 0;
+  DRV_CHECK_HIP(hipMemcpy(&bad, d_count, sizeof(bad), hipMemcpyDeviceToHost));
+  *differing_out = bad;
   return 0;
 }
 

@@ -282,7 +282,8 @@ struct PutFlagArgs {
   int rounds;
   int pe_a, pe_b;
   int with_signal;       // 0: putmem_wg, quiet, relaxed flag store; 1: putmem_signal_wg;
-                         // 2 / 3: putmem_nbi_wave / putmem_nbi pieces, quiet by all, flag
+                         // 2 / 3: putmem_nbi_wave / putmem_nbi pieces, quiet by all, flag;
+                         // 4 / 5: as 0 / 1 with the source in the producer's LDS
   unsigned spin_limit;
   rocshmem_ctx_t ctx_a;
   unsigned long long *mismatches;
@@ -325,7 +326,9 @@ __global__ void put_flag_kernel(PutFlagArgs a) {
   const bool producer = (blockIdx.x & 1) == 0;
   const size_t nwords = a.nbytes / 4;
   char *data = a.data_a + static_cast<size_t>(pair) * a.nbytes;
-  uint32_t *stage = a.staging + static_cast<size_t>(pair) * nwords;
+  extern __shared__ __attribute__((aligned(16))) uint32_t put_flag_lds[];
+  const bool from_lds = a.with_signal >= 4;
+  uint32_t *stage = from_lds ? put_flag_lds : a.staging + static_cast<size_t>(pair) * nwords;
   // Own-PE views of the two control words.
   uint64_t *flag_on_b = a.flag_b + pair;
   uint64_t *ack_on_a = a.ack_a + pair;
@@ -333,7 +336,7 @@ __global__ void put_flag_kernel(PutFlagArgs a) {
     if (producer) {
       for (size_t i = threadIdx.x; i < nwords; i += blockDim.x) stage[i] = put_flag_word(pair, r, i);
       __syncthreads();
-      if (a.with_signal == 1) {
+      if (a.with_signal == 1 || a.with_signal == 5) {
         // flag_on_b is pe_b's address; the call wants pe_a's.
         uint64_t *flag_sym = reinterpret_cast<uint64_t *>(reinterpret_cast<char *>(flag_on_b) - a.a_to_b);
         rocshmem_ctx_putmem_signal_wg(a.ctx_a, data, stage, a.nbytes, flag_sym,
@@ -807,12 +810,15 @@ int rocshmem_amd_put_flag_check(void *data, uint64_t *flags, size_t nbytes, int 
   auto &r = runtime::rt();
   if (!valid_pe(pe_a) || !valid_pe(pe_b) || pe_a == pe_b || pairs < 1 || pairs > 128 ||
       !valid_launch(2 * pairs, wg_size) || rounds < 0 || nbytes == 0 || (nbytes & 3) ||
-      with_signal < 0 || with_signal > 3)
+      with_signal < 0 || with_signal > 5)
     return -1;
+  // Modes 4 and 5 stage the message in the producer's LDS.
+  const size_t lds_bytes = with_signal >= 4 ? nbytes : 0;
+  if (lds_bytes > (size_t{64} << 10)) return -1;
   const size_t total = nbytes * static_cast<size_t>(pairs);
   if (!sym_ok_on(data, total, pe_a) || !sym_ok_on(flags, 16u * pairs, pe_a)) return -1;
   if (!mismatches_out || !timed_out_out) return -1;
-  if (!grid_fits(put_flag_kernel, 2L * pairs, wg_size)) return -1;
+  if (!grid_fits(put_flag_kernel, 2L * pairs, wg_size, lds_bytes)) return -1;
   const int64_t a_to_b = static_cast<int64_t>(pe_b - pe_a) * static_cast<int64_t>(r.pe_stride);
   uint32_t *staging;
   unsigned long long *d_bad;
@@ -841,7 +847,7 @@ int rocshmem_amd_put_flag_check(void *data, uint64_t *flags, size_t nbytes, int 
   a.ctx_a = r.driver_ctx_handle(pe_a);
   a.mismatches = d_bad;
   a.timed_out = d_timed_out;
-  hipLaunchKernelGGL(put_flag_kernel, dim3(2 * pairs), dim3(wg_size), 0, s, a);
+  hipLaunchKernelGGL(put_flag_kernel, dim3(2 * pairs), dim3(wg_size), lds_bytes, s, a);
   DRV_CHECK_HIP(hipGetLastError());
   DRV_CHECK_HIP(hipStreamSynchronize(s));
   unsigned long long bad = 0;

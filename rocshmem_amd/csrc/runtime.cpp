@@ -15,6 +15,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <map>
+#include <atomic>
 #include <mutex>
 #include <thread>
 #include <vector>
@@ -45,6 +46,17 @@ std::vector<detail::StateUploader> &uploaders() {
   static std::vector<detail::StateUploader> v;
   return v;
 }
+// Uploaders registered while the runtime is live (a library with device code
+// loaded after rocshmem_init): their first upload waits until the next call
+// into the runtime, because registration runs among the static initialisers of
+// the library being loaded, possibly before HIP has registered that library's
+// device code, when a copy to its symbols would fail.
+std::mutex g_uploader_lock;
+std::vector<detail::StateUploader> &late_uploaders() {
+  static std::vector<detail::StateUploader> v;
+  return v;
+}
+std::atomic<bool> g_late_uploaders{false};
 
 Runtime g_rt;
 int g_requested_npes = 0;
@@ -69,7 +81,21 @@ int ilog2(int x) {
 
 }  // namespace
 
-Runtime &rt() { return g_rt; }
+Runtime &rt() {
+  if (g_late_uploaders.load(std::memory_order_acquire)) {
+    std::vector<detail::StateUploader> todo;
+    {
+      std::lock_guard<std::mutex> guard(g_uploader_lock);
+      todo.swap(late_uploaders());
+      g_late_uploaders.store(false, std::memory_order_release);
+    }
+    if (g_rt.live && !todo.empty()) {
+      for (auto fn : todo) fn(&g_rt.state);
+      RT_CHECK_HIP(hipDeviceSynchronize());
+    }
+  }
+  return g_rt;
+}
 
 // ---- one thread per PE -------------------------------------------------------
 namespace {
@@ -187,25 +213,31 @@ void Runtime::write_team(int pool_index, int pe, const detail::TeamInfo &world,
 }
 
 // ---- the device allocation behind the symmetric heap ---------------------------
-// The heap is UNCACHED device memory (hipDeviceMallocUncached), as the
-// reference's is (src/memory/hip_allocator.hpp:58-65, heap_type.hpp:50).  The
-// L2 of an XCD then never holds a line of it, clean or dirty, and that is what
-// makes ordering cheap on this part: an agent-scope release is an L2 write-back
-// (buffer_wbl2), which on MI355X occupies the XCD's L2 for about 0.3 us
-// whenever the L2 holds lines that loads brought in — dirty or not — and for a
-// few ns when it holds none.  Measured, 256 MiB copied in 16 KiB tiles by 1024
-// work-groups of 256 with one release per tile: 760 us with a cached heap
-// (hipMalloc, or fine-grained), 156 us with an uncached one, 87 us without
-// releases; the copy itself runs at the same rate on either.  Stores to the
-// heap never sit dirty either, plain ones included, so quiet / fence / barriers
-// on a default context publish them at once.
+// The heap is UNCACHED device memory (hipDeviceMallocUncached).  That is this
+// library's choice, not the reference's: built for the IPC backend with
+// USE_COHERENT_HEAP, the reference takes HeapMemory<HIPAllocator>, plain
+// hipMalloc (src/memory/heap_type.hpp:41-51); its uncached allocator
+// (src/memory/hip_allocator.hpp:58-65) serves the other configurations.
+// With an uncached heap the L2 of an XCD never holds a line of it, clean or
+// dirty, and that is what makes ordering cheap on this part: an agent-scope
+// release is an L2 write-back (buffer_wbl2), which on MI355X occupies the
+// XCD's L2 for about 0.3 us whenever the L2 holds lines that loads brought in
+// — dirty or not — and for a few ns when it holds none.  Measured, 256 MiB
+// copied in 16 KiB tiles by 1024 work-groups of 256 with one release per tile:
+// 760 us with a cached heap (hipMalloc, or fine-grained), 156 us with an
+// uncached one, 87 us without releases; the copy itself runs at the same rate
+// on either.  Stores to the heap never sit dirty either, plain ones included.
+// The price: a kernel that reads symmetric data more than once (a GEMM over
+// received rows) gets no L2 reuse from the heap; ROCSHMEM_EMU_HEAP_CACHED=1
+// selects plain hipMalloc / hipFree for such programs.
 //
 // Uncached memory is never given back while the process lives: on this class
 // of machines memory allocated after such a release has shown wrong values.
 // rocshmem_finalize marks the block idle, and a later rocshmem_init reuses
 // the smallest idle block that is large enough before it allocates another.
-// ROCSHMEM_EMU_HEAP_CACHED=1 selects plain hipMalloc / hipFree instead
-// (measurements).
+// What the process holds that way is bounded by ROCSHMEM_EMU_HEAP_HELD_LIMIT
+// (bytes; default: the device memory), reported by heap_held() and, with
+// ROCSHMEM_EMU_VERBOSE=1, logged at every reuse and every new block.
 namespace {
 struct HeapBlock {
   char *base;
@@ -216,6 +248,15 @@ std::mutex g_heap_lock;
 std::vector<HeapBlock> g_heap_blocks;  // uncached blocks of this process, never freed
 
 bool heap_cached_mode() { return env_size("ROCSHMEM_EMU_HEAP_CACHED", 0) != 0; }
+bool verbose() { return env_size("ROCSHMEM_EMU_VERBOSE", 0) != 0; }
+
+void held_unlocked(size_t *total, size_t *idle) {
+  *total = *idle = 0;
+  for (const HeapBlock &b : g_heap_blocks) {
+    *total += b.bytes;
+    if (!b.in_use) *idle += b.bytes;
+  }
+}
 
 // An idle uncached block of at least `bytes`, or nullptr.
 char *reuse_heap_block(size_t bytes, size_t *block_bytes) {
@@ -226,16 +267,42 @@ char *reuse_heap_block(size_t bytes, size_t *block_bytes) {
   if (!best) return nullptr;
   best->in_use = true;
   *block_bytes = best->bytes;
+  if (verbose())
+    fprintf(stderr, "rocshmem: heap of %zu B reuses an idle uncached block of %zu B\n", bytes,
+            best->bytes);
   return best->base;
 }
 
 hipError_t new_heap_block(char **base, size_t bytes) {
   if (heap_cached_mode()) return hipMalloc(reinterpret_cast<void **>(base), bytes);
+  {
+    std::lock_guard<std::mutex> guard(g_heap_lock);
+    size_t total = 0, idle = 0, free_b = 0, device_b = 0;
+    held_unlocked(&total, &idle);
+    (void)hipMemGetInfo(&free_b, &device_b);
+    const size_t limit = env_size("ROCSHMEM_EMU_HEAP_HELD_LIMIT", device_b);
+    if (total + bytes > limit) {
+      fprintf(stderr,
+              "rocshmem: a new uncached heap block of %zu B is refused: this process already holds "
+              "%zu B of uncached heap blocks (%zu B of them idle, none large enough; they are kept "
+              "until the process ends), and the limit is %zu B (ROCSHMEM_EMU_HEAP_HELD_LIMIT)\n",
+              bytes, total, idle, limit);
+      return hipErrorOutOfMemory;
+    }
+  }
   const hipError_t e =
       hipExtMallocWithFlags(reinterpret_cast<void **>(base), bytes, hipDeviceMallocUncached);
   if (e == hipSuccess) {
     std::lock_guard<std::mutex> guard(g_heap_lock);
     g_heap_blocks.push_back(HeapBlock{*base, bytes, true});
+    if (verbose()) {
+      size_t total = 0, idle = 0;
+      held_unlocked(&total, &idle);
+      fprintf(stderr,
+              "rocshmem: new uncached heap block of %zu B; the process now holds %zu B in %zu "
+              "blocks (%zu B idle)\n",
+              bytes, total, g_heap_blocks.size(), idle);
+    }
   }
   return e;
 }
@@ -252,6 +319,11 @@ void release_heap_block(char *base) {
   RT_CHECK_HIP(hipFree(base));  // a cached-mode block
 }
 }  // namespace
+
+void heap_held(size_t *total, size_t *idle) {
+  std::lock_guard<std::mutex> guard(g_heap_lock);
+  held_unlocked(total, idle);
+}
 
 int Runtime::init(int want_npes, size_t want_heap) {
   if (live) return 0;
@@ -349,7 +421,8 @@ int Runtime::init(int want_npes, size_t want_heap) {
     exit(EXIT_FAILURE);
   }
   heap_alloc_bytes = alloc_bytes;
-  if (env_size("ROCSHMEM_EMU_VERBOSE", 0) != 0)
+  heap_uncached = !heap_cached_mode();
+  if (verbose())
     fprintf(stderr, "rocshmem: %d PEs, heap %zu B per PE, slices %zu B apart, %zu B allocated%s%s\n",
             npes, heap_size, pe_stride, alloc_bytes, anchored ? " (placed)" : "",
             heap_cached_mode() ? " (cached)" : " (uncached)");
@@ -638,8 +711,12 @@ void Runtime::set_pe_rule(int rule) {
 
 namespace detail {
 void register_state_uploader(StateUploader fn) {
+  std::lock_guard<std::mutex> guard(runtime::g_uploader_lock);
   runtime::uploaders().push_back(fn);
-  if (runtime::rt().live) fn(&runtime::rt().state);
+  if (runtime::g_rt.live) {
+    runtime::late_uploaders().push_back(fn);
+    runtime::g_late_uploaders.store(true, std::memory_order_release);
+  }
 }
 }  // namespace detail
 

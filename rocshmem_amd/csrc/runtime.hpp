@@ -31,6 +31,7 @@ struct Runtime {
   size_t pe_stride = 0;
   size_t ws_stride = 0;
   size_t heap_alloc_bytes = 0;  // size of the device allocation that holds the slices
+  bool heap_uncached = true;    // false under ROCSHMEM_EMU_HEAP_CACHED=1
   char *heap_base = nullptr;
   char *d_ws = nullptr;
   detail::Team *d_teams = nullptr;         // [max_teams][npes]
@@ -106,6 +107,10 @@ struct Runtime {
 };
 
 Runtime &rt();
+
+// Uncached heap blocks this process holds (they are kept until it ends): all
+// of them, and those no live runtime uses.
+void heap_held(size_t *total, size_t *idle);
 
 // ---- one thread per PE (rocshmem_emu_run_pes) --------------------------------
 // Collective host calls made by PE threads meet here.  The callers are the

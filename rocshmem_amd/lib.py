@@ -40,6 +40,8 @@ SIGNATURES = {
     "rocshmem_amd_heap_avail": (_sz, []),
     "rocshmem_amd_pe_stride": (_sz, []),
     "rocshmem_amd_heap_alloc_bytes": (_sz, []),
+    "rocshmem_amd_heap_is_uncached": (_i, []),
+    "rocshmem_amd_heap_held": (_i, [C.POINTER(_sz), C.POINTER(_sz)]),
     "rocshmem_amd_coresident": (_i, [C.c_long, _i, _i]),
     "rocshmem_amd_hw_queues_suffice": (_i, [_sz, _sz]),
     "rocshmem_amd_heap_model_create": (_vp, [_u64, _u64]),
@@ -65,8 +67,7 @@ SIGNATURES = {
     "rocshmem_amd_copy_in": (_i, [_vp, _vp, _sz]),
     "rocshmem_amd_copy_out": (_i, [_vp, _vp, _sz]),
     "rocshmem_amd_fill": (_i, [_vp, _i, _sz]),
-    "rocshmem_amd_hbm_probe": (_i, [_i, _vp, _sz, _vp]),
-    "rocshmem_amd_release_probe": (_i, [_i, _vp, _vp, _sz, _sz, _i, _i, _vp]),
+    "rocshmem_amd_compare": (_i, [_vp, _vp, _sz, C.POINTER(_u64), _vp]),
     "rocshmem_amd_fill_every_pe": (_i, [_vp, _i, _sz, _vp]),
     "rocshmem_amd_copy_dev": (_i, [_vp, _vp, _sz]),
     "rocshmem_amd_stream_sync": (_i, [_vp]),
@@ -76,6 +77,7 @@ SIGNATURES = {
     "rocshmem_amd_timer_elapsed_ms": (C.c_float, [_vp]),
     "rocshmem_amd_timer_destroy": (_i, [_vp]),
     "rocshmem_amd_rma": (_i, [_i, _i, _vp, _vp, _sz, _sz, _i, _i, _i, _i, _i, _vp]),
+    "rocshmem_amd_rma_messages": (_i, [_i, _i, _vp, _vp, _sz, _sz, _i, _i, _i, _i, _i, _i, _vp]),
     "rocshmem_amd_rma_staged": (_i, [_i, _vp, _vp, _vp, _sz, _i, _i, _i, _vp]),
     "rocshmem_amd_flat_ids": (_i, [_i, _i, _i, _vp]),
     "rocshmem_amd_ctx_pe": (_i, [_vp]),
@@ -92,9 +94,10 @@ SIGNATURES = {
     "rocshmem_amd_getmem": (_i, [_vp, _vp, _sz, _i, _i, _vp]),
     "rocshmem_amd_wf_coalesce": (_i, [_vp, _vp, _vp, _vp, _u64, _vp, _vp]),
     "rocshmem_amd_wg_reduce": (_i, [_i, _i, _vp, _vp, _vp, _i, _i, _vp]),
-    "rocshmem_amd_wg_reduce_teams": (_i, [_i, _i, C.POINTER(_vp), _i, _vp, _vp, _i, _i, _i, _vp]),
+    "rocshmem_amd_wg_reduce_teams": (_i, [_i, _i, C.POINTER(_vp), _i, _vp, _vp, _i, _i, _i, _i, _vp]),
     "rocshmem_amd_wg_reduce_teams_static": (_i, [_i, _i, C.POINTER(_vp), _i, _vp, _vp, _i, _i, _i,
-                                                 _vp]),
+                                                 _i, _vp]),
+    "rocshmem_amd_fold_shares": (_i, [_vp, _vp, _i, C.POINTER(_i), _vp]),
     "rocshmem_amd_wg_alltoall": (_i, [_i, _vp, _vp, _vp, _i, _i, _vp]),
     "rocshmem_amd_wg_broadcast": (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "rocshmem_amd_wg_fcollect": (_i, [_i, _vp, _vp, _vp, _i, _i, _vp]),
@@ -118,18 +121,28 @@ SIGNATURES = {
 }
 
 
+# The benchmark's measuring probes (include/rocshmem_amd_probes.h), a library of
+# their own next to the product.
+PROBES_PATH = os.path.join(_HERE, "lib", "librocshmem_amd_probes.so")
+PROBE_SIGNATURES = {
+    "rocshmem_amd_hbm_probe": (_i, [_i, _vp, _sz, _vp]),
+    "rocshmem_amd_release_probe": (_i, [_i, _vp, _vp, _sz, _sz, _i, _i, _vp]),
+    "rocshmem_amd_reuse_probe": (_i, [_vp, _sz, _sz, _i, _i, _i, _vp]),
+}
+
+
 class Library:
     """The loaded shared library with typed entry points as attributes
     (``lib.malloc`` is ``rocshmem_amd_malloc`` and so on)."""
 
-    def __init__(self, path=LIB_PATH):
+    def __init__(self, path=LIB_PATH, signatures=None):
         if not os.path.exists(path):
             raise RuntimeError(
                 f"{path} is not built; run `make -C rocshmem_amd/csrc` "
                 "(or __graft_entry__.build()). There is no CPU fallback.")
         self.path = path
         self.cdll = C.CDLL(path, mode=C.RTLD_GLOBAL)
-        for name, (res, args) in SIGNATURES.items():
+        for name, (res, args) in (SIGNATURES if signatures is None else signatures).items():
             fn = getattr(self.cdll, name)
             fn.restype = res
             fn.argtypes = args
@@ -144,3 +157,16 @@ def load():
     if _LIB is None:
         _LIB = Library()
     return _LIB
+
+
+_PROBES = None
+
+
+def load_probes():
+    """The measuring probes; loads the product library first (they run on its
+    runtime)."""
+    global _PROBES
+    load()
+    if _PROBES is None:
+        _PROBES = Library(PROBES_PATH, PROBE_SIGNATURES)
+    return _PROBES

@@ -12,11 +12,12 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, "include", "rocshmem_amd.h")
+PROBES_HEADER = os.path.join(ROOT, "include", "rocshmem_amd_probes.h")
 REFERENCE = "/root/reference"
 
 
-def declared_symbols():
-    text = open(HEADER).read()
+def declared_symbols(header=HEADER):
+    text = open(header).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(rocshmem_amd_\w+)\s*\(", text)))
 
@@ -37,6 +38,18 @@ def test_library_exports_every_declared_symbol(L):
 
 def test_python_binding_matches_header(L):
     assert sorted(L.SIGNATURES) == declared_symbols()
+
+
+def test_measuring_probes_live_in_a_library_of_their_own(L):
+    """The benchmark's yardsticks are declared in their own header, exported by
+    their own library and by nothing in the product's."""
+    names = declared_symbols(PROBES_HEADER)
+    assert sorted(L.PROBE_SIGNATURES) == names and names
+    probes = ctypes.CDLL(L.PROBES_PATH)
+    assert not [n for n in names if not hasattr(probes, n)]
+    product = ctypes.CDLL(L.LIB_PATH)
+    assert not [n for n in names if hasattr(product, n)]
+    assert not set(names) & set(declared_symbols())
 
 
 def test_calls_before_init_fail_cleanly(L):

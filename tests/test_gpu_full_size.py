@@ -1,5 +1,5 @@
-"""The two workloads of the benchmark that are otherwise only timed, at their
-full size and checked: the put_signal dispatch (4096 tokens per PE, rows of
+"""The workloads of the benchmark that are otherwise only timed, at their
+full size and checked: the headline put in its exact launch, the put_signal dispatch (4096 tokens per PE, rows of
 7168 bf16, top-8-of-256 Zipf(1.1) routing) and 16 Mi int64 fetch_add onto 4096
 counters.  Through the C entry points, default and NOSTORE contexts."""
 import ctypes
@@ -18,6 +18,53 @@ MiB = 1 << 20
 @pytest.fixture(params=[0, 1], ids=["default_ctx", "nostore_ctx"])
 def ctx_kind(request):
     return request.param
+
+
+def test_headline_launch_moves_every_byte(rt, L, orc, ctx_kind, monkeypatch):
+    """The benchmark's headline launch exactly: a 256 MiB message between two of
+    8 slices in the spread layout (ROCSHMEM_EMU_SPREAD=1, 8 GiB per PE), one
+    rocshmem_ctx_putmem_wg of a 4 KiB tile per work-group of 128 (65536
+    work-groups), one quiet per work-group, on a ROCSHMEM_CTX_NOSTORE context
+    and on a default one (src/ipc/context_ipc_device.cpp:109-125).  All 256 MiB
+    and the bytes either side compared with the source on the host, and once
+    more on the device with the compare the benchmark uses; a flipped byte is
+    found by that compare."""
+    monkeypatch.setenv("ROCSHMEM_EMU_SPREAD", "1")
+    rt.down()
+    l = rt.up(P, 8 << 30)
+    assert l.pe_stride() >= 16 << 30
+    n, tile, wg = 256 * MiB, 4096, 128
+    src, dst = l.malloc(n), l.malloc(n + 4096)
+    assert src and dst
+    me, pe = 3, 4
+    T = 4 * MiB
+    host_tile = orc.fill_u8(T, 21, me)
+    base = l.pe_ptr(src, me)
+    rt.put_bytes(base, host_tile)
+    done = T
+    while done < n:
+        assert l.putmem(base + done, base, done, me, me, None) == 0
+        done *= 2
+    l.fill(l.pe_ptr(dst, pe), 0x5A, n + 4096)
+    before = l.set_ctx_options(ctx_kind)
+    rc = l.rma(L.PUT, L.WG, l.pe_ptr(dst, me), l.pe_ptr(src, me), n, tile, me, pe, n // tile, wg, 1, None)
+    l.set_ctx_options(before)
+    assert rc == 0
+    l.stream_sync(None)
+    got = rt.get_bytes(l.pe_ptr(dst, pe), n + 4096)
+    assert np.array_equal(got[:n].reshape(-1, T), np.broadcast_to(host_tile, (n // T, T)))
+    assert (got[n:] == 0x5A).all()
+    del got
+    differing = ctypes.c_uint64(99)
+    assert l.compare(l.pe_ptr(dst, pe), l.pe_ptr(src, me), n, ctypes.byref(differing), None) == 0
+    assert differing.value == 0
+    for at in (123456789, n - 1):
+        l.fill(l.pe_ptr(dst, pe) + at, int(host_tile[at % T]) ^ 0xFF, 1)
+    assert l.compare(l.pe_ptr(dst, pe), l.pe_ptr(src, me), n, ctypes.byref(differing), None) == 0
+    assert differing.value == 2
+    l.free(src)
+    l.free(dst)
+    rt.down()
 
 
 def test_dispatch_put_signal_full_size(rt, L, orc, ctx_kind):

@@ -39,11 +39,11 @@ def test_reduce_grid_that_cannot_be_resident_is_refused_and_launches_nothing(rt,
         rt.put_bytes(l.pe_ptr(src, p), ones)
         l.fill(l.pe_ptr(dst, p), 0x5A, n * 4)
     for entry in (l.wg_reduce_teams, l.wg_reduce_teams_static):
-        assert entry(L.INT, L.SUM, teams, n_teams, dst, src, n, 1024, 1, None) == -1
+        assert entry(L.INT, L.SUM, teams, n_teams, dst, src, n, 0, 1024, 1, None) == -1
     l.stream_sync(None)
     for p in range(P):
         assert (rt.get_bytes(l.pe_ptr(dst, p), n * 4) == 0x5A).all()
-    assert l.wg_reduce_teams(L.INT, L.SUM, teams, 16, dst, src, n, 256, 1, None) == 0
+    assert l.wg_reduce_teams(L.INT, L.SUM, teams, 16, dst, src, n, 0, 256, 1, None) == 0
     for p in range(P):
         assert (rt.get_bytes(l.pe_ptr(dst, p), n * 4, np.int32) == P).all()
     # the other drivers whose work-groups wait for each other share the rule

@@ -190,22 +190,27 @@ def test_many_teams_reduce_their_slices_at_once(rt, L, orc, n_teams):
                 l.fill(l.pe_ptr(b.dst, p), 0x5A, (n + 8) * es)
             for k, p in enumerate(pes):
                 rt.put_bytes(l.pe_ptr(b.src, p), srcs[k])
-            assert l.wg_reduce_teams(getattr(L, dtype_name), getattr(L, op_name), teams, n_teams,
-                                     l.pe_ptr(b.dst, pes[0]), l.pe_ptr(b.src, pes[0]), n, 256, 1, None) == 0
             want = orc.to_all(getattr(orc, dtype_name), getattr(orc, op_name), srcs)
-            for p in range(8):
-                got = rt.get_bytes(l.pe_ptr(b.dst, p), (n + 8) * es, np_t)
-                if p in pes:
-                    assert np.array_equal(got[:n].view(np.uint8), want.view(np.uint8)), (dtype_name, n, p)
-                    assert (got[n:].view(np.uint8) == 0x5A).all()
-                else:
-                    assert (got.view(np.uint8) == 0x5A).all()
+            # one slice per team, then slices of `chunk` elements dealt out in turn
+            # (a chunk that is no whole number of vectors, one larger than the array)
+            for chunk in (0, 1000, 4 * n):
+                assert l.wg_reduce_teams(getattr(L, dtype_name), getattr(L, op_name), teams, n_teams,
+                                         l.pe_ptr(b.dst, pes[0]), l.pe_ptr(b.src, pes[0]), n, chunk, 256, 1,
+                                         None) == 0
+                for p in range(8):
+                    got = rt.get_bytes(l.pe_ptr(b.dst, p), (n + 8) * es, np_t)
+                    if p in pes:
+                        assert np.array_equal(got[:n].view(np.uint8), want.view(np.uint8)), (dtype_name, n, p, chunk)
+                        assert (got[n:].view(np.uint8) == 0x5A).all()
+                    else:
+                        assert (got.view(np.uint8) == 0x5A).all()
+                    l.fill(l.pe_ptr(b.dst, p), 0x5A, (n + 8) * es)
             b.free()
         # the same team twice, or teams over different PEs, are refused
         if n_teams >= 2:
             twice = (ctypes.c_void_p * 2)(teams[0], teams[0])
             assert l.wg_reduce_teams(L.INT, L.SUM, twice, 2, l.pe_ptr(b.src, pes[0]), l.pe_ptr(b.src, pes[0]),
-                                     0, 64, 1, None) == -1
+                                     0, 0, 64, 1, None) == -1
         for t in range(n_teams):
             l.team_destroy(teams[t])
     l.set_pe(0)
@@ -255,14 +260,59 @@ def test_config1_int32_sum_two_pes_one_mi(rt, L, orc):
     rt.up(8, HEAP)
 
 
-def test_team_too_large_for_reduce_is_an_error(rt, L, orc):
-    """2*P > ROCSHMEM_REDUCE_SYNC_SIZE -> ROCSHMEM_ERROR
-    (src/ipc/context_ipc_tmpl_device.hpp:412-415)."""
-    l = rt.up(130, 2 << 20)
-    buf = l.malloc(1024)
-    l.fill(buf, 0, 1024)
-    assert l.wg_reduce(L.INT, L.SUM, l.team_world(), buf, buf, 16, 64, None) == 1
-    l.free(buf)
+@pytest.mark.parametrize("P,nreduce", [(130, 4), (130, 7), (130, 8), (130, 16), (256, 4), (256, 5),
+                                       (128, 16), (128, 20000)])
+def test_team_too_large_for_reduce_follows_the_reference_selector(rt, L, orc, P, nreduce):
+    """A team with 2*P > ROCSHMEM_REDUCE_SYNC_SIZE is refused only when the
+    reference's direct path does not fit either (P * nreduce elements against
+    max(nreduce/2 + 1, 1024)): src/ipc/context_ipc_tmpl_device.hpp:361-418.
+    Status against the oracle's restatement of that selector; data, where the
+    call is accepted, against the ascending fold; a refused call leaves the
+    destination alone."""
+    l = rt.up(P, 2 << 20)
+    plan = orc.reduce_plan(P, nreduce)
+    b = Buffers(rt, l, nreduce * 4)
+    srcs = make_inputs(orc, "INT", P, nreduce, 11)
+    for p in range(P):
+        rt.put_bytes(l.pe_ptr(b.src, p), srcs[p])
+        l.fill(l.pe_ptr(b.dst, p), 0x5A, nreduce * 4)
+    rc = l.wg_reduce(L.INT, L.SUM, l.team_world(), b.dst, b.src, nreduce, 64, None)
+    assert rc == plan["status"], (P, nreduce, plan)
+    want = orc.to_all(orc.INT, orc.SUM, srcs)
+    for p in (0, 1, P // 2, P - 1):
+        got = rt.get_bytes(l.pe_ptr(b.dst, p), nreduce * 4, np.int32)
+        if rc == 0:
+            assert np.array_equal(got, want), (P, nreduce, p)
+        else:
+            assert (got.view(np.uint8) == 0x5A).all(), (P, nreduce, p)
+    b.free()
+    rt.up(8, HEAP)
+
+
+@pytest.mark.parametrize("P,lanes", [(3, [64, 192, 1024]), (8, [1024, 64, 256, 192, 1, 640, 128, 65]),
+                                     (2, [100, 1000]), (5, [7, 1024, 64, 64, 333])])
+@pytest.mark.parametrize("n", [5, 4099, 300007])
+def test_member_shares_do_not_depend_on_work_group_sizes(rt, L, orc, P, lanes, n):
+    """Team members may run work-groups of different sizes (they are separate
+    work-groups, possibly separate kernels): the split of the index range among
+    them must tile it all the same.  Each member's share computed with its own
+    lane count; every element of every destination against the oracle."""
+    import ctypes
+    l = rt.up(P, 64 << 20)
+    b = Buffers(rt, l, (n + 8) * 4)
+    srcs = make_inputs(orc, "INT", P, n, 5)
+    for p in range(P):
+        rt.put_bytes(l.pe_ptr(b.src, p), srcs[p])
+        l.fill(l.pe_ptr(b.dst, p), 0x5A, (n + 8) * 4)
+    arr = (ctypes.c_int * P)(*lanes)
+    assert l.fold_shares(l.pe_ptr(b.dst, 0), l.pe_ptr(b.src, 0), n, arr, None) == 0
+    l.stream_sync(None)
+    want = orc.to_all(orc.INT, orc.SUM, srcs)
+    for p in range(P):
+        got = rt.get_bytes(l.pe_ptr(b.dst, p), (n + 8) * 4, np.int32)
+        assert np.array_equal(got[:n], want), (P, lanes, n, p)
+        assert (got[n:].view(np.uint8) == 0x5A).all()
+    b.free()
     rt.up(8, HEAP)
 
 

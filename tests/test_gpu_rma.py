@@ -176,6 +176,53 @@ def test_put_quiet_flag_seen_in_order(rt, L, env, ctx_options, with_signal, nbyt
     l.free(flags)
 
 
+@pytest.mark.parametrize("with_signal", [4, 5])
+@pytest.mark.parametrize("ctx_options", [0, 1])
+@pytest.mark.parametrize("nbytes,pairs,wg", [(4096, 1, 64), (65536, 16, 256), (16384 + 4, 128, 1024)])
+def test_put_from_lds_then_flag_seen_in_order(rt, L, env, ctx_options, with_signal, nbytes, pairs, wg):
+    """The same message passing with the producer's source in its LDS: the copy
+    then takes the path for local buffers that global loads cannot reach, and
+    its stores to the destination must be complete before the flag (quiet on
+    either kind of context, or the signal of putmem_signal_wg) like any other
+    put's."""
+    test_put_quiet_flag_seen_in_order(rt, L, env, ctx_options, with_signal, nbytes, pairs, wg)
+
+
+@pytest.mark.parametrize("gran", GRANS)
+@pytest.mark.parametrize("op", ["PUT", "GET", "PUT_NBI"])
+@pytest.mark.parametrize("ctx_options", [0, 1])
+def test_scattered_messages(rt, L, orc, env, op, gran, ctx_options):
+    """Many small messages whose neighbours in the wavefront are far apart
+    (every message visited once through a permutation of the slots), and the
+    same messages with lanes that continue one another: the destination is the
+    source either way, byte for byte, guards untouched."""
+    l = env["l"]
+    src, dst, host = env["src"], env["dst"], env["host"]
+    o, g = getattr(L, op), getattr(L, gran)
+    for msg, count in [(8, 1 << 14), (64, 1 << 12), (24, 1 << 10), (4096, 64), (1, 256)]:
+        n = msg * count
+        for scattered in (1, 0):
+            landing = l.pe_ptr(dst, 1) + GUARD
+            l.fill(landing - GUARD, 0xA5, n + 2 * GUARD)
+            before = l.set_ctx_options(ctx_options)
+            if o == L.GET:
+                rt.put_bytes(l.pe_ptr(src, 1), host[:n])
+                rc = l.rma_messages(o, g, l.pe_ptr(dst, 1) + GUARD, l.pe_ptr(src, 0), n, msg, scattered, 0,
+                                    1, 8, 128, 1, None)
+            else:
+                rc = l.rma_messages(o, g, l.pe_ptr(dst, 0) + GUARD, l.pe_ptr(src, 0), n, msg, scattered, 0,
+                                    1, 8, 128, 1, None)
+            l.set_ctx_options(before)
+            assert rc == 0
+            l.stream_sync(None)
+            got = rt.get_bytes(landing - GUARD, n + 2 * GUARD)
+            assert np.array_equal(got[GUARD:GUARD + n], host[:n]), (op, gran, msg, count, scattered)
+            assert (got[:GUARD] == 0xA5).all() and (got[GUARD + n:] == 0xA5).all()
+    # a number of tiles that is no power of two cannot be permuted this way
+    assert l.rma_messages(o, g, l.pe_ptr(dst, 0), l.pe_ptr(src, 0), 24 * 1000, 24, 1, 0, 1, 8, 128, 1,
+                          None) == -1
+
+
 def test_every_pe_pair(rt, L, orc, env):
     for me in range(P):
         for pe in range(P):
@@ -222,13 +269,16 @@ def test_hbm_probe_reads_and_writes_only_what_it_is_given(rt, L):
     fills the buffer with (1, 2, 3, vector index) and stays inside it, the
     read probe changes nothing."""
     l = rt.up(P, HEAP)
+    pr = L.load_probes()
     n = 4 << 20
     buf = l.malloc(n + 4096)
     l.fill(buf, 0x6B, n + 4096)
-    assert l.hbm_probe(0, buf, n, None) == 0
+    assert pr.hbm_probe(0, buf, n, None) == 0
+    assert pr.reuse_probe(buf, n, 65536, 3, 64, 256, None) == 0
     l.stream_sync(None)
     assert (rt.get_bytes(buf, n + 4096) == 0x6B).all()
-    assert l.hbm_probe(1, buf, n, None) == 0
+    assert pr.reuse_probe(buf, n, 100, 3, 64, 256, None) == -1  # tiles are whole vectors
+    assert pr.hbm_probe(1, buf, n, None) == 0
     l.stream_sync(None)
     got = rt.get_bytes(buf, n + 4096, np.uint32)
     body = got[:n // 4].reshape(-1, 4)
@@ -236,9 +286,9 @@ def test_hbm_probe_reads_and_writes_only_what_it_is_given(rt, L):
     assert np.array_equal(body, np.stack([np.ones_like(idx), 2 * np.ones_like(idx),
                                           3 * np.ones_like(idx), idx], 1))
     assert (got[n // 4:].view(np.uint8) == 0x6B).all()   # nothing past the end
-    assert l.hbm_probe(0, buf + 4, n, None) == -1         # misaligned
-    assert l.hbm_probe(1, buf, 1024, None) == -1          # too small to mean anything
-    assert l.hbm_probe(1, None, n, None) == -1
+    assert pr.hbm_probe(0, buf + 4, n, None) == -1         # misaligned
+    assert pr.hbm_probe(1, buf, 1024, None) == -1          # too small to mean anything
+    assert pr.hbm_probe(1, None, n, None) == -1
     l.free(buf)
 
 
