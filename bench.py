@@ -333,13 +333,19 @@ def message_rates(b, steps):
         n_wgs = max(256, min(8192, count // groups_per_wg))
         for scattered in (0, 1):
             for cname, opt in CTX_KINDS:
-                l.set_ctx_options(opt)
-                ms = b.time_ms(lambda: l.rma_messages(L.PUT, gran, l.pe_ptr(dst, 0), l.pe_ptr(src, 0),
-                                                      count * msg, msg, scattered, 0, 1, n_wgs, 256, 1, None),
-                               max(3, steps // 10), 1)
-                key = "%s_%dB_%s_%s" % (gname, msg, "scattered" if scattered else "contiguous", cname)
-                res[key] = {"ms": round(ms, 4), "msgs": count, "mmsg_per_s": round(count / ms / 1e3, 1),
-                            "gbs": round(2 * count * msg / ms / 1e6, 1)}
+                # thread-level puts also with the coalescing front end, which looks
+                # for one run across the wavefront before every call
+                for coalesce in ((0, 1) if gran == L.THREAD else (0,)):
+                    l.set_ctx_options(opt)
+                    l.set_coalesce_puts(coalesce)
+                    ms = b.time_ms(lambda: l.rma_messages(L.PUT, gran, l.pe_ptr(dst, 0), l.pe_ptr(src, 0),
+                                                          count * msg, msg, scattered, 0, 1, n_wgs, 256, 1,
+                                                          None), max(3, steps // 10), 1)
+                    key = "%s_%dB_%s_%s%s" % (gname, msg, "scattered" if scattered else "contiguous", cname,
+                                              "_coalescing" if coalesce else "")
+                    res[key] = {"ms": round(ms, 4), "msgs": count, "mmsg_per_s": round(count / ms / 1e3, 1),
+                                "gbs": round(2 * count * msg / ms / 1e6, 1)}
+    l.set_coalesce_puts(0)
     l.set_ctx_options(0)
     l.free(src)
     l.free(dst)
@@ -348,8 +354,11 @@ def message_rates(b, steps):
 
 def reuse_config(b, steps):
     """What a consumer that re-reads symmetric data gets from the caches: a
-    256 MiB symmetric buffer read four times, tile by tile (256 KiB tiles, each
-    read four times in a row by its work-group), against one pass."""
+    256 MiB symmetric buffer read four times, tile by tile (8 KiB tiles, each
+    read four times in a row by its work-group), against one pass.  The tiles
+    of the work-groups resident on an XCD together fit its 4 MiB L2 (256
+    work-groups of 256 lanes, 8 KiB each), so on cached memory the later passes
+    are L2 hits."""
     l = b.l
     n = 256 * MiB
     buf = l.malloc(n)
@@ -357,7 +366,7 @@ def reuse_config(b, steps):
     b.fill_random(buf, n, 0, 91)
     res = {}
     for passes in (1, 4):
-        ms = b.time_ms(lambda: b.probes.reuse_probe(buf, n, 256 << 10, passes, 1024, 256, None),
+        ms = b.time_ms(lambda: b.probes.reuse_probe(buf, n, 8 << 10, passes, 2048, 256, None),
                        max(5, steps // 4), 2)
         res["read_x%d_gbs" % passes] = round(passes * n / ms / 1e6, 1)
     l.free(buf)

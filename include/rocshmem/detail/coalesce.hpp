@@ -11,9 +11,9 @@
 // instead of ds_bpermute-based shuffles, and the run length comes from the
 // ballot of absorbed lanes.
 //
-// On the load/store path this is a utility, not part of putmem: merging 64
-// four-byte stores of one instruction into one lane's serial copy would slow
-// them down.  It pays where a message has a fixed cost (a NIC work request).
+// Merging a run into the lowest lane's serial copy would slow a load/store
+// path down; what the thread-level put does with a run instead is move it with
+// the whole wavefront (detail/rma.hpp::put_as_one_run).
 #ifndef ROCSHMEM_AMD_DETAIL_COALESCE_HPP_
 #define ROCSHMEM_AMD_DETAIL_COALESCE_HPP_
 

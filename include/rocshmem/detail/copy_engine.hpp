@@ -261,6 +261,9 @@ __device__ __forceinline__ void copy_lanes(void *dst, const void *src, size_t n,
 // One lane copies n bytes on its own: 16-byte moves, then 8/4/2/1.  A lone
 // lane is bound by memory latency, so large messages keep eight loads in
 // flight (measured: 1 MiB from one thread in 7 ms with one load at a time).
+// Plain loads and stores through generic pointers: either side may be LDS or
+// a stack variable.  Used where the destination is the caller's own buffer
+// (gets); a put goes through copy_thread_through.
 __device__ __forceinline__ void copy_thread(void *dst, const void *src,
                                             size_t n) {
   char *d = static_cast<char *>(dst);
@@ -290,6 +293,88 @@ __device__ __forceinline__ void copy_thread(void *dst, const void *src,
     d += 2; s += 2;
   }
   if (n & 1) *d = *s;
+}
+
+// ---- write-through stores of a single lane -----------------------------------
+// A lane's own stores cannot be buffer stores (the resource is wave-uniform,
+// the lanes of a thread-level put go to different places), and global stores
+// carry the sc1 bit only as atomic stores: naturally aligned pieces of 1, 2, 4
+// or 8 bytes.  `d` names device memory.
+typedef __attribute__((address_space(1))) uint64_t *GlobalU64;
+typedef __attribute__((address_space(1))) uint32_t *GlobalU32;
+typedef __attribute__((address_space(1))) uint16_t *GlobalU16;
+typedef __attribute__((address_space(1))) uint8_t *GlobalU8;
+__device__ __forceinline__ void store_through8(char *d, uint64_t v) {
+  __hip_atomic_store((GlobalU64)d, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // NOLINT
+}
+__device__ __forceinline__ void store_through4(char *d, uint32_t v) {
+  __hip_atomic_store((GlobalU32)d, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // NOLINT
+}
+__device__ __forceinline__ void store_through2(char *d, uint16_t v) {
+  __hip_atomic_store((GlobalU16)d, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // NOLINT
+}
+__device__ __forceinline__ void store_through1(char *d, uint8_t v) {
+  __hip_atomic_store((GlobalU8)d, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // NOLINT
+}
+
+// One lane copies n bytes to device memory with write-through stores, so that
+// the payload of a thread-level put is visible at agent scope once the lane's
+// stores are acknowledged (s_waitcnt) — no L2 write-back.  The destination is
+// peeled to 8-byte alignment with the largest pieces its address allows, then
+// moved eight 8-byte pieces at a time (all loads of a batch before its
+// stores), then finished the same way.  The source may sit anywhere (device
+// memory, LDS, a stack variable) at any alignment.
+__device__ __forceinline__ void copy_thread_through(void *dst, const void *src, size_t n) {
+  char *d = static_cast<char *>(dst);
+  const char *s = static_cast<const char *>(src);
+  // One piece: the largest power of two that the address is aligned to, that
+  // fits, and that a store can carry.
+  auto piece = [&]() {
+    size_t a = reinterpret_cast<uintptr_t>(d) & 7u;
+    a = a ? (a & (~a + 1)) : 8;
+    while (a > n) a >>= 1;
+    if (a == 8) store_through8(d, *reinterpret_cast<const u64_any *>(s));
+    else if (a == 4) store_through4(d, *reinterpret_cast<const u32_any *>(s));
+    else if (a == 2) store_through2(d, *reinterpret_cast<const u16_any *>(s));
+    else store_through1(d, static_cast<uint8_t>(*s));
+    d += a; s += a; n -= a;
+  };
+  while (n && (reinterpret_cast<uintptr_t>(d) & 7u)) piece();
+  while (n >= 64) {
+    uint64_t v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const u64_any *>(s + 8 * u);
+#pragma unroll
+    for (int u = 0; u < 8; ++u) store_through8(d + 8 * u, v[u]);
+    d += 64; s += 64; n -= 64;
+  }
+  while (n) piece();
+}
+
+// A single value of 1, 2, 4 or 8 bytes (or a multiple of 8) at a naturally
+// aligned device address, written through: rocshmem_<T>_p.
+template <typename T>
+__device__ __forceinline__ void store_value_through(T *dst, T value) {
+  char *d = reinterpret_cast<char *>(dst);
+  if constexpr (sizeof(T) == 8) {
+    uint64_t b;
+    __builtin_memcpy(&b, &value, 8);
+    store_through8(d, b);
+  } else if constexpr (sizeof(T) == 4) {
+    uint32_t b;
+    __builtin_memcpy(&b, &value, 4);
+    store_through4(d, b);
+  } else if constexpr (sizeof(T) == 2) {
+    uint16_t b;
+    __builtin_memcpy(&b, &value, 2);
+    store_through2(d, b);
+  } else if constexpr (sizeof(T) == 1) {
+    uint8_t b;
+    __builtin_memcpy(&b, &value, 1);
+    store_through1(d, b);
+  } else {
+    copy_thread_through(d, &value, sizeof(T));
+  }
 }
 
 // Rank of this lane among the currently active lanes of its wavefront, and

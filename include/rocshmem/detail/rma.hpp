@@ -2,6 +2,7 @@
 #ifndef ROCSHMEM_AMD_DETAIL_RMA_HPP_
 #define ROCSHMEM_AMD_DETAIL_RMA_HPP_
 
+#include "coalesce.hpp"
 #include "copy_engine.hpp"
 #include "state.hpp"
 #include "sync.hpp"
@@ -18,17 +19,42 @@ __device__ __forceinline__ int translate_pe(rocshmem_ctx_t ctx, int pe) {
   return ti ? ti->pe_start + ti->stride * pe : pe;
 }
 
-// A context created with ROCSHMEM_CTX_NOSTORE promises that its quiet / fence
-// need not order the caller's own plain stores (the reference turns its flush
-// off for such contexts, src/fence_policy.hpp:45-63).  Everything the library
-// itself writes for a _wave / _wg put is a write-through store, so on such a
-// context completion is a wait on the issuing wavefront's own counters and the
-// L2 write-back of a release is skipped.  That write-back is the expensive
-// part when many work-groups end a put each: the L2 of an XCD serves them one
-// after another, about 60 ns each when idle and a memory round trip each while
-// stores are in flight.
+// ---- what completes a put, and what quiet / fence add -------------------------
+// Every store the library makes to the symmetric heap is a write-through store
+// (sc1): buffer stores in the cooperative copies and folds, atomic stores in
+// the single-lane copy.  Such a store is acknowledged once it is visible at
+// agent scope, so a wavefront completes its own puts by waiting for its own
+// memory operations (drain_own_stores) — no L2 write-back.  That is how the
+// blocking thread- and wavefront-level puts return with their payload
+// delivered on every kind of context, as the reference's do through a fence
+// after each copy (src/ipc/context_ipc_device.cpp:62-69,137-144), at a
+// fortieth of the cost: an agent-scope fence is an L2 write-back plus
+// invalidate, which an XCD's L2 serves one after another (measured on MI355X,
+// 2 Mi putmem_wave calls of 512 bytes from every CU: 70 M calls/s with a fence
+// per call, 2.7 G calls/s with the wait).
+//
+// What a put does NOT publish is the caller's own plain stores.  That is the
+// job of quiet and fence: on a default context a full agent-scope release
+// (L2 write-back; cumulative, so it also covers stores that other wavefronts
+// of the work-group made before a barrier).  A context created with
+// ROCSHMEM_CTX_NOSTORE promises that quiet / fence need not order the caller's
+// plain stores (the reference turns its flush off for such contexts,
+// src/fence_policy.hpp:45-63): there they are the wait alone.  The work-group
+// put ends in a barrier, not in a completion (as in the reference, :109-116);
+// on a NOSTORE context every wavefront also waits for its own share first, so
+// that a quiet by any one thread covers the whole work-group's put.
 __device__ __forceinline__ bool no_store_order(const Context *c) {
   return (ctx_view(c)->options & static_cast<unsigned>(ROCSHMEM_CTX_NOSTORE)) != 0;
+}
+// True when the heap is ordinary cached device memory (ROCSHMEM_EMU_HEAP_CACHED):
+// an XCD's L2 may then hold a stale copy of a line that another XCD has written
+// through to memory, and a get invalidates before it reads.  On the default
+// uncached heap no L2 ever holds a line of the heap.
+__device__ __forceinline__ bool heap_cached(const Context *c) {
+  return (ctx_view(c)->options & kCtxHeapCached) != 0;
+}
+__device__ __forceinline__ void fresh_reads(const Context *c) {
+  if (heap_cached(c)) fence_acquire();
 }
 // quiet / fence on context c.
 __device__ __forceinline__ void ctx_release(const Context *c) {
@@ -36,66 +62,101 @@ __device__ __forceinline__ void ctx_release(const Context *c) {
   else fence_release();
 }
 
-// ---- thread granularity: copy, then order (context_ipc_device.cpp:62-88) ---
+// ---- thread granularity (context_ipc_device.cpp:62-88) ----------------------
+// The reference puts a coalescing step in front of its per-thread messages
+// (src/wf_coal_policy.cpp:57-172).  Here, when the runtime asks for it
+// (DeviceState::coalesce_puts), a thread-level put first looks whether the
+// messages of all active lanes continue one another to the same PE; such a
+// run is one message, moved by the whole wavefront with the cooperative copy
+// (16 bytes per lane and step, whatever the size of a lane's own message).
+// Returns false, having done nothing, for anything else.
+__device__ __forceinline__ bool put_as_one_run(Context *c, void *dest, const void *source,
+                                               size_t n, int pe) {
+  size_t merged = n;
+  const bool sender = wf_coalesce(pe, source, dest, &merged);
+  const unsigned long long senders = __ballot(sender);
+  // One sender means every other active lane was absorbed, which needs the
+  // lane below it to be active: the run starts at the lowest active lane.
+  if (senders & (senders - 1)) return false;
+  // From here on everything is taken from the sender's lane, so that all
+  // lanes decide and address alike.
+  const int leader = __ffsll(static_cast<long long>(senders)) - 1;
+  const size_t total = read_lane(static_cast<unsigned long long>(merged), leader);
+  const size_t own = read_lane(static_cast<unsigned long long>(n), leader);
+  if (total == own) return false;  // a lone lane: nothing to share
+  char *d = reinterpret_cast<char *>(read_lane(reinterpret_cast<unsigned long long>(dest), leader));
+  const char *s = reinterpret_cast<const char *>(
+      read_lane(reinterpret_cast<unsigned long long>(source), leader));
+  const int to = read_lane(pe, leader);
+  copy_wave(remote_addr(c, d, to), s, total, g_state.nt_bytes);
+  drain_own_stores();
+  return true;
+}
+
 __device__ __forceinline__ void putmem(Context *c, void *dest, const void *source,
                                        size_t n, int pe) {
-  copy_thread(remote_addr(c, static_cast<char *>(dest), pe), source, n);
-  fence_full();
+  if (g_state.coalesce_puts && put_as_one_run(c, dest, source, n, pe)) return;
+  copy_thread_through(remote_addr(c, static_cast<char *>(dest), pe), source, n);
+  drain_own_stores();
 }
 __device__ __forceinline__ void getmem(Context *c, void *dest, const void *source,
                                        size_t n, int pe) {
+  fresh_reads(c);
   copy_thread(dest, remote_addr(c, static_cast<const char *>(source), pe), n);
-  fence_full();
+}
+// rocshmem_<T>_p / _g: one naturally aligned value.
+template <typename T>
+__device__ __forceinline__ void put_value(Context *c, T *dest, T value, int pe) {
+  store_value_through(remote_addr(c, dest, pe), value);
+  drain_own_stores();
 }
 
 // Non-blocking forms: the call only issues the copy; rocshmem_ctx_quiet (or
 // fence) by the same thread completes it.  The reference's _nbi calls are its
 // blocking ones; here a thread or wavefront that issues many small messages
-// pays for one completion instead of one per message.  A thread-level copy
-// leaves through plain stores, which only a full release makes visible, so on
-// a NOSTORE context (whose quiet does not write the L2 back) the call still
-// completes before it returns.
+// pays for one completion instead of one per message.
 __device__ __forceinline__ void putmem_nbi(Context *c, void *dest, const void *source,
                                            size_t n, int pe) {
-  copy_thread(remote_addr(c, static_cast<char *>(dest), pe), source, n);
-  if (no_store_order(c)) fence_full();
+  copy_thread_through(remote_addr(c, static_cast<char *>(dest), pe), source, n);
 }
 __device__ __forceinline__ void getmem_nbi(Context *c, void *dest, const void *source,
                                            size_t n, int pe) {
+  fresh_reads(c);
   copy_thread(dest, remote_addr(c, static_cast<const char *>(source), pe), n);
-  if (no_store_order(c)) fence_full();
 }
 
 // ---- wavefront granularity (context_ipc_device.cpp:137-164) ---------------
-// The ordering option is looked at before the copy although it is only needed
-// after it: the context's hot fields share one scalar load, and a call then
-// waits for the scalar data path once, not once per field (a scalar load that
-// hits costs about 100 ns, which a small message feels).
 __device__ __forceinline__ void putmem_wave(Context *c, void *dest, const void *source,
                                             size_t n, int pe) {
-  const bool relaxed = no_store_order(c);
   copy_wave(remote_addr(c, static_cast<char *>(dest), pe), source, n, g_state.nt_bytes);
-  if (relaxed) drain_own_stores();
-  else fence_full();
+  drain_own_stores();
 }
+// A get's stores go to the caller's own buffer; the wait makes them complete
+// for whoever reads it after a barrier.
 __device__ __forceinline__ void getmem_wave(Context *c, void *dest, const void *source,
                                             size_t n, int pe) {
+  fresh_reads(c);
   copy_wave(dest, remote_addr(c, static_cast<const char *>(source), pe), n, g_state.nt_bytes);
-  fence_full();
+  drain_own_stores();
 }
 
-// Non-blocking wavefront forms: write-through stores, complete at the calling
-// wavefront's quiet on either kind of context.
+// Non-blocking wavefront forms: complete at the calling wavefront's quiet on
+// either kind of context.
 __device__ __forceinline__ void putmem_nbi_wave(Context *c, void *dest, const void *source,
                                                 size_t n, int pe) {
   copy_wave(remote_addr(c, static_cast<char *>(dest), pe), source, n, g_state.nt_bytes);
 }
 __device__ __forceinline__ void getmem_nbi_wave(Context *c, void *dest, const void *source,
                                                 size_t n, int pe) {
+  fresh_reads(c);
   copy_wave(dest, remote_addr(c, static_cast<const char *>(source), pe), n, g_state.nt_bytes);
 }
 
 // ---- work-group granularity: copy, then __syncthreads (:109-125) ----------
+// The ordering option is looked at before the copy although it is only needed
+// after it: the context's hot fields share one scalar load, and a call then
+// waits for the scalar data path once, not once per field (a scalar load that
+// hits costs about 100 ns, which a small message feels).
 __device__ __forceinline__ void putmem_wg(Context *c, void *dest, const void *source,
                                           size_t n, int pe) {
   const bool relaxed = no_store_order(c);
@@ -108,6 +169,7 @@ __device__ __forceinline__ void putmem_wg(Context *c, void *dest, const void *so
 }
 __device__ __forceinline__ void getmem_wg(Context *c, void *dest, const void *source,
                                           size_t n, int pe) {
+  fresh_reads(c);
   copy_lanes(dest, remote_addr(c, static_cast<const char *>(source), pe), n,
              flat_thread_id(), flat_block_size(), g_state.nt_bytes);
   __syncthreads();
@@ -116,11 +178,9 @@ __device__ __forceinline__ void getmem_wg(Context *c, void *dest, const void *so
 // ---- signal update by the one lane that leads the call (:221-298) ---------
 // On a default context the store / add is a release at agent scope, which
 // orders it after the payload and after everything else the caller's group
-// wrote before it.  On a ROCSHMEM_CTX_NOSTORE context the payload of a _wave /
-// _wg put is already complete when the leader gets here (write-through
-// stores, drained by each wavefront), so a relaxed update suffices; the
-// thread-granularity put moves its payload with plain stores and keeps the
-// release.
+// wrote before it.  On a ROCSHMEM_CTX_NOSTORE context the payload is already
+// complete when the leader gets here (write-through stores, waited for by
+// each wavefront or thread), so a relaxed update suffices.
 __device__ __forceinline__ void signal_update(Context *c, uint64_t *sig_addr,
                                               uint64_t signal, int sig_op, int pe,
                                               bool relaxed = false) {
@@ -142,7 +202,7 @@ __device__ __forceinline__ void putmem_signal(Context *c, void *dest, const void
                                               size_t n, uint64_t *sig_addr,
                                               uint64_t signal, int sig_op, int pe) {
   putmem(c, dest, source, n, pe);
-  signal_update(c, sig_addr, signal, sig_op, pe);
+  signal_update(c, sig_addr, signal, sig_op, pe, no_store_order(c));
 }
 __device__ __forceinline__ void putmem_signal_wave(Context *c, void *dest,
                                                    const void *source, size_t n,

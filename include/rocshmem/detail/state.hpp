@@ -92,6 +92,10 @@ struct Team {
   void *pWrk;          // ROCSHMEM_REDUCE_MIN_WRKDATA_SIZE * 8 bytes
 };
 
+// Library-internal bit of Context::options, beside the public ROCSHMEM_CTX_*
+// ones: the heap is ordinary cached device memory (ROCSHMEM_EMU_HEAP_CACHED).
+constexpr unsigned kCtxHeapCached = 1u << 30;
+
 // Per-PE communication context (device memory, pooled).  Kernels never write
 // a context: the host fills them all in at initialisation, so device code
 // reads them through the scalar data path (see ctx_view).
@@ -100,7 +104,7 @@ struct Context {
   // load brings all three.
   uint64_t pe_stride;   // bytes between consecutive slices
   int my_pe;
-  unsigned options;     // ROCSHMEM_CTX_* bits, fixed per object
+  unsigned options;     // ROCSHMEM_CTX_* bits and kCtxHeapCached, fixed per object
   char *heap_base;      // base of PE 0's slice
   uint64_t ws_stride;   // bytes between consecutive PEs' work/sync areas
   int num_pes;
@@ -139,6 +143,8 @@ struct DeviceState {
   char *ws_base;          // work/sync area of PE 0
   uint64_t nt_bytes;      // copies at least this large use non-temporal accesses
   QueueBinding *queue_table;  // [kQueueTableSize], indexed by queue id modulo the size
+  int coalesce_puts;      // thread-level puts first look for one run across the wavefront
+  int pad_;
 };
 
 #if defined(__HIPCC__)

@@ -29,10 +29,6 @@ __device__ __forceinline__ void fence_release() {
 __device__ __forceinline__ void fence_acquire() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
 }
-// fence()/quiet(): order everything issued before against everything after.
-__device__ __forceinline__ void fence_full() {
-  __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "agent");
-}
 // Wait until every memory operation this wavefront has issued is acknowledged.
 // A write-through (sc1) store is acknowledged once it is visible at agent
 // scope, so after this the wavefront's cooperative-copy stores are complete

@@ -76,10 +76,10 @@ __device__ ATTR_NO_INLINE inline void rocshmem_getmem_nbi(void *dest, const void
   }                                                                                      \
   __device__ ATTR_NO_INLINE inline void rocshmem_ctx_##TN##_p(rocshmem_ctx_t ctx,        \
                                                               T *dest, T value, int pe) {\
-    rocshmem_ctx_putmem(ctx, dest, &value, sizeof(T), pe);                               \
+    detail::put_value<T>(detail::ctx_of(ctx), dest, value, detail::translate_pe(ctx, pe));\
   }                                                                                      \
   __device__ ATTR_NO_INLINE inline void rocshmem_##TN##_p(T *dest, T value, int pe) {    \
-    rocshmem_putmem(dest, &value, sizeof(T), pe);                                        \
+    rocshmem_ctx_##TN##_p(rocshmem_ctx_t{nullptr, nullptr}, dest, value, pe);            \
   }                                                                                      \
   __device__ ATTR_NO_INLINE inline void rocshmem_ctx_##TN##_get(                         \
       rocshmem_ctx_t ctx, T *dest, const T *source, size_t nelems, int pe) {             \

@@ -132,6 +132,13 @@ int rocshmem_amd_set_pe_rule(int rule);
  * the reference's flush off for that option).  Returns the previous options,
  * -1 before init. */
 int64_t rocshmem_amd_set_ctx_options(int64_t options);
+/* Whether thread-level puts (rocshmem_putmem / rocshmem_<T>_put) first look
+ * for one run across the active lanes of the wavefront — messages to the same
+ * PE that continue one another, what the reference's coalescing policy merges
+ * (src/wf_coal_policy.cpp:57-172) — and move such a run with the whole
+ * wavefront.  Initial value: ROCSHMEM_COALESCE_PUTS (default 0).  Returns the
+ * previous setting, -1 before rocshmem_init. */
+int rocshmem_amd_set_coalesce_puts(int on);
 /* rocshmem_malloc / rocshmem_free (rocshmem.hpp:115-123): NULL on size 0 or
  * exhaustion; the object exists at the same offset on every PE. */
 void *rocshmem_amd_malloc(size_t size);
@@ -295,6 +302,15 @@ int rocshmem_amd_putmem(void *dest, const void *source, size_t nbytes, int my_pe
 int rocshmem_amd_getmem(void *dest, const void *source, size_t nbytes, int my_pe, int pe,
                         rocshmem_amd_stream_t stream);
 
+/* One wavefront whose lanes each make their own rocshmem_ctx_putmem call
+ * (src/ipc/context_ipc_device.cpp:62-69 behind the coalescing front end,
+ * src/wf_coal_policy.cpp:57-172): lane i, when bit i of active_mask is set,
+ * puts size[i] bytes from source + src_off[i] to dest + dst_off[i] (a symmetric
+ * address on my_pe) on PE pe[i].  Host arrays of 64 entries.  Waits for the
+ * kernel. */
+int rocshmem_amd_lane_puts(void *dest, const void *source, const int *pe, const uint64_t *src_off,
+                           const uint64_t *dst_off, const uint64_t *size, uint64_t active_mask,
+                           int my_pe, rocshmem_amd_stream_t stream);
 /* wf_coal_policy coalesce (src/wf_coal_policy.cpp:57-172) on one wavefront:
  * lane i of the 64 is active iff bit i of active_mask; inputs are 64-entry
  * host arrays; outputs say whether the lane must send and its message size. */

@@ -31,6 +31,12 @@ int rocshmem_amd_set_pe_rule(int rule) {
   rt().set_pe_rule(rule);
   return 0;
 }
+int rocshmem_amd_set_coalesce_puts(int on) {
+  if (!rt().live) return -1;
+  const int before = rt().state.coalesce_puts;
+  rt().set_coalesce_puts(on);
+  return before;
+}
 int64_t rocshmem_amd_set_ctx_options(int64_t options) {
   if (!rt().live) return -1;
   const int64_t before = rt().driver_ctx_options;

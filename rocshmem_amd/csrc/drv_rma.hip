@@ -226,6 +226,24 @@ __global__ void coalesce_kernel(const int *pe, const uint64_t *src, const uint64
   size_out[lane] = sz;
 }
 
+// One wavefront whose lanes each make their own rocshmem_ctx_putmem call: lane
+// i, when its bit of active_mask is set, puts size[i] bytes from source +
+// src_off[i] to dest + dst_off[i] on PE pe[i].
+struct LanePutArgs {
+  char *dest;
+  const char *source;
+  const int *pe;
+  const uint64_t *src_off, *dst_off, *size;
+  uint64_t active_mask;
+  rocshmem_ctx_t ctx;
+};
+__global__ void lane_puts_kernel(LanePutArgs a) {
+  const unsigned lane = threadIdx.x;
+  if (!((a.active_mask >> lane) & 1ull)) return;
+  rocshmem_ctx_putmem(a.ctx, a.dest + a.dst_off[lane], a.source + a.src_off[lane], a.size[lane],
+                      a.pe[lane]);
+}
+
 }  // namespace drv
 }  // namespace rocshmem
 
@@ -383,6 +401,47 @@ int rocshmem_amd_getmem(void *dest, const void *source, size_t nbytes, int my_pe
   const char *origin = static_cast<const char *>(source) +
                        static_cast<int64_t>(pe - my_pe) * static_cast<int64_t>(runtime::rt().pe_stride);
   launch_bulk(static_cast<char *>(dest), origin, nbytes, as_stream(stream));
+  return 0;
+}
+
+int rocshmem_amd_lane_puts(void *dest, const void *source, const int *pe, const uint64_t *src_off,
+                           const uint64_t *dst_off, const uint64_t *size, uint64_t active_mask,
+                           int my_pe, rocshmem_amd_stream_t stream) {
+  if (!valid_pe(my_pe) || !pe || !src_off || !dst_off || !size) return -1;
+  for (int i = 0; i < 64; ++i) {
+    if (!((active_mask >> i) & 1ull)) continue;
+    if (!valid_pe(pe[i])) return -1;
+    if (!sym_ok_on(static_cast<char *>(dest) + dst_off[i], size[i], my_pe)) return -1;
+    if (!local_ok(static_cast<const char *>(source) + src_off[i], size[i])) return -1;
+  }
+  // The per-lane tables live in one device block: 64 x (pe, three offsets).
+  struct Tables {
+    int pe[64];
+    uint64_t src_off[64], dst_off[64], size[64];
+  } host;
+  for (int i = 0; i < 64; ++i) {
+    host.pe[i] = pe[i];
+    host.src_off[i] = src_off[i];
+    host.dst_off[i] = dst_off[i];
+    host.size[i] = size[i];
+  }
+  Tables *dev;
+  DRV_CHECK_HIP(hipMalloc(&dev, sizeof(Tables)));
+  DRV_CHECK_HIP(hipMemcpy(dev, &host, sizeof(Tables), hipMemcpyHostToDevice));
+  LanePutArgs a;
+  a.dest = static_cast<char *>(dest);
+  a.source = static_cast<const char *>(source);
+  a.pe = dev->pe;
+  a.src_off = dev->src_off;
+  a.dst_off = dev->dst_off;
+  a.size = dev->size;
+  a.active_mask = active_mask;
+  a.ctx = runtime::rt().driver_ctx_handle(my_pe);
+  hipStream_t s = as_stream(stream);
+  hipLaunchKernelGGL(lane_puts_kernel, dim3(1), dim3(64), 0, s, a);
+  DRV_CHECK_HIP(hipGetLastError());
+  DRV_CHECK_HIP(hipStreamSynchronize(s));
+  DRV_CHECK_HIP(hipFree(dev));
   return 0;
 }
 

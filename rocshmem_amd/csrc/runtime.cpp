@@ -452,7 +452,7 @@ int Runtime::init(int want_npes, size_t want_heap) {
     c.num_pes = npes;
     c.tinfo = &d_teams[pe].wrt_world;
     c.world_sync = reinterpret_cast<detail::SyncPad *>(d_ws + static_cast<size_t>(pe) * ws_stride);
-    c.options = 0;
+    c.options = heap_uncached ? 0u : detail::kCtxHeapCached;
     c.pool_slot = slot;
   };
   // Rows [0, npes) are the default contexts; rows [npes, 2*npes) are the same
@@ -461,7 +461,7 @@ int Runtime::init(int want_npes, size_t want_heap) {
   for (int pe = 0; pe < npes; ++pe) {
     fill_ctx(ctxs[pe], pe, -1);
     fill_ctx(ctxs[npes + pe], pe, -1);
-    ctxs[npes + pe].options = static_cast<unsigned>(ROCSHMEM_CTX_NOSTORE);
+    ctxs[npes + pe].options |= static_cast<unsigned>(ROCSHMEM_CTX_NOSTORE);
   }
   RT_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&d_default_ctx),
                          sizeof(detail::Context) * ctxs.size()));
@@ -480,7 +480,7 @@ int Runtime::init(int want_npes, size_t want_heap) {
     for (int s = 0; s < max_ctxs; ++s) {
       fill_ctx(row[s], pe, s);
       fill_ctx(row[max_ctxs + s], pe, s);
-      row[max_ctxs + s].options = static_cast<unsigned>(ROCSHMEM_CTX_NOSTORE);
+      row[max_ctxs + s].options |= static_cast<unsigned>(ROCSHMEM_CTX_NOSTORE);
     }
     detail::CtxPool &p = pools[pe];
     memset(&p, 0, sizeof(p));
@@ -524,6 +524,7 @@ int Runtime::init(int want_npes, size_t want_heap) {
   state.ctx_pool = d_pools;
   state.ws_base = d_ws;
   state.nt_bytes = env_size("ROCSHMEM_NT_THRESHOLD", detail::kNonTemporalBytes);
+  state.coalesce_puts = static_cast<int>(env_size("ROCSHMEM_COALESCE_PUTS", 0));
   live = true;
   push_state();
   ROCSHMEM_TEAM_WORLD = team_handle(0, acting_pe);
@@ -691,6 +692,14 @@ void Runtime::set_pe(int pe) {
   ROCSHMEM_TEAM_WORLD = team_handle(0, pe);
   if (state.fixed_pe != pe) {
     state.fixed_pe = pe;
+    push_state();
+  }
+}
+
+void Runtime::set_coalesce_puts(int on) {
+  require_live("rocshmem_amd_set_coalesce_puts");
+  if (state.coalesce_puts != (on ? 1 : 0)) {
+    state.coalesce_puts = on ? 1 : 0;
     push_state();
   }
 }

@@ -76,6 +76,7 @@ struct Runtime {
 
   void set_pe(int pe);
   void set_pe_rule(int rule);
+  void set_coalesce_puts(int on);
 
   // Context handle of PE `pe` bound to its member object of team slot `slot`.
   rocshmem_ctx_t default_ctx_handle(int pe, int slot = 0) const {

@@ -32,6 +32,7 @@ SIGNATURES = {
     "rocshmem_amd_set_pe": (_i, [_i]),
     "rocshmem_amd_set_pe_rule": (_i, [_i]),
     "rocshmem_amd_set_ctx_options": (C.c_int64, [C.c_int64]),
+    "rocshmem_amd_set_coalesce_puts": (_i, [_i]),
     "rocshmem_amd_malloc": (_vp, [_sz]),
     "rocshmem_amd_free": (_i, [_vp]),
     "rocshmem_amd_pe_ptr": (_vp, [_vp, _i]),
@@ -92,6 +93,7 @@ SIGNATURES = {
                                          C.POINTER(_u64), C.POINTER(_i), _vp]),
     "rocshmem_amd_putmem": (_i, [_vp, _vp, _sz, _i, _i, _vp]),
     "rocshmem_amd_getmem": (_i, [_vp, _vp, _sz, _i, _i, _vp]),
+    "rocshmem_amd_lane_puts": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _u64, _i, _vp]),
     "rocshmem_amd_wf_coalesce": (_i, [_vp, _vp, _vp, _vp, _u64, _vp, _vp]),
     "rocshmem_amd_wg_reduce": (_i, [_i, _i, _vp, _vp, _vp, _i, _i, _vp]),
     "rocshmem_amd_wg_reduce_teams": (_i, [_i, _i, C.POINTER(_vp), _i, _vp, _vp, _i, _i, _i, _i, _vp]),

@@ -571,3 +571,66 @@ def test_wf_coalesce_matches_oracle(rt, L, orc, seed):
     assert np.array_equal(out[act], wout[act])
     if seed == 1:
         assert sends.sum() == 3 and (out[0], out[9], out[10]) == (72, 8, 432)
+
+
+@pytest.mark.parametrize("coalesce", [0, 1])
+@pytest.mark.parametrize("seed", range(10))
+def test_per_lane_puts_with_and_without_coalescing(rt, L, orc, seed, coalesce):
+    """Every active lane of one wavefront makes its own rocshmem_putmem call
+    (src/ipc/context_ipc_device.cpp:62-69): mixed runs, lone lanes, inactive
+    lanes, several target PEs, sizes that are no multiple of anything, and —
+    seeds 0 to 2 — one run across the whole wavefront, which the coalescing
+    front end moves as a single message (src/wf_coal_policy.cpp:57-172).  With
+    the front end off and on, the destination on every PE must be what the
+    oracle's plain copies of the sending lanes give; where the oracle's
+    coalescing finds exactly one sender, its merged size is the whole run."""
+    l = rt.up(P, HEAP)
+    rng = np.random.default_rng(100 + seed)
+    span = 1 << 16
+    src_sym, dst_sym = l.malloc(span), l.malloc(span)
+    payload = orc.fill_u8(span, 9, seed)
+    rt.put_bytes(l.pe_ptr(src_sym, 2), payload)
+    for p in range(P):
+        l.fill(l.pe_ptr(dst_sym, p), 0xEE, span)
+    if seed < 3:
+        unit = [8, 64, 12][seed]
+        size = np.full(64, unit, np.uint64)
+        pe = np.full(64, 5, np.int32)
+        src = 40 + unit * np.arange(64, dtype=np.uint64)
+        dst = 24 + unit * np.arange(64, dtype=np.uint64)
+        mask = (1 << 64) - 1 if seed != 2 else ((1 << 64) - 1) & ~((1 << 7) - 1)  # lanes 7..63
+    else:
+        size = rng.choice([1, 3, 4, 8, 8, 8, 16, 100], 64).astype(np.uint64)
+        pe = rng.choice([0, 5, 5, 5], 64).astype(np.int32)
+        src = np.zeros(64, np.uint64)
+        dst = np.zeros(64, np.uint64)
+        so, do = 16, 48
+        for k in range(64):
+            if rng.random() < 0.2:
+                so += 64
+            if rng.random() < 0.1:
+                do += 128
+            src[k], dst[k] = so, do
+            so += int(size[k])
+            do += int(size[k])
+        mask = int(rng.integers(1, 1 << 63, dtype=np.uint64)) | 1
+    before = l.set_coalesce_puts(coalesce)
+    rc = l.lane_puts(l.pe_ptr(dst_sym, 2), l.pe_ptr(src_sym, 2), pe.ctypes.data, src.ctypes.data,
+                     dst.ctypes.data, size.ctypes.data, mask, 2, None)
+    l.set_coalesce_puts(before)
+    assert rc == 0
+    want = {p: np.full(span, 0xEE, np.uint8) for p in range(P)}
+    for k in range(64):
+        if (mask >> k) & 1:
+            n = int(size[k])
+            piece = np.empty(n, np.uint8)
+            orc.lib.orc_copy(piece.ctypes.data, payload[int(src[k]):int(src[k]) + n].ctypes.data, n)
+            want[int(pe[k])][int(dst[k]):int(dst[k]) + n] = piece
+    for p in range(P):
+        assert np.array_equal(rt.get_bytes(l.pe_ptr(dst_sym, p), span), want[p]), (seed, coalesce, p)
+    sends, merged = orc.wf_coalesce(pe, src, dst, size, mask)
+    act = np.array([(mask >> k) & 1 for k in range(64)], bool)
+    if seed < 3:
+        assert sends[act].sum() == 1 and merged[act][0] == size[act].sum()
+    l.free(src_sym)
+    l.free(dst_sym)
