@@ -354,11 +354,11 @@ def message_rates(b, steps):
 
 def reuse_config(b, steps):
     """What a consumer that re-reads symmetric data gets from the caches: a
-    256 MiB symmetric buffer read four times, tile by tile (8 KiB tiles, each
-    read four times in a row by its work-group), against one pass.  The tiles
-    of the work-groups resident on an XCD together fit its 4 MiB L2 (256
-    work-groups of 256 lanes, 8 KiB each), so on cached memory the later passes
-    are L2 hits."""
+    256 MiB symmetric buffer read four times, tile by tile (each 64 KiB tile
+    four times in a row by its work-group of 1024 lanes, one work-group per
+    CU), against one pass.  A tile is larger than a CU's vector L1, and the
+    tiles in flight on an XCD (32 x 64 KiB) fit its 4 MiB L2: on cached memory
+    the later passes are L2 hits."""
     l = b.l
     n = 256 * MiB
     buf = l.malloc(n)
@@ -366,7 +366,7 @@ def reuse_config(b, steps):
     b.fill_random(buf, n, 0, 91)
     res = {}
     for passes in (1, 4):
-        ms = b.time_ms(lambda: b.probes.reuse_probe(buf, n, 8 << 10, passes, 2048, 256, None),
+        ms = b.time_ms(lambda: b.probes.reuse_probe(buf, n, 64 << 10, passes, 256, 1024, None),
                        max(5, steps // 4), 2)
         res["read_x%d_gbs" % passes] = round(passes * n / ms / 1e6, 1)
     l.free(buf)

@@ -316,37 +316,51 @@ __device__ __forceinline__ void store_through2(char *d, uint16_t v) {
 __device__ __forceinline__ void store_through1(char *d, uint8_t v) {
   __hip_atomic_store((GlobalU8)d, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // NOLINT
 }
+// Sixteen bytes at a 16-byte aligned device address.  No builtin gives a
+// global store of this width the sc1 bit, so the instruction is written out;
+// the compiler does not count it among the outstanding memory operations,
+// which only makes its own waits stricter, and callers wait for the lane's
+// stores themselves (drain_own_stores).  The s_nop keeps a following write to
+// the data registers one wait state away, as a store of more than 8 bytes
+// needs on this family.
+__device__ __forceinline__ void store_through16(char *d, u32x4 v) {
+  asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 0"
+               :
+               : "v"(reinterpret_cast<unsigned long long>(d)), "v"(v)
+               : "memory");
+}
 
 // One lane copies n bytes to device memory with write-through stores, so that
 // the payload of a thread-level put is visible at agent scope once the lane's
 // stores are acknowledged (s_waitcnt) — no L2 write-back.  The destination is
-// peeled to 8-byte alignment with the largest pieces its address allows, then
-// moved eight 8-byte pieces at a time (all loads of a batch before its
+// peeled to 16-byte alignment with the largest pieces its address allows, then
+// moved eight 16-byte vectors at a time (all loads of a batch before its
 // stores), then finished the same way.  The source may sit anywhere (device
 // memory, LDS, a stack variable) at any alignment.
 __device__ __forceinline__ void copy_thread_through(void *dst, const void *src, size_t n) {
   char *d = static_cast<char *>(dst);
   const char *s = static_cast<const char *>(src);
-  // One piece: the largest power of two that the address is aligned to, that
-  // fits, and that a store can carry.
+  // One piece: the largest power of two up to 16 that the address is aligned
+  // to and that fits.
   auto piece = [&]() {
-    size_t a = reinterpret_cast<uintptr_t>(d) & 7u;
-    a = a ? (a & (~a + 1)) : 8;
+    size_t a = reinterpret_cast<uintptr_t>(d) & 15u;
+    a = a ? (a & (~a + 1)) : 16;
     while (a > n) a >>= 1;
-    if (a == 8) store_through8(d, *reinterpret_cast<const u64_any *>(s));
+    if (a == 16) store_through16(d, *reinterpret_cast<const u32x4_any *>(s));
+    else if (a == 8) store_through8(d, *reinterpret_cast<const u64_any *>(s));
     else if (a == 4) store_through4(d, *reinterpret_cast<const u32_any *>(s));
     else if (a == 2) store_through2(d, *reinterpret_cast<const u16_any *>(s));
     else store_through1(d, static_cast<uint8_t>(*s));
     d += a; s += a; n -= a;
   };
-  while (n && (reinterpret_cast<uintptr_t>(d) & 7u)) piece();
-  while (n >= 64) {
-    uint64_t v[8];
+  while (n && (reinterpret_cast<uintptr_t>(d) & 15u)) piece();
+  while (n >= 128) {
+    u32x4 v[8];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const u64_any *>(s + 8 * u);
+    for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const u32x4_any *>(s + 16 * u);
 #pragma unroll
-    for (int u = 0; u < 8; ++u) store_through8(d + 8 * u, v[u]);
-    d += 64; s += 64; n -= 64;
+    for (int u = 0; u < 8; ++u) store_through16(d + 16 * u, v[u]);
+    d += 128; s += 128; n -= 128;
   }
   while (n) piece();
 }

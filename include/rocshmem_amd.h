@@ -136,7 +136,7 @@ int64_t rocshmem_amd_set_ctx_options(int64_t options);
  * for one run across the active lanes of the wavefront — messages to the same
  * PE that continue one another, what the reference's coalescing policy merges
  * (src/wf_coal_policy.cpp:57-172) — and move such a run with the whole
- * wavefront.  Initial value: ROCSHMEM_COALESCE_PUTS (default 0).  Returns the
+ * wavefront.  Initial value: ROCSHMEM_COALESCE_PUTS (default 1: on).  Returns the
  * previous setting, -1 before rocshmem_init. */
 int rocshmem_amd_set_coalesce_puts(int on);
 /* rocshmem_malloc / rocshmem_free (rocshmem.hpp:115-123): NULL on size 0 or

@@ -28,7 +28,7 @@ __device__ __forceinline__ size_t tile_slot(size_t i, uint32_t scatter_mask) {
 }
 
 // One API call per tile; group g takes tiles g, g+G, ...
-template <int kOp, int kGran>
+template <int kOp, int kGran, bool kScattered>
 __global__ void rma_kernel(RmaArgs a) {
   size_t group, groups;
   const size_t tid = threadIdx.x, bs = blockDim.x;
@@ -43,10 +43,17 @@ __global__ void rma_kernel(RmaArgs a) {
     group = blockIdx.x * bs + tid;
     groups = gridDim.x * bs;
   }
-  const size_t ntiles = (a.nbytes + a.tile - 1) / a.tile;
+  // No division and no multiplication on the way to a group's first load: the
+  // walk is by offsets, and the scattered walk keeps the tile index beside it.
+  const size_t stride = groups * a.tile;
   for (int it = 0; it < a.iters; ++it) {
-    for (size_t i = group; i < ntiles; i += groups) {
-      const size_t off = tile_slot(i, a.scatter_mask) * a.tile;
+    size_t i = group;
+    for (size_t walk = group * a.tile; walk < a.nbytes; walk += stride) {
+      size_t off = walk;
+      if constexpr (kScattered) {
+        off = tile_slot(i, a.scatter_mask) * a.tile;
+        i += groups;
+      }
       const size_t len = a.nbytes - off < a.tile ? a.nbytes - off : a.tile;
       if constexpr (kOp == ROCSHMEM_AMD_PUT) {
         if constexpr (kGran == ROCSHMEM_AMD_WG)
@@ -296,8 +303,11 @@ int rocshmem_amd_rma_messages(int rma_op, int gran, void *dest, const void *sour
   }
   hipStream_t s = as_stream(stream);
   const dim3 g(n_wgs), b(wg_size);
-#define RMA_CASE(OP, GR)                                                          \
-  if (rma_op == OP && gran == GR) hipLaunchKernelGGL((rma_kernel<OP, GR>), g, b, 0, s, a);
+#define RMA_CASE(OP, GR)                                                               \
+  if (rma_op == OP && gran == GR) {                                                    \
+    if (a.scatter_mask) hipLaunchKernelGGL((rma_kernel<OP, GR, true>), g, b, 0, s, a);  \
+    else hipLaunchKernelGGL((rma_kernel<OP, GR, false>), g, b, 0, s, a);                \
+  }
   RMA_CASE(ROCSHMEM_AMD_PUT, ROCSHMEM_AMD_THREAD)
   RMA_CASE(ROCSHMEM_AMD_PUT, ROCSHMEM_AMD_WAVE)
   RMA_CASE(ROCSHMEM_AMD_PUT, ROCSHMEM_AMD_WG)

@@ -524,7 +524,7 @@ int Runtime::init(int want_npes, size_t want_heap) {
   state.ctx_pool = d_pools;
   state.ws_base = d_ws;
   state.nt_bytes = env_size("ROCSHMEM_NT_THRESHOLD", detail::kNonTemporalBytes);
-  state.coalesce_puts = static_cast<int>(env_size("ROCSHMEM_COALESCE_PUTS", 0));
+  state.coalesce_puts = env_size("ROCSHMEM_COALESCE_PUTS", 1) != 0 ? 1 : 0;
   live = true;
   push_state();
   ROCSHMEM_TEAM_WORLD = team_handle(0, acting_pe);
