@@ -668,8 +668,17 @@ def profile_kernels():
     l.free(src)
     l.free(dst)
     a2a = alltoall_config(b, 6)
+    red = to_all_configs(b, 6, 2, which=("fp32_sum",))  # includes the many-teams device all-reduce
+    reuse = {"uncached_heap": reuse_config(b, 8)}       # 7 launches per number of passes (1, then 4)
     l.finalize()
+    # the same reads once more on a cached heap: the later launches of reuse_probe_kernel
+    bring_up(L, 1 << 30, ROCSHMEM_EMU_SPREAD=None, ROCSHMEM_EMU_HEAP_CACHED="1")
+    reuse["cached_heap"] = reuse_config(b, 8)
+    l.finalize()
+    os.environ.pop("ROCSHMEM_EMU_HEAP_CACHED", None)
     print(json.dumps({"putmem_wg_nostore_gbs": round(head["gbs"], 1),
+                      "wg_reduce_teams": {k: v for k, v in red.items() if "teams" in k},
+                      "reuse_256MiB": reuse,
                       "putmem_wg_default_gbs": round(head["default_ctx_gbs"], 1),
                       "host_putmem_gbs": round(head["host_putmem_gbs"], 1),
                       "to_all_fp32_sum_gbs": round(2 * P * m * 4 / ms_red / 1e6, 1),

@@ -42,10 +42,11 @@ __device__ __forceinline__ void barrier_all(Context *c) {
 // All-reduce over the team.  Replaces the reference's direct / ring selector
 // and its two algorithms (src/ipc/context_ipc_tmpl_device.hpp:166-418) by a
 // direct reduce-scatter + all-gather in one pass: after every member has
-// arrived, member k folds its share of the index range (every P-th block of
-// kShareVectors vectors, whatever the size of its work-group) from all P
-// sources in ascending member order and stores the result into all P
-// destinations; a second barrier ends the operation.  Each element is computed
+// arrived, the members fold the index range between them — blocks drawn in
+// index order from a counter for large arrays, every P-th block of
+// kShareVectors vectors for small ones, either way whatever the sizes of their
+// work-groups — from all P sources in ascending member order and store the
+// result into all P destinations; a second barrier ends the operation.  Each element is computed
 // once, so all members hold bit-identical results.
 //
 // The reference's selector (:361-418) takes its direct path when P * nreduce
@@ -54,6 +55,11 @@ __device__ __forceinline__ void barrier_all(Context *c) {
 // 2 * P <= ROCSHMEM_REDUCE_SYNC_SIZE, and otherwise returns ROCSHMEM_ERROR.
 // Nothing here needs those buffers, but the same calls are refused so that a
 // program sees the same status on either library.
+// Arrays of at least this many bytes per member are shared out through the
+// counter (tens of draws per wavefront; below that the draw's round trip is
+// not worth it).
+constexpr size_t kTicketBytesFrom = size_t{1} << 20;
+
 __device__ __forceinline__ bool reduce_accepted(int P, int nreduce) {
   const size_t direct_wrk = static_cast<size_t>(P) * static_cast<size_t>(nreduce);
   size_t provided_wrk = static_cast<size_t>(nreduce / 2 + 1);
@@ -71,27 +77,37 @@ __device__ __forceinline__ int wg_reduce(Context *c, Team *t,
   const int P = t->num_pes;
   if (!reduce_accepted(P, nreduce)) return ROCSHMEM_ERROR;
 
+  const size_t n = static_cast<size_t>(nreduce);
+  // Large arrays are handed out block by block from a counter on the team's
+  // first member (see fold_window), which that member zeroes before it
+  // arrives: nobody draws before the entry barrier has seen every member, and
+  // every draw of the call before has been answered by its exit barrier.
+  // Small ones are split by rule, which costs no round trip to the counter.
+  const bool by_tickets = n * sizeof(S) >= kTicketBytesFrom && n * sizeof(S) <= kWindowBytes;
+  SyncPad *const first_pad = remote_ws(c, &t->sync[SYNC_REDUCE], t->wrt_world.pe_start);
+  unsigned long long *const tickets = &first_pad->tickets;
+  if (by_tickets && t->my_pe == 0 && is_block_leader()) store_through(tickets, 0ull);
+
   // Entry: every member's source, which its caller may have written with plain
   // stores, is final.
   team_pad_sync(c, t, SYNC_REDUCE, publish_of(c));
 
-  const size_t n = static_cast<size_t>(nreduce);
   const int64_t to_first = static_cast<int64_t>(t->wrt_world.pe_start - ctx_view(c)->my_pe) *
                            static_cast<int64_t>(ctx_view(c)->pe_stride);
   const int64_t hop = static_cast<int64_t>(t->wrt_world.stride) *
                       static_cast<int64_t>(ctx_view(c)->pe_stride);
   S *dst0 = reinterpret_cast<S *>(reinterpret_cast<char *>(dest) + to_first);
   const S *src0 = reinterpret_cast<const S *>(reinterpret_cast<const char *>(source) + to_first);
-  // The members share the whole range block by block (see fold_window).  Arrays
-  // that are streamed once are read and written with the non-temporal hint, as
-  // the bulk copy does.
+  // Arrays that are streamed once are read and written with the non-temporal
+  // hint, as the bulk copy does.
   const size_t part = static_cast<size_t>(t->my_pe), nparts = static_cast<size_t>(P);
-  if (n * sizeof(S) >= g_state.nt_bytes)
-    fold_span_any<E, Op, true, true>(dst0, src0, hop, P, 0, n, flat_thread_id(), flat_block_size(),
-                                     part, nparts);
+  const unsigned tid = flat_thread_id(), bs = flat_block_size();
+  if (by_tickets)
+    fold_span_any<E, Op, true, SHARE_TICKETS>(dst0, src0, hop, P, 0, n, tid, bs, part, nparts, tickets);
+  else if (n * sizeof(S) >= g_state.nt_bytes)
+    fold_span_any<E, Op, true, SHARE_BLOCKS>(dst0, src0, hop, P, 0, n, tid, bs, part, nparts);
   else
-    fold_span_any<E, Op, false, true>(dst0, src0, hop, P, 0, n, flat_thread_id(),
-                                      flat_block_size(), part, nparts);
+    fold_span_any<E, Op, false, SHARE_BLOCKS>(dst0, src0, hop, P, 0, n, tid, bs, part, nparts);
 
   // Exit: the results were written by the fold, through to memory.
   team_pad_sync(c, t, SYNC_REDUCE, PUBLISH_LIBRARY);

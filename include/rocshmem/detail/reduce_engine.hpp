@@ -153,8 +153,8 @@ constexpr size_t kShareVectors = 1024;
 // (hi - lo) * sizeof(element) must not exceed kWindowBytes.  Results leave as
 // write-through buffer stores, one resource per destination.
 //
-// With kShared the range is shared by `nparts` such groups (the members of a
-// team, one work-group each, of any sizes): group `part` takes the blocks
+// With kShared == SHARE_BLOCKS the range is shared by `nparts` such groups (the
+// members of a team, one work-group each, of any sizes): group `part` takes the blocks
 // part, part + nparts, ... of kShareVectors vectors each and strides through
 // a block with its own lanes, so the groups work side by side through the
 // arrays.  Group 0 also takes the unaligned head, the last group the tail.
@@ -162,11 +162,25 @@ constexpr size_t kShareVectors = 1024;
 // 6.3-6.4 TB/s for this split and for contiguous chunks alike, against 6.45
 // for one-vector work-groups; issuing a lane's next loads ahead of its stores
 // gained nothing and cost 20-40 registers.)
-template <typename E, ROCSHMEM_OP Op, int kP, bool kNonTemporal, bool kShared = false>
+//
+// With kShared == SHARE_TICKETS the groups do not split the vectors by rule:
+// every wavefront draws the next block of kTicketVectors vectors from a
+// counter that all groups share (`tickets`, zero when the first draw is made),
+// so the blocks are taken in index order whatever the pace of each group, and
+// at any moment the groups together work on one narrow stretch of every array.
+// (Work-groups that loop over a fixed share drift apart; on MI355X the P = 8
+// fp32 fold then runs at 6.2 TB/s against 6.55 for work-groups that are started
+// in index order.)  Each wavefront draws its next block before it loads the
+// current one, so the draw travels with the block's loads.
+enum ShareKind : int { SHARE_NONE = 0, SHARE_BLOCKS = 1, SHARE_TICKETS = 2 };
+constexpr size_t kTicketVectors = 256;
+
+template <typename E, ROCSHMEM_OP Op, int kP, bool kNonTemporal, int kShared = SHARE_NONE>
 __device__ __forceinline__ void fold_window(
     typename ElemTraits<E>::storage *dst0,
     const typename ElemTraits<E>::storage *src0, int64_t hop, int np,
-    size_t lo, size_t hi, size_t lane, size_t nlanes, size_t part = 0, size_t nparts = 1) {
+    size_t lo, size_t hi, size_t lane, size_t nlanes, size_t part = 0, size_t nparts = 1,
+    unsigned long long *tickets = nullptr) {
   using Tr = ElemTraits<E>;
   using S = typename Tr::storage;
   using A = typename Tr::accum;
@@ -207,7 +221,29 @@ __device__ __forceinline__ void fold_window(
   };
   // Calls body(v) for every vector index this lane owns.
   auto for_my_vectors = [&](auto &&body) {
-    if constexpr (kShared) {
+    if constexpr (kShared == SHARE_TICKETS) {
+      unsigned count;
+      const unsigned rank = active_lane_rank(&count);
+      // The lowest active lane draws; the others learn the block from it.
+      auto draw = [&]() -> unsigned long long {
+        unsigned long long t = 0;
+        if (rank == 0)
+          t = __hip_atomic_fetch_add(tickets, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return t;
+      };
+      auto drawn = [&](unsigned long long t) -> size_t {
+        const uint32_t tl = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(t));
+        const uint32_t th = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(t >> 32));
+        return ((static_cast<size_t>(th) << 32) | tl) * kTicketVectors;
+      };
+      size_t b = drawn(draw());
+      while (b < nvec) {
+        const unsigned long long next = draw();
+        const size_t bend = b + kTicketVectors < nvec ? b + kTicketVectors : nvec;
+        for (size_t v = b + rank; v < bend; v += count) body(v);
+        b = drawn(next);
+      }
+    } else if constexpr (kShared == SHARE_BLOCKS) {
       for (size_t b = part * kShareVectors; b < nvec; b += nparts * kShareVectors) {
         const size_t bend = b + kShareVectors < nvec ? b + kShareVectors : nvec;
         for (size_t v = b + lane; v < bend; v += nlanes) body(v);
@@ -265,30 +301,36 @@ __device__ __forceinline__ void fold_window(
     for (size_t k = tlo + lane; k < hi; k += nlanes) scalar_one(k);
 }
 
-// Any range: windows of at most kWindowBytes.
-template <typename E, ROCSHMEM_OP Op, int kP, bool kNonTemporal, bool kShared = false>
+// Any range: windows of at most kWindowBytes.  A range whose blocks are drawn
+// from a counter must fit one window (the counter counts from zero once).
+template <typename E, ROCSHMEM_OP Op, int kP, bool kNonTemporal, int kShared = SHARE_NONE>
 __device__ __forceinline__ void fold_span(
     typename ElemTraits<E>::storage *dst0,
     const typename ElemTraits<E>::storage *src0, int64_t hop, int np,
-    size_t lo, size_t hi, size_t lane, size_t nlanes, size_t part = 0, size_t nparts = 1) {
+    size_t lo, size_t hi, size_t lane, size_t nlanes, size_t part = 0, size_t nparts = 1,
+    unsigned long long *tickets = nullptr) {
   constexpr size_t kWin = kWindowBytes / sizeof(typename ElemTraits<E>::storage);
-  while (hi - lo > kWin) {
-    fold_window<E, Op, kP, kNonTemporal, kShared>(dst0, src0, hop, np, lo, lo + kWin, lane, nlanes,
-                                                  part, nparts);
-    lo += kWin;
+  if constexpr (kShared != SHARE_TICKETS) {
+    while (hi - lo > kWin) {
+      fold_window<E, Op, kP, kNonTemporal, kShared>(dst0, src0, hop, np, lo, lo + kWin, lane, nlanes,
+                                                    part, nparts);
+      lo += kWin;
+    }
   }
   fold_window<E, Op, kP, kNonTemporal, kShared>(dst0, src0, hop, np, lo, hi, lane, nlanes, part,
-                                                nparts);
+                                                nparts, tickets);
 }
 
 // Dispatch on the team size so the common sizes get fully unrolled loads.
-template <typename E, ROCSHMEM_OP Op, bool kNonTemporal, bool kShared = false>
+template <typename E, ROCSHMEM_OP Op, bool kNonTemporal, int kShared = SHARE_NONE>
 __device__ __forceinline__ void fold_span_any(
     typename ElemTraits<E>::storage *dst0,
     const typename ElemTraits<E>::storage *src0, int64_t hop, int np,
-    size_t lo, size_t hi, size_t lane, size_t nlanes, size_t part = 0, size_t nparts = 1) {
-#define ROCSHMEM_AMD_FOLD_CASE(KP) \
-  fold_span<E, Op, KP, kNonTemporal, kShared>(dst0, src0, hop, np, lo, hi, lane, nlanes, part, nparts)
+    size_t lo, size_t hi, size_t lane, size_t nlanes, size_t part = 0, size_t nparts = 1,
+    unsigned long long *tickets = nullptr) {
+#define ROCSHMEM_AMD_FOLD_CASE(KP)                                                               \
+  fold_span<E, Op, KP, kNonTemporal, kShared>(dst0, src0, hop, np, lo, hi, lane, nlanes, part, \
+                                              nparts, tickets)
   switch (np) {
     case 2: ROCSHMEM_AMD_FOLD_CASE(2); break;
     case 4: ROCSHMEM_AMD_FOLD_CASE(4); break;

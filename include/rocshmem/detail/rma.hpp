@@ -46,16 +46,13 @@ __device__ __forceinline__ int translate_pe(rocshmem_ctx_t ctx, int pe) {
 __device__ __forceinline__ bool no_store_order(const Context *c) {
   return (ctx_view(c)->options & static_cast<unsigned>(ROCSHMEM_CTX_NOSTORE)) != 0;
 }
-// True when the heap is ordinary cached device memory (ROCSHMEM_EMU_HEAP_CACHED):
-// an XCD's L2 may then hold a stale copy of a line that another XCD has written
-// through to memory, and a get invalidates before it reads.  On the default
-// uncached heap no L2 ever holds a line of the heap.
-__device__ __forceinline__ bool heap_cached(const Context *c) {
-  return (ctx_view(c)->options & kCtxHeapCached) != 0;
-}
-__device__ __forceinline__ void fresh_reads(const Context *c) {
-  if (heap_cached(c)) fence_acquire();
-}
+// A get reads what memory holds now: the L1 of the CU and the L2 of the XCD may
+// keep a line of the heap that another XCD has since written through to
+// memory (measured with the L2's hit counters: reads of the heap are cached in
+// the L2 whether the heap was allocated cached or uncached), and a loop that
+// polls with gets must not be served that line for ever.  So every get
+// invalidates first (an agent-scope acquire), as every successful wait does.
+__device__ __forceinline__ void fresh_reads() { fence_acquire(); }
 // quiet / fence on context c.
 __device__ __forceinline__ void ctx_release(const Context *c) {
   if (no_store_order(c)) drain_own_stores();
@@ -101,7 +98,7 @@ __device__ __forceinline__ void putmem(Context *c, void *dest, const void *sourc
 }
 __device__ __forceinline__ void getmem(Context *c, void *dest, const void *source,
                                        size_t n, int pe) {
-  fresh_reads(c);
+  fresh_reads();
   copy_thread(dest, remote_addr(c, static_cast<const char *>(source), pe), n);
 }
 // rocshmem_<T>_p / _g: one naturally aligned value.
@@ -109,6 +106,22 @@ template <typename T>
 __device__ __forceinline__ void put_value(Context *c, T *dest, T value, int pe) {
   store_value_through(remote_addr(c, dest, pe), value);
   drain_own_stores();
+}
+
+// One value of 1, 2, 4 or 8 bytes comes as a single load that goes to memory
+// (what a loop that polls with rocshmem_<T>_g needs, at no invalidate);
+// anything wider as a get.
+template <typename T>
+__device__ __forceinline__ T get_value(Context *c, const T *source, int pe) {
+  const T *from = remote_addr(c, source, pe);
+  if constexpr (sizeof(T) == 1 || sizeof(T) == 2 || sizeof(T) == 4 || sizeof(T) == 8) {
+    return load_through(from);
+  } else {
+    T value;
+    fresh_reads();
+    copy_thread(&value, from, sizeof(T));
+    return value;
+  }
 }
 
 // Non-blocking forms: the call only issues the copy; rocshmem_ctx_quiet (or
@@ -121,7 +134,7 @@ __device__ __forceinline__ void putmem_nbi(Context *c, void *dest, const void *s
 }
 __device__ __forceinline__ void getmem_nbi(Context *c, void *dest, const void *source,
                                            size_t n, int pe) {
-  fresh_reads(c);
+  fresh_reads();
   copy_thread(dest, remote_addr(c, static_cast<const char *>(source), pe), n);
 }
 
@@ -135,7 +148,7 @@ __device__ __forceinline__ void putmem_wave(Context *c, void *dest, const void *
 // for whoever reads it after a barrier.
 __device__ __forceinline__ void getmem_wave(Context *c, void *dest, const void *source,
                                             size_t n, int pe) {
-  fresh_reads(c);
+  fresh_reads();
   copy_wave(dest, remote_addr(c, static_cast<const char *>(source), pe), n, g_state.nt_bytes);
   drain_own_stores();
 }
@@ -148,7 +161,7 @@ __device__ __forceinline__ void putmem_nbi_wave(Context *c, void *dest, const vo
 }
 __device__ __forceinline__ void getmem_nbi_wave(Context *c, void *dest, const void *source,
                                                 size_t n, int pe) {
-  fresh_reads(c);
+  fresh_reads();
   copy_wave(dest, remote_addr(c, static_cast<const char *>(source), pe), n, g_state.nt_bytes);
 }
 
@@ -169,7 +182,7 @@ __device__ __forceinline__ void putmem_wg(Context *c, void *dest, const void *so
 }
 __device__ __forceinline__ void getmem_wg(Context *c, void *dest, const void *source,
                                           size_t n, int pe) {
-  fresh_reads(c);
+  fresh_reads();
   copy_lanes(dest, remote_addr(c, static_cast<const char *>(source), pe), n,
              flat_thread_id(), flat_block_size(), g_state.nt_bytes);
   __syncthreads();

@@ -67,7 +67,10 @@ struct SyncPad {
   static constexpr int kMaxPes = 256;
   unsigned long long slots[kMaxPes];
   unsigned long long epoch;
-  unsigned long long pad_[7];
+  // On the first member of a team: the counter from which the members'
+  // wavefronts draw blocks of a large all-reduce (detail/reduce_engine.hpp).
+  unsigned long long tickets;
+  unsigned long long pad_[6];
 };
 
 enum SyncKind : int {
@@ -92,10 +95,6 @@ struct Team {
   void *pWrk;          // ROCSHMEM_REDUCE_MIN_WRKDATA_SIZE * 8 bytes
 };
 
-// Library-internal bit of Context::options, beside the public ROCSHMEM_CTX_*
-// ones: the heap is ordinary cached device memory (ROCSHMEM_EMU_HEAP_CACHED).
-constexpr unsigned kCtxHeapCached = 1u << 30;
-
 // Per-PE communication context (device memory, pooled).  Kernels never write
 // a context: the host fills them all in at initialisation, so device code
 // reads them through the scalar data path (see ctx_view).
@@ -104,7 +103,7 @@ struct Context {
   // load brings all three.
   uint64_t pe_stride;   // bytes between consecutive slices
   int my_pe;
-  unsigned options;     // ROCSHMEM_CTX_* bits and kCtxHeapCached, fixed per object
+  unsigned options;     // ROCSHMEM_CTX_* bits, fixed per object
   char *heap_base;      // base of PE 0's slice
   uint64_t ws_stride;   // bytes between consecutive PEs' work/sync areas
   int num_pes;

@@ -99,14 +99,10 @@ __device__ ATTR_NO_INLINE inline void rocshmem_getmem_nbi(void *dest, const void
   }                                                                                      \
   __device__ ATTR_NO_INLINE inline T rocshmem_ctx_##TN##_g(rocshmem_ctx_t ctx,           \
                                                            const T *source, int pe) {    \
-    T value;                                                                             \
-    rocshmem_ctx_getmem(ctx, &value, source, sizeof(T), pe);                             \
-    return value;                                                                        \
+    return detail::get_value<T>(detail::ctx_of(ctx), source, detail::translate_pe(ctx, pe)); \
   }                                                                                      \
   __device__ ATTR_NO_INLINE inline T rocshmem_##TN##_g(const T *source, int pe) {        \
-    T value;                                                                             \
-    rocshmem_getmem(&value, source, sizeof(T), pe);                                      \
-    return value;                                                                        \
+    return rocshmem_ctx_##TN##_g(rocshmem_ctx_t{nullptr, nullptr}, source, pe);          \
   }
 
 ROCSHMEM_AMD_RMA_TYPES(ROCSHMEM_AMD_TYPED_RMA)

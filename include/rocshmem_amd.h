@@ -492,6 +492,21 @@ int rocshmem_amd_put_signal(int gran, void *dest, const void *source, size_t nby
 int rocshmem_amd_signal_fetch(int gran, const uint64_t *sig_addr, int my_pe,
                               uint64_t *value_out);
 
+/* A loop that polls with gets, and nothing else, must come to see a value that
+ * another PE has put (OpenSHMEM forward progress; the reference's gets end in a
+ * fence, src/ipc/context_ipc_device.cpp:71-78,146-154).  `pairs` (<= 128)
+ * work-groups act for pe_a, each with a poller acting for pe_b.  Per round the
+ * poller reads its own eight words once (so the old value is in its caches),
+ * tells its partner, and then polls with rocshmem_ctx_uint64_g (kind 0),
+ * rocshmem_ctx_getmem of the 64 bytes (1), rocshmem_ctx_getmem_wave (2) or
+ * rocshmem_ctx_getmem_wg (3) until the last word holds the round's number,
+ * which the partner writes with rocshmem_ctx_uint64_p.  No wait_until, no
+ * fence.  words: 8*pairs symmetric uint64, ready: pairs symmetric uint64
+ * (addresses on pe_a).  Every wait is bounded: timed_out_out = 1 if one ran out
+ * (all work-groups then leave). */
+int rocshmem_amd_poll_with_gets(uint64_t *words, uint64_t *ready, int pairs, int rounds, int pe_a,
+                                int pe_b, int kind, int wg_size, int *timed_out_out,
+                                rocshmem_amd_stream_t stream);
 /* Put, quiet, then raise a flag — the pattern quiet exists for (OpenSHMEM
  * message passing; rocshmem_ctx_quiet, include/rocshmem/rocshmem.hpp:408;
  * src/ipc/context_ipc_device.cpp:100-102) — with the receiver checking the

@@ -139,7 +139,7 @@ struct FoldSharesArgs {
 __global__ void fold_shares_kernel(FoldSharesArgs a) {
   const int mine = a.lanes[blockIdx.x];
   if (static_cast<int>(threadIdx.x) >= mine) return;
-  detail::fold_span_any<int, ROCSHMEM_SUM, false, true>(a.dst0, a.src0, a.hop, a.np, 0,
+  detail::fold_span_any<int, ROCSHMEM_SUM, false, detail::SHARE_BLOCKS>(a.dst0, a.src0, a.hop, a.np, 0,
                                                         static_cast<size_t>(a.nelems), threadIdx.x,
                                                         mine, blockIdx.x, a.np);
 }

@@ -673,6 +673,75 @@ int run_wait(int wait_fn, void *ivars, size_t nelems, const int *status, int cmp
   return 0;
 }
 
+// ---------------------------------------------------------------------------
+// A loop that polls with gets must see a value another PE has put
+// ---------------------------------------------------------------------------
+struct PollGetArgs {
+  uint64_t *word_a;      // [pairs][8] words on pe_a (the call's symmetric address)
+  int64_t a_to_b;        // bytes from pe_a's slice to pe_b's
+  uint64_t *ready_a;     // [pairs] on pe_a: round the poller has read the old value in
+  int rounds;
+  int pe_a, pe_b;
+  int kind;              // 0: rocshmem_ctx_uint64_g, 1: getmem of 8 bytes, 2: getmem_wave, 3: getmem_wg (64 bytes)
+  unsigned spin_limit;
+  rocshmem_ctx_t ctx_a, ctx_b;
+  int *timed_out;
+};
+
+// Even work-groups act for pe_a and put; odd ones act for pe_b and poll their
+// own copy of the word with gets from themselves — no wait_until, no fence:
+// what ends the loop is that a get reads memory, not a cached line.  Every
+// wait is bounded.
+__global__ void poll_get_kernel(PollGetArgs a) {
+  const int pair = blockIdx.x >> 1;
+  const bool putter = (blockIdx.x & 1) == 0;
+  uint64_t *word = a.word_a + 8 * pair;  // pe_a's address of the pair's eight words
+  uint64_t *word_on_b = reinterpret_cast<uint64_t *>(reinterpret_cast<char *>(word) + a.a_to_b);
+  uint64_t *ready = a.ready_a + pair;
+  __shared__ uint64_t got[8];
+  for (int r = 1; r <= a.rounds; ++r) {
+    if (putter) {
+      // the poller has the old value in its caches: now change it
+      if (!put_flag_wait(ready, static_cast<uint64_t>(r), a.spin_limit, a.timed_out)) return;
+      if (threadIdx.x < 8)
+        rocshmem_ctx_uint64_p(a.ctx_a, word + threadIdx.x, static_cast<uint64_t>(r), a.pe_b);
+    } else {
+      __shared__ int seen;
+      int outcome = 0;
+      if (threadIdx.x == 0) seen = 0;
+      __syncthreads();
+      for (unsigned spin = 0; spin < a.spin_limit; ++spin) {
+        if (a.kind == 0) {
+          if (threadIdx.x == 0) got[7] = rocshmem_ctx_uint64_g(a.ctx_b, word_on_b + 7, a.pe_b);
+        } else if (a.kind == 1) {
+          if (threadIdx.x == 0) rocshmem_ctx_getmem(a.ctx_b, got, word_on_b, 64, a.pe_b);
+        } else if (a.kind == 2) {
+          if (threadIdx.x < 64) rocshmem_ctx_getmem_wave(a.ctx_b, got, word_on_b, 64, a.pe_b);
+        } else {
+          rocshmem_ctx_getmem_wg(a.ctx_b, got, word_on_b, 64, a.pe_b);
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+          if (got[7] == static_cast<uint64_t>(r)) seen = 1;
+          // first look of the round done: let the putter go
+          if (spin == 0) detail::store_through(reinterpret_cast<uint64_t *>(
+                                                   reinterpret_cast<char *>(ready)), static_cast<uint64_t>(r));
+          if (detail::load_through(a.timed_out)) seen = 2;
+        }
+        __syncthreads();
+        outcome = seen;
+        __syncthreads();  // everybody has read it before anybody can write it again
+        if (outcome) break;
+        __builtin_amdgcn_s_sleep(4);
+      }
+      if (outcome != 1) {
+        if (threadIdx.x == 0) detail::store_through(a.timed_out, 1);
+        return;
+      }
+    }
+  }
+}
+
 }  // namespace drv
 }  // namespace rocshmem
 
@@ -800,6 +869,45 @@ int rocshmem_amd_pingpong(void *buf, uint64_t *sig, size_t nbytes, int iters, in
     DRV_CHECK_HIP(hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev));
     *tick_hz_out = static_cast<double>(khz) * 1e3;
   }
+  return 0;
+}
+
+int rocshmem_amd_poll_with_gets(uint64_t *words, uint64_t *ready, int pairs, int rounds, int pe_a,
+                                int pe_b, int kind, int wg_size, int *timed_out_out,
+                                rocshmem_amd_stream_t stream) {
+  auto &r = runtime::rt();
+  if (!valid_pe(pe_a) || !valid_pe(pe_b) || pe_a == pe_b || pairs < 1 || pairs > 128 ||
+      !valid_launch(2 * pairs, wg_size) || wg_size < 64 || rounds < 0 || kind < 0 || kind > 3 ||
+      !timed_out_out)
+    return -1;
+  if (!sym_ok_on(words, 64u * pairs, pe_a) || !sym_ok_on(ready, 8u * pairs, pe_a)) return -1;
+  if (!grid_fits(poll_get_kernel, 2L * pairs, wg_size)) return -1;
+  const int64_t a_to_b = static_cast<int64_t>(pe_b - pe_a) * static_cast<int64_t>(r.pe_stride);
+  int *d_timed_out;
+  hipStream_t s = as_stream(stream);
+  DRV_CHECK_HIP(hipMalloc(&d_timed_out, sizeof(int)));
+  DRV_CHECK_HIP(hipMemsetAsync(d_timed_out, 0, sizeof(int), s));
+  DRV_CHECK_HIP(hipMemsetAsync(reinterpret_cast<char *>(words) + a_to_b, 0, 64u * pairs, s));
+  DRV_CHECK_HIP(hipMemsetAsync(ready, 0, 8u * pairs, s));
+  PollGetArgs a;
+  a.word_a = words;
+  a.a_to_b = a_to_b;
+  a.ready_a = ready;
+  a.rounds = rounds;
+  a.pe_a = pe_a;
+  a.pe_b = pe_b;
+  a.kind = kind;
+  a.spin_limit = 1u << 20;
+  a.ctx_a = r.driver_ctx_handle(pe_a);
+  a.ctx_b = r.driver_ctx_handle(pe_b);
+  a.timed_out = d_timed_out;
+  hipLaunchKernelGGL(poll_get_kernel, dim3(2 * pairs), dim3(wg_size), 0, s, a);
+  DRV_CHECK_HIP(hipGetLastError());
+  DRV_CHECK_HIP(hipStreamSynchronize(s));
+  int timed_out = 0;
+  DRV_CHECK_HIP(hipMemcpy(&timed_out, d_timed_out, sizeof(timed_out), hipMemcpyDeviceToHost));
+  DRV_CHECK_HIP(hipFree(d_timed_out));
+  *timed_out_out = timed_out;
   return 0;
 }
 

@@ -452,7 +452,7 @@ int Runtime::init(int want_npes, size_t want_heap) {
     c.num_pes = npes;
     c.tinfo = &d_teams[pe].wrt_world;
     c.world_sync = reinterpret_cast<detail::SyncPad *>(d_ws + static_cast<size_t>(pe) * ws_stride);
-    c.options = heap_uncached ? 0u : detail::kCtxHeapCached;
+    c.options = 0;
     c.pool_slot = slot;
   };
   // Rows [0, npes) are the default contexts; rows [npes, 2*npes) are the same

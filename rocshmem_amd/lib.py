@@ -89,6 +89,7 @@ SIGNATURES = {
     "rocshmem_amd_host_wait_test": (_i, [_i, _i, _vp, _sz, _vp, _i, _vp, C.c_long,
                                          C.POINTER(_sz), _vp]),
     "rocshmem_amd_broadcast_active_set": (_i, [_vp, _vp, _sz, _i, _i, _i, _i, _vp]),
+    "rocshmem_amd_poll_with_gets": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, C.POINTER(_i), _vp]),
     "rocshmem_amd_put_flag_check": (_i, [_vp, _vp, _sz, _i, _i, _i, _i, _i, _i,
                                          C.POINTER(_u64), C.POINTER(_i), _vp]),
     "rocshmem_amd_putmem": (_i, [_vp, _vp, _sz, _i, _i, _vp]),

@@ -113,3 +113,8 @@ def test_dispatch_put_signal(rt, L, orc, cached, rows_per_call):
 def test_pingpong(rt, L, orc, cached, nbytes, pairs):
     amo_tests.test_pingpong(rt, L, orc, nbytes, pairs)
     assert cached.heap_is_uncached() == 0
+
+
+@pytest.mark.parametrize("kind", [0, 1, 2, 3])
+def test_polling_with_gets_sees_the_put(rt, L, env, kind):
+    rma_tests.test_polling_with_gets_sees_the_put(rt, L, env, 0, kind, 64, 256)

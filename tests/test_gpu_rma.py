@@ -223,6 +223,29 @@ def test_scattered_messages(rt, L, orc, env, op, gran, ctx_options):
                           None) == -1
 
 
+@pytest.mark.parametrize("kind", [0, 1, 2, 3])
+@pytest.mark.parametrize("ctx_options", [0, 1])
+@pytest.mark.parametrize("pairs,wg", [(1, 64), (64, 256)])
+def test_polling_with_gets_sees_the_put(rt, L, env, ctx_options, kind, pairs, wg):
+    """A poller that has the old value in its caches and then only calls
+    rocshmem_<T>_g / getmem / getmem_wave / getmem_wg in a loop (no wait_until,
+    no fence) sees the value its partner puts, round after round: a get reads
+    memory, not a cached line."""
+    import ctypes as C
+    l = env["l"]
+    words, ready = l.malloc(64 * pairs), l.malloc(8 * pairs)
+    timed_out = C.c_int(99)
+    before = l.set_ctx_options(ctx_options)
+    rc = l.poll_with_gets(l.pe_ptr(words, 1), l.pe_ptr(ready, 1), pairs, 20, 1, 6, kind, wg,
+                          C.byref(timed_out), None)
+    l.set_ctx_options(before)
+    assert rc == 0 and timed_out.value == 0
+    got = rt.get_bytes(l.pe_ptr(words, 6), 64 * pairs, np.uint64)
+    assert (got == 20).all()
+    l.free(words)
+    l.free(ready)
+
+
 def test_every_pe_pair(rt, L, orc, env):
     for me in range(P):
         for pe in range(P):
