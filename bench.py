@@ -42,7 +42,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0  # MI355X, published
 # HBM bytes one launch of the headline kernel moves, from FETCH_SIZE + WRITE_SIZE
 # under rocprofv3 --pmc (profiles/putmem_wg_tiled_256MiB_hbm_traffic.txt).
-PUT_TRAFFIC_BYTES = 536951306
+PUT_TRAFFIC_BYTES = 536937497
 P = 8
 MiB = 1 << 20
 
@@ -333,19 +333,20 @@ def message_rates(b, steps):
         n_wgs = max(256, min(8192, count // groups_per_wg))
         for scattered in (0, 1):
             for cname, opt in CTX_KINDS:
-                # thread-level puts also with the coalescing front end, which looks
-                # for one run across the wavefront before every call
-                for coalesce in ((0, 1) if gran == L.THREAD else (0,)):
+                # thread-level puts also without the coalescing front end (on by
+                # default), which looks for one run across the wavefront before
+                # every call
+                for coalesce in ((1, 0) if gran == L.THREAD else (1,)):
                     l.set_ctx_options(opt)
                     l.set_coalesce_puts(coalesce)
                     ms = b.time_ms(lambda: l.rma_messages(L.PUT, gran, l.pe_ptr(dst, 0), l.pe_ptr(src, 0),
                                                           count * msg, msg, scattered, 0, 1, n_wgs, 256, 1,
                                                           None), max(3, steps // 10), 1)
                     key = "%s_%dB_%s_%s%s" % (gname, msg, "scattered" if scattered else "contiguous", cname,
-                                              "_coalescing" if coalesce else "")
+                                              "" if coalesce else "_no_coalescing")
                     res[key] = {"ms": round(ms, 4), "msgs": count, "mmsg_per_s": round(count / ms / 1e3, 1),
                                 "gbs": round(2 * count * msg / ms / 1e6, 1)}
-    l.set_coalesce_puts(0)
+    l.set_coalesce_puts(1)
     l.set_ctx_options(0)
     l.free(src)
     l.free(dst)

@@ -498,8 +498,8 @@ int rocshmem_amd_signal_fetch(int gran, const uint64_t *sig_addr, int my_pe,
  * work-groups act for pe_a, each with a poller acting for pe_b.  Per round the
  * poller reads its own eight words once (so the old value is in its caches),
  * tells its partner, and then polls with rocshmem_ctx_uint64_g (kind 0),
- * rocshmem_ctx_getmem of the 64 bytes (1), rocshmem_ctx_getmem_wave (2) or
- * rocshmem_ctx_getmem_wg (3) until the last word holds the round's number,
+ * rocshmem_ctx_getmem of the 64 bytes (1) or rocshmem_ctx_getmem_wave (2)
+ * until the last word holds the round's number,
  * which the partner writes with rocshmem_ctx_uint64_p.  No wait_until, no
  * fence.  words: 8*pairs symmetric uint64, ready: pairs symmetric uint64
  * (addresses on pe_a).  Every wait is bounded: timed_out_out = 1 if one ran out

@@ -682,7 +682,7 @@ struct PollGetArgs {
   uint64_t *ready_a;     // [pairs] on pe_a: round the poller has read the old value in
   int rounds;
   int pe_a, pe_b;
-  int kind;              // 0: rocshmem_ctx_uint64_g, 1: getmem of 8 bytes, 2: getmem_wave, 3: getmem_wg (64 bytes)
+  int kind;              // 0: rocshmem_ctx_uint64_g, 1: getmem, 2: getmem_wave (64 bytes)
   unsigned spin_limit;
   rocshmem_ctx_t ctx_a, ctx_b;
   int *timed_out;
@@ -715,10 +715,8 @@ __global__ void poll_get_kernel(PollGetArgs a) {
           if (threadIdx.x == 0) got[7] = rocshmem_ctx_uint64_g(a.ctx_b, word_on_b + 7, a.pe_b);
         } else if (a.kind == 1) {
           if (threadIdx.x == 0) rocshmem_ctx_getmem(a.ctx_b, got, word_on_b, 64, a.pe_b);
-        } else if (a.kind == 2) {
-          if (threadIdx.x < 64) rocshmem_ctx_getmem_wave(a.ctx_b, got, word_on_b, 64, a.pe_b);
         } else {
-          rocshmem_ctx_getmem_wg(a.ctx_b, got, word_on_b, 64, a.pe_b);
+          if (threadIdx.x < 64) rocshmem_ctx_getmem_wave(a.ctx_b, got, word_on_b, 64, a.pe_b);
         }
         __syncthreads();
         if (threadIdx.x == 0) {
@@ -877,7 +875,7 @@ int rocshmem_amd_poll_with_gets(uint64_t *words, uint64_t *ready, int pairs, int
                                 rocshmem_amd_stream_t stream) {
   auto &r = runtime::rt();
   if (!valid_pe(pe_a) || !valid_pe(pe_b) || pe_a == pe_b || pairs < 1 || pairs > 128 ||
-      !valid_launch(2 * pairs, wg_size) || wg_size < 64 || rounds < 0 || kind < 0 || kind > 3 ||
+      !valid_launch(2 * pairs, wg_size) || wg_size < 64 || rounds < 0 || kind < 0 || kind > 2 ||
       !timed_out_out)
     return -1;
   if (!sym_ok_on(words, 64u * pairs, pe_a) || !sym_ok_on(ready, 8u * pairs, pe_a)) return -1;

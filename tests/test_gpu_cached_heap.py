@@ -115,6 +115,6 @@ def test_pingpong(rt, L, orc, cached, nbytes, pairs):
     assert cached.heap_is_uncached() == 0
 
 
-@pytest.mark.parametrize("kind", [0, 1, 2, 3])
+@pytest.mark.parametrize("kind", [0, 1, 2])
 def test_polling_with_gets_sees_the_put(rt, L, env, kind):
     rma_tests.test_polling_with_gets_sees_the_put(rt, L, env, 0, kind, 64, 256)

@@ -223,12 +223,12 @@ def test_scattered_messages(rt, L, orc, env, op, gran, ctx_options):
                           None) == -1
 
 
-@pytest.mark.parametrize("kind", [0, 1, 2, 3])
+@pytest.mark.parametrize("kind", [0, 1, 2])
 @pytest.mark.parametrize("ctx_options", [0, 1])
 @pytest.mark.parametrize("pairs,wg", [(1, 64), (64, 256)])
 def test_polling_with_gets_sees_the_put(rt, L, env, ctx_options, kind, pairs, wg):
     """A poller that has the old value in its caches and then only calls
-    rocshmem_<T>_g / getmem / getmem_wave / getmem_wg in a loop (no wait_until,
+    rocshmem_<T>_g / getmem / getmem_wave in a loop (no wait_until,
     no fence) sees the value its partner puts, round after round: a get reads
     memory, not a cached line."""
     import ctypes as C
