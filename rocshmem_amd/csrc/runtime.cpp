@@ -218,18 +218,18 @@ void Runtime::write_team(int pool_index, int pe, const detail::TeamInfo &world,
 // USE_COHERENT_HEAP, the reference takes HeapMemory<HIPAllocator>, plain
 // hipMalloc (src/memory/heap_type.hpp:41-51); its uncached allocator
 // (src/memory/hip_allocator.hpp:58-65) serves the other configurations.
-// With an uncached heap the L2 of an XCD never holds a line of it, clean or
-// dirty, and that is what makes ordering cheap on this part: an agent-scope
-// release is an L2 write-back (buffer_wbl2), which on MI355X occupies the
-// XCD's L2 for about 0.3 us whenever the L2 holds lines that loads brought in
-// — dirty or not — and for a few ns when it holds none.  Measured, 256 MiB
-// copied in 16 KiB tiles by 1024 work-groups of 256 with one release per tile:
-// 760 us with a cached heap (hipMalloc, or fine-grained), 156 us with an
-// uncached one, 87 us without releases; the copy itself runs at the same rate
-// on either.  Stores to the heap never sit dirty either, plain ones included.
-// The price: a kernel that reads symmetric data more than once (a GEMM over
-// received rows) gets no L2 reuse from the heap; ROCSHMEM_EMU_HEAP_CACHED=1
-// selects plain hipMalloc / hipFree for such programs.
+// What the flag changes on MI355X, measured: an agent-scope release is an L2
+// write-back (buffer_wbl2), which costs about 41 ns device-wide while a copy
+// runs on ordinary cached memory and 4-6 ns on memory allocated uncached
+// (256 MiB copied in 16 KiB tiles by 1024 work-groups of 256 with one release
+// per tile: 760 us against 156 us, 87 us without releases; the copy itself runs
+// at the same rate on either).  Stores to the heap never sit dirty, plain ones
+// included.  Reads are cached all the same: re-reading a tile hits the L2 as
+// often on either kind of heap (67 % in a probe that reads each 64 KiB tile
+// four times), so a consumer of symmetric data loses nothing, and a reader
+// still has to invalidate before it trusts a line (waits, barriers and thread-
+// or wavefront-level gets do).  ROCSHMEM_EMU_HEAP_CACHED=1 selects plain
+// hipMalloc / hipFree.
 //
 // Uncached memory is never given back while the process lives: on this class
 // of machines memory allocated after such a release has shown wrong values.
