@@ -144,6 +144,10 @@ struct DeviceState {
   QueueBinding *queue_table;  // [kQueueTableSize], indexed by queue id modulo the size
   int coalesce_puts;      // thread-level puts first look for one run across the wavefront
   int pad_;
+  // Polls after which a wait or barrier gives up, counts itself in *gave_up and
+  // returns as if satisfied; 0 = wait for ever, as the reference does.
+  uint64_t spin_limit;
+  unsigned long long *gave_up;
 };
 
 #if defined(__HIPCC__)

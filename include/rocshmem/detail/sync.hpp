@@ -344,6 +344,20 @@ __device__ __forceinline__ bool compare(T x, int cmp, T val) {
   }
 }
 
+// Between two polls of a wait.  The reference's waits spin without bound
+// (src/context_tmpl_device.hpp:201-218); so do these unless the runtime has
+// been given a limit (ROCSHMEM_EMU_SPIN_LIMIT): then a wait that has polled
+// that often records the fact (DeviceState::gave_up, which the host reads) and
+// returns, so that a kernel whose partner never comes ends instead of holding
+// the GPU.  Returns false when the caller should stop waiting.
+__device__ __forceinline__ bool keep_waiting(uint64_t *polls) {
+  __builtin_amdgcn_s_sleep(1);
+  const uint64_t limit = g_state.spin_limit;
+  if (limit == 0 || ++*polls < limit) return true;
+  __hip_atomic_fetch_add(g_state.gave_up, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return false;
+}
+
 // One poll.  A successful poll acquires, so data published before the value
 // was written (put_signal payloads) is visible afterwards.
 template <typename T>
@@ -357,7 +371,9 @@ __device__ __forceinline__ int test(T *ivar, int cmp, T val) {
 
 template <typename T>
 __device__ __forceinline__ void wait_until(T *ivar, int cmp, T val) {
-  while (!compare(load_through(ivar), cmp, val)) __builtin_amdgcn_s_sleep(1);
+  uint64_t polls = 0;
+  while (!compare(load_through(ivar), cmp, val))
+    if (!keep_waiting(&polls)) break;
   fence_acquire();
 }
 
@@ -376,12 +392,13 @@ __device__ __forceinline__ size_t wait_until_any(T *ivars, size_t nelems,
   if (!nelems) return SIZE_MAX;
   const size_t pos = first_unmasked(nelems, status);
   if (pos == nelems) return SIZE_MAX;
+  uint64_t polls = 0;
   for (;;) {
     for (size_t i = pos; i < nelems; ++i) {
       if (status && status[i]) continue;
       if (test(ivars + i, cmp, val)) return i;
     }
-    __builtin_amdgcn_s_sleep(1);
+    if (!keep_waiting(&polls)) return SIZE_MAX;
   }
 }
 
@@ -408,12 +425,13 @@ __device__ __forceinline__ size_t wait_until_some(T *ivars, size_t nelems,
   const size_t pos = first_unmasked(nelems, status);
   if (pos == nelems) return 0;
   size_t ncompleted = 0;
+  uint64_t polls = 0;
   while (ncompleted == 0) {
     for (size_t i = pos; i < nelems; ++i) {
       if (status && status[i]) continue;
       if (test(ivars + i, cmp, val)) indices[ncompleted++] = i;
     }
-    if (ncompleted == 0) __builtin_amdgcn_s_sleep(1);
+    if (ncompleted == 0 && !keep_waiting(&polls)) break;
   }
   return ncompleted;
 }
@@ -461,7 +479,9 @@ __device__ __forceinline__ void sync_pes(const Context *c, SyncPad *pad,
       store_through(&peer->slots[my_index], round);
     }
     for (unsigned j = tid; j < static_cast<unsigned>(size); j += nl) {
-      while (load_through(&pad->slots[j]) < round) __builtin_amdgcn_s_sleep(1);
+      uint64_t polls = 0;
+      while (load_through(&pad->slots[j]) < round)
+        if (!keep_waiting(&polls)) break;
     }
     fence_acquire();
     // All lanes of this wavefront have left their polling loops here.

@@ -132,6 +132,17 @@ int rocshmem_amd_set_pe_rule(int rule);
  * the reference's flush off for that option).  Returns the previous options,
  * -1 before init. */
 int64_t rocshmem_amd_set_ctx_options(int64_t options);
+/* The reference's device-side waits and barriers spin without bound
+ * (src/context_tmpl_device.hpp:201-218, src/ipc/context_ipc_device_coll.cpp:31-99),
+ * and by default so do these.  With a limit (polls per wait; initial value
+ * ROCSHMEM_EMU_SPIN_LIMIT, 0 = none) a wait_until* or barrier that has polled
+ * that often counts itself, stops waiting and returns, so that a kernel whose
+ * partner never arrives ends instead of holding the GPU; what it returns with
+ * is then not to be trusted.  rocshmem_amd_waits_given_up returns how many
+ * waits have ended that way since the count was last cleared (clear != 0
+ * clears it); call it after waiting for the kernels.  -1 before rocshmem_init. */
+int rocshmem_amd_set_spin_limit(uint64_t polls);
+int64_t rocshmem_amd_waits_given_up(int clear);
 /* Whether thread-level puts (rocshmem_putmem / rocshmem_<T>_put) first look
  * for one run across the active lanes of the wavefront — messages to the same
  * PE that continue one another, what the reference's coalescing policy merges

@@ -31,6 +31,15 @@ int rocshmem_amd_set_pe_rule(int rule) {
   rt().set_pe_rule(rule);
   return 0;
 }
+int rocshmem_amd_set_spin_limit(uint64_t polls) {
+  if (!rt().live) return -1;
+  rt().set_spin_limit(polls);
+  return 0;
+}
+int64_t rocshmem_amd_waits_given_up(int clear) {
+  if (!rt().live) return -1;
+  return static_cast<int64_t>(rt().waits_given_up(clear != 0));
+}
 int rocshmem_amd_set_coalesce_puts(int on) {
   if (!rt().live) return -1;
   const int before = rt().state.coalesce_puts;

@@ -631,8 +631,9 @@ int run_wait(int wait_fn, void *ivars, size_t nelems, const int *status, int cmp
              uint64_t delay_ticks, size_t *ret_out, size_t *indices_out) {
   if (!local_ok(ivars, (nelems ? nelems : 1) * sizeof(T))) return -1;
   // A blocking form with nobody to wake it would spin for ever on a condition
-  // that does not hold yet: refused, nothing launched.
-  if (!woken && wait_fn != ROCSHMEM_AMD_TEST &&
+  // that does not hold yet: refused, nothing launched — unless the runtime's
+  // waits give up after a limit.
+  if (!woken && wait_fn != ROCSHMEM_AMD_TEST && runtime::rt().state.spin_limit == 0 &&
       !wait_already_satisfied<T>(wait_fn, static_cast<const T *>(ivars), nelems, status, cmp,
                                  *static_cast<const T *>(value)))
     return -2;

@@ -525,6 +525,10 @@ int Runtime::init(int want_npes, size_t want_heap) {
   state.ws_base = d_ws;
   state.nt_bytes = env_size("ROCSHMEM_NT_THRESHOLD", detail::kNonTemporalBytes);
   state.coalesce_puts = env_size("ROCSHMEM_COALESCE_PUTS", 1) != 0 ? 1 : 0;
+  state.spin_limit = env_size("ROCSHMEM_EMU_SPIN_LIMIT", 0);
+  RT_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&d_gave_up), sizeof(unsigned long long)));
+  RT_CHECK_HIP(hipMemset(d_gave_up, 0, sizeof(unsigned long long)));
+  state.gave_up = d_gave_up;
   live = true;
   push_state();
   ROCSHMEM_TEAM_WORLD = team_handle(0, acting_pe);
@@ -536,6 +540,8 @@ void Runtime::finalize() {
   RT_CHECK_HIP(hipDeviceSynchronize());
   RT_CHECK_HIP(hipFree(d_queue_table));
   d_queue_table = nullptr;
+  RT_CHECK_HIP(hipFree(d_gave_up));
+  d_gave_up = nullptr;
   RT_CHECK_HIP(hipHostFree(h_bind_problem));
   h_bind_problem = nullptr;
   RT_CHECK_HIP(hipFree(d_pools));
@@ -694,6 +700,22 @@ void Runtime::set_pe(int pe) {
     state.fixed_pe = pe;
     push_state();
   }
+}
+
+void Runtime::set_spin_limit(uint64_t polls) {
+  require_live("rocshmem_amd_set_spin_limit");
+  if (state.spin_limit != polls) {
+    state.spin_limit = polls;
+    push_state();
+  }
+}
+
+uint64_t Runtime::waits_given_up(bool clear) {
+  require_live("rocshmem_amd_waits_given_up");
+  unsigned long long n = 0;
+  RT_CHECK_HIP(hipMemcpy(&n, d_gave_up, sizeof(n), hipMemcpyDeviceToHost));
+  if (clear && n) RT_CHECK_HIP(hipMemset(d_gave_up, 0, sizeof(n)));
+  return n;
 }
 
 void Runtime::set_coalesce_puts(int on) {

@@ -39,6 +39,7 @@ struct Runtime {
   detail::Context *d_ctx_slots = nullptr;  // [npes][2 * max_ctxs]: per slot one object per ordering option
   detail::CtxPool *d_pools = nullptr;      // [npes]
   detail::QueueBinding *d_queue_table = nullptr;  // [kQueueTableSize]
+  unsigned long long *d_gave_up = nullptr;  // waits and barriers that ran into the spin limit
   int *h_bind_problem = nullptr;  // pinned, [kQueueTableSize]: what each stream binding reported
   std::vector<detail::Team> h_teams;       // host mirror of d_teams
   std::vector<bool> team_slot_used;
@@ -77,6 +78,8 @@ struct Runtime {
   void set_pe(int pe);
   void set_pe_rule(int rule);
   void set_coalesce_puts(int on);
+  void set_spin_limit(uint64_t polls);
+  uint64_t waits_given_up(bool clear);
 
   // Context handle of PE `pe` bound to its member object of team slot `slot`.
   rocshmem_ctx_t default_ctx_handle(int pe, int slot = 0) const {

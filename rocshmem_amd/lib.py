@@ -33,6 +33,8 @@ SIGNATURES = {
     "rocshmem_amd_set_pe_rule": (_i, [_i]),
     "rocshmem_amd_set_ctx_options": (C.c_int64, [C.c_int64]),
     "rocshmem_amd_set_coalesce_puts": (_i, [_i]),
+    "rocshmem_amd_set_spin_limit": (_i, [_u64]),
+    "rocshmem_amd_waits_given_up": (C.c_int64, [_i]),
     "rocshmem_amd_malloc": (_vp, [_sz]),
     "rocshmem_amd_free": (_i, [_vp]),
     "rocshmem_amd_pe_ptr": (_vp, [_vp, _i]),

@@ -89,6 +89,27 @@ def test_reference_examples_compile_unchanged(example, tmp_path):
 
 @pytest.mark.skipif(not os.path.isdir(REFERENCE) or not shutil.which("hipcc"),
                     reason="needs the reference tree and hipcc (build container only)")
+@pytest.mark.parametrize("extra", [["-mcode-object-version=4"], ["-DUSE_FUNC_CALL"]],
+                         ids=["code_object_v4", "real_calls"])
+def test_headers_compile_with_an_older_code_object_and_with_real_calls(extra, tmp_path):
+    """The public headers read the work-group extents from the implicit kernel
+    arguments of code object version 5 and later and fall back to blockDim
+    before that; USE_FUNC_CALL keeps the reference's real calls to the device
+    API (include/rocshmem/rocshmem_common.hpp in the reference).  Either way a
+    reference example compiles for gfx950."""
+    src = os.path.join(REFERENCE, "examples", "rocshmem_allreduce_test.cc")
+    out = tmp_path / "ex.o"
+    cmd = ["hipcc", "--offload-arch=gfx950", "-std=c++17", "-O1", "-x", "hip",
+           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           "-Wno-unused-command-line-argument", "-DROCSHMEM_AMD_NO_MPI_HEADER", *extra,
+           "-I", os.path.join(ROOT, "include"), "-c", src, "-o", str(out)]
+    r = subprocess.run(cmd, capture_output=True, text=True, timeout=600)
+    assert r.returncode == 0, r.stderr[-3000:]
+    assert out.exists()
+
+
+@pytest.mark.skipif(not os.path.isdir(REFERENCE) or not shutil.which("hipcc"),
+                    reason="needs the reference tree and hipcc (build container only)")
 def test_every_function_name_of_the_reference_headers_is_declared(tmp_path):
     """Every rocshmem_* function the reference's public headers declare
     (include/rocshmem/*.hpp, over a thousand once the type tables are stamped

@@ -57,6 +57,42 @@ def test_reduce_grid_that_cannot_be_resident_is_refused_and_launches_nothing(rt,
     rt.down()
 
 
+def test_waits_give_up_after_the_spin_limit(rt, L):
+    """With a spin limit the runtime's waits stop after that many polls, count
+    themselves and return, so a wait that nobody will satisfy ends its kernel
+    normally (the reference's would spin for ever,
+    src/context_tmpl_device.hpp:201-218).  Without a limit nothing changes: the
+    same call is refused before launch, satisfied waits count nothing."""
+    l = rt.up(P, HEAP)
+    vals = np.array([5, 0, 5, 0, 0, 0], np.int64)
+    iv = rt.dev_array(vals)
+    five, nine = np.array([5], np.int64), np.array([9], np.int64)
+    ret = ctypes.c_size_t(77)
+    idx = (ctypes.c_size_t * 6)()
+    assert l.waits_given_up(1) == 0
+    assert l.wait_test(L.WAIT_UNTIL, L.LONG, iv, 1, None, L.CMP_EQ, nine.ctypes.data, ctypes.byref(ret), None) == -2
+    assert l.set_spin_limit(2000) == 0
+    try:
+        assert l.wait_test(L.WAIT_UNTIL, L.LONG, iv, 1, None, L.CMP_EQ, nine.ctypes.data, ctypes.byref(ret),
+                           None) == 0
+        assert l.waits_given_up(0) == 1
+        assert l.wait_test(L.WAIT_UNTIL_ANY, L.LONG, iv, 6, None, L.CMP_EQ, nine.ctypes.data,
+                           ctypes.byref(ret), None) == 0
+        assert ret.value == L.SIZE_MAX          # nothing was satisfied
+        assert l.wait_test(L.WAIT_UNTIL_SOME, L.LONG, iv, 6, None, L.CMP_EQ, nine.ctypes.data,
+                           ctypes.byref(ret), idx) == 0
+        assert ret.value == 0
+        assert l.waits_given_up(1) == 3 and l.waits_given_up(0) == 0
+        # a wait whose condition holds does not count
+        assert l.wait_test(L.WAIT_UNTIL, L.LONG, iv, 1, None, L.CMP_EQ, five.ctypes.data, ctypes.byref(ret),
+                           None) == 0
+        assert l.waits_given_up(0) == 0
+    finally:
+        assert l.set_spin_limit(0) == 0
+    assert l.wait_test(L.WAIT_UNTIL, L.LONG, iv, 1, None, L.CMP_EQ, nine.ctypes.data, ctypes.byref(ret), None) == -2
+    l.dev_free(iv)
+
+
 def test_blocking_wait_that_nobody_will_satisfy_is_refused(rt, L):
     """rocshmem_amd_wait_test launches a wait with no waker: if the condition
     does not hold already the kernel would spin for ever, so the call returns
