@@ -7,6 +7,9 @@
 // address on PE q is   addr + (q - my_pe) * pe_stride   — the closed form of
 // the reference's  ipc_bases[pe] + (dest - ipc_bases[my_pe])  translation
 // (src/ipc/context_ipc_device.cpp:62-69,109-125) for slices at a fixed stride.
+// When every PE is a process of its own (rocshmem_amd/launch.py), a process
+// holds its own slice and has the others' mapped through HIP IPC at whatever
+// addresses it was given; the distance then comes from a table (remote_addr).
 //
 // Every translation unit that includes the public header owns a private
 // __constant__ copy of DeviceState; the host runtime refreshes all registered
@@ -104,7 +107,11 @@ struct Context {
   uint64_t pe_stride;   // bytes between consecutive slices
   int my_pe;
   unsigned options;     // ROCSHMEM_CTX_* bits, fixed per object
-  char *heap_base;      // base of PE 0's slice
+  // With one process per PE the other PEs' slices are mapped wherever HIP put
+  // them: peer_delta[pe] = (where PE pe's slice is mapped here) - (my slice).
+  // nullptr when all slices sit pe_stride apart in one allocation.
+  const int64_t *peer_delta;
+  char *heap_base;      // base of PE 0's slice (of this PE's own slice with one process per PE)
   uint64_t ws_stride;   // bytes between consecutive PEs' work/sync areas
   int num_pes;
   int pool_slot;        // index in the context pool, -1 for default contexts
@@ -207,11 +214,17 @@ __device__ __forceinline__ ContextView *ctx_view(const Context *c) {
   return (ContextView *)c;  // NOLINT: address-space cast
 }
 
-// Address of the same symmetric object on PE `pe`.
+// Address of the same symmetric object on PE `pe`: my address plus the distance
+// between the two slices — the reference's ipc_bases[pe] + (dest - ipc_bases[my_pe])
+// (src/ipc/context_ipc_device.cpp:62-69).  With all slices in one allocation
+// the distance is a product; with one process per PE (and, by the same code,
+// with one GPU per PE) it comes from the context's table of mapped slices.
 template <typename T>
 __device__ __forceinline__ T *remote_addr(const Context *c, T *local, int pe) {
-  const int64_t hop = static_cast<int64_t>(pe - ctx_view(c)->my_pe) *
-                      static_cast<int64_t>(ctx_view(c)->pe_stride);
+  const int64_t *table = ctx_view(c)->peer_delta;
+  const int64_t hop = table ? table[pe]
+                            : static_cast<int64_t>(pe - ctx_view(c)->my_pe) *
+                                  static_cast<int64_t>(ctx_view(c)->pe_stride);
   return reinterpret_cast<T *>(
       reinterpret_cast<char *>(const_cast<typename std::remove_const<T>::type *>(local)) + hop);
 }

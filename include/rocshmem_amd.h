@@ -132,6 +132,35 @@ int rocshmem_amd_set_pe_rule(int rule);
  * the reference's flush off for that option).  Returns the previous options,
  * -1 before init. */
 int64_t rocshmem_amd_set_ctx_options(int64_t options);
+/* One process per PE.  The reference runs one process per PE under an MPI
+ * launcher and exchanges the heaps' IPC handles with MPI_Allgather
+ * (src/ipc_policy.cpp:34-118, src/ipc/backend_ipc.cpp:274-357).  Here
+ * `python -m rocshmem_amd.launch -n P prog args...` starts P processes of an
+ * unchanged program with ROCSHMEM_EMU_PROCS / _RANK / _RDV set; rocshmem_init
+ * then allocates this PE's heap (below 2 GiB), publishes its HIP IPC handle
+ * through the rendezvous file, maps the other PEs' heaps, and device code
+ * finds a peer's slice through a table (detail/state.hpp::remote_addr).  The
+ * host API works between the processes (put / get / atomics / waits on mapped
+ * memory, barriers and collective malloc / free through the rendezvous file,
+ * to_all / reduce / broadcast / alltoall / fcollect by pulling); device-side
+ * collectives and barriers between processes are not supported, and the test
+ * drivers of this header are for the one-process harness.
+ *
+ * The rendezvous on its own (no GPU needed, for tests and other launchers):
+ * a zero-filled file of rocshmem_amd_procs_file_bytes() bytes shared by the
+ * processes; attach maps it for rank `rank` of `nprocs`; barrier meets the
+ * other members of the strided PE set (0, or -1 after ROCSHMEM_EMU_RDV_TIMEOUT_S
+ * seconds, default 120, or once a process has asked the job to end); publish
+ * stores up to 192 bytes in this rank's area and fetch reads a rank's area
+ * (meet in between); request_abort asks every process to leave at its next
+ * meeting, abort_requested returns the status asked for or -1. */
+size_t rocshmem_amd_procs_file_bytes(void);
+int rocshmem_amd_procs_attach(const char *path, int nprocs, int rank);
+int rocshmem_amd_procs_barrier(int PE_start, int PE_stride, int PE_size);
+int rocshmem_amd_procs_publish(const void *bytes, size_t n);
+int rocshmem_amd_procs_fetch(int rank, void *bytes, size_t n);
+int rocshmem_amd_procs_request_abort(int status);
+int rocshmem_amd_procs_abort_requested(void);
 /* The reference's device-side waits and barriers spin without bound
  * (src/context_tmpl_device.hpp:201-218, src/ipc/context_ipc_device_coll.cpp:31-99),
  * and by default so do these.  With a limit (polls per wait; initial value

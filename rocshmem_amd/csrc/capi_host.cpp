@@ -6,6 +6,7 @@
 #include <cstdlib>
 
 #include "drv_common.hpp"
+#include "proc_group.hpp"
 #include "rocshmem_amd.h"
 
 using rocshmem::runtime::rt;
@@ -31,6 +32,25 @@ int rocshmem_amd_set_pe_rule(int rule) {
   rt().set_pe_rule(rule);
   return 0;
 }
+size_t rocshmem_amd_procs_file_bytes(void) { return sizeof(rocshmem::runtime::ProcShared); }
+int rocshmem_amd_procs_attach(const char *path, int nprocs, int rank) {
+  return rocshmem::runtime::procs().attach(path, nprocs, rank);
+}
+int rocshmem_amd_procs_barrier(int PE_start, int PE_stride, int PE_size) {
+  return rocshmem::runtime::procs().barrier(PE_start, PE_stride, PE_size);
+}
+int rocshmem_amd_procs_publish(const void *bytes, size_t n) {
+  return rocshmem::runtime::procs().publish(bytes, n);
+}
+int rocshmem_amd_procs_fetch(int rank, void *bytes, size_t n) {
+  return rocshmem::runtime::procs().fetch(rank, bytes, n);
+}
+int rocshmem_amd_procs_request_abort(int status) {
+  if (!rocshmem::runtime::procs().active()) return -1;
+  rocshmem::runtime::procs().request_abort(status);
+  return 0;
+}
+int rocshmem_amd_procs_abort_requested(void) { return rocshmem::runtime::procs().abort_requested(); }
 int rocshmem_amd_set_spin_limit(uint64_t polls) {
   if (!rt().live) return -1;
   rt().set_spin_limit(polls);

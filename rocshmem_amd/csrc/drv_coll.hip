@@ -3,6 +3,7 @@
 #include <mutex>
 
 #include "drv_common.hpp"
+#include "proc_group.hpp"
 #include "rocshmem_amd.h"
 
 namespace rocshmem {
@@ -400,6 +401,35 @@ void launch_grid_move(char *dest0, const char *src0, int64_t hop, int np, int ro
   DRV_CHECK_HIP(hipGetLastError());
 }
 
+// ---------------------------------------------------------------------------
+// One process per PE: host collectives by pulling.  Every member's process
+// reads the other members' buffers through its own mappings of their slices
+// (which sit at unrelated addresses, hence a table of pointers) and writes its
+// own result; the processes meet before (sources final) and after (everybody
+// has read them).
+// ---------------------------------------------------------------------------
+constexpr int kMaxTableMembers = 64;
+template <typename E>
+struct TableReduceArgs {
+  const typename detail::ElemTraits<E>::storage *src[kMaxTableMembers];  // ascending members
+  typename detail::ElemTraits<E>::storage *out;
+  size_t n;
+  int np;
+};
+template <typename E, ROCSHMEM_OP Op>
+__global__ void table_reduce_kernel(TableReduceArgs<E> a) {
+  using Tr = detail::ElemTraits<E>;
+  using A = typename Tr::accum;
+  const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < a.n; i += stride) {
+    A acc = Tr::widen(a.src[0][i]);
+    for (int p = 1; p < a.np; ++p) acc = detail::combine<A, Op>(acc, Tr::widen(a.src[p][i]));
+    a.out[i] = Tr::narrow(acc);
+  }
+}
+
+void launch_bulk(char *dst, const char *src, size_t nbytes, hipStream_t stream);
+
 // Resolve a team handle (of the acting PE) to what the kernels need.
 struct TeamView {
   const detail::Team *host;
@@ -551,10 +581,17 @@ int wg_move_common(int elem_size, rocshmem_amd_team_t team, void *dest, const vo
 }
 
 template <int kMove>
+int procs_move(void *dest, const void *source, size_t nbytes, int root, int start, int stride, int size,
+               hipStream_t s);
+
+template <int kMove>
 int grid_move_common(rocshmem_amd_team_t team, void *dest, const void *source, size_t nbytes,
                      int root, hipStream_t s) {
   TeamView v;
   if (!view_team(team, &v)) return -1;
+  if (runtime::rt().nprocs)
+    return procs_move<kMove>(dest, source, nbytes, root, v.host->wrt_world.pe_start,
+                             v.host->wrt_world.stride, v.host->num_pes, s);
   {
     const size_t all = nbytes * v.host->num_pes;
     const int me = runtime::rt().me();
@@ -567,6 +604,88 @@ int grid_move_common(rocshmem_amd_team_t team, void *dest, const void *source, s
   const int64_t hop = static_cast<int64_t>(v.host->wrt_world.stride) * r.pe_stride;
   launch_grid_move<kMove>(on_pe0(dest) + first, on_pe0(source) + first, hop, v.host->num_pes,
                           root, nbytes, s);
+  return 0;
+}
+
+// ---- one process per PE -------------------------------------------------------
+struct ProcSet {
+  int start, stride, size, my_index;
+};
+// The caller's place in the strided set of world PEs, or false if it is none.
+bool proc_member(int start, int stride, int size, ProcSet *out) {
+  auto &r = runtime::rt();
+  const int off = r.me() - start;
+  if (size < 1 || size > kMaxTableMembers || stride < 1 || off < 0 || off % stride || off / stride >= size)
+    return false;
+  *out = ProcSet{start, stride, size, off / stride};
+  return true;
+}
+
+int procs_reduce(int dtype, int op, void *dest, const void *source, int nreduce, int start, int stride,
+                 int size, hipStream_t s) {
+  auto &r = runtime::rt();
+  ProcSet set;
+  if (nreduce < 0 || !proc_member(start, stride, size, &set)) return -1;
+  const size_t es = dtype_size(dtype);
+  const size_t bytes = static_cast<size_t>(nreduce) * es;
+  if (!sym_ok(dest, bytes) || !sym_ok(source, bytes)) return -1;
+  const uint64_t dst_off = r.offset_of(dest), src_off = r.offset_of(source);
+  if (nreduce == 0) return 0;
+  char *temp = nullptr;
+  DRV_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&temp), bytes));
+  runtime::procs_meet(start, stride, size);  // every member's source is final
+  const bool ok = for_dtype_op(dtype, op, [&](auto *tag, auto opc) {
+    using T = typename std::remove_pointer<decltype(tag)>::type;
+    using E = typename EngineTag<T>::type;
+    using S = typename detail::ElemTraits<E>::storage;
+    TableReduceArgs<E> a;
+    for (int k = 0; k < size; ++k)
+      a.src[k] = reinterpret_cast<const S *>(r.slice_base(start + k * stride) + src_off);
+    a.out = reinterpret_cast<S *>(temp);
+    a.n = static_cast<size_t>(nreduce);
+    a.np = size;
+    const size_t want = (a.n + 255) / 256;
+    hipLaunchKernelGGL((table_reduce_kernel<E, decltype(opc)::value>),
+                       dim3(static_cast<unsigned>(want < 4096 ? want : 4096)), dim3(256), 0, s, a);
+  });
+  if (ok) DRV_CHECK_HIP(hipGetLastError());
+  DRV_CHECK_HIP(hipStreamSynchronize(s));
+  runtime::procs_meet(start, stride, size);  // everybody has read every source: dest may alias one
+  if (ok) {
+    launch_bulk(r.slice_base(r.me()) + dst_off, temp, bytes, s);
+    DRV_CHECK_HIP(hipStreamSynchronize(s));
+  }
+  DRV_CHECK_HIP(hipFree(temp));
+  return ok ? 0 : -1;
+}
+
+// kMove as in the device forms; nbytes per block; root: index in the set.
+template <int kMove>
+int procs_move(void *dest, const void *source, size_t nbytes, int root, int start, int stride, int size,
+               hipStream_t s) {
+  auto &r = runtime::rt();
+  ProcSet set;
+  if (!proc_member(start, stride, size, &set)) return -1;
+  if (kMove == MOVE_BROADCAST && (root < 0 || root >= size)) return -1;
+  const size_t all = nbytes * size;
+  if (!sym_ok(dest, kMove == MOVE_BROADCAST ? nbytes : all)) return -1;
+  if (!sym_ok(source, kMove == MOVE_ALLTOALL ? all : nbytes)) return -1;
+  const uint64_t dst_off = r.offset_of(dest), src_off = r.offset_of(source);
+  if (!nbytes) return 0;
+  char *mine = r.slice_base(r.me()) + dst_off;
+  runtime::procs_meet(start, stride, size);
+  if (kMove == MOVE_BROADCAST) {
+    if (set.my_index != root)
+      launch_bulk(mine, r.slice_base(start + root * stride) + src_off, nbytes, s);
+  } else {
+    for (int j = 0; j < size; ++j) {
+      const char *from = r.slice_base(start + j * stride) + src_off +
+                         (kMove == MOVE_ALLTOALL ? static_cast<size_t>(set.my_index) * nbytes : 0);
+      launch_bulk(mine + static_cast<size_t>(j) * nbytes, from, nbytes, s);
+    }
+  }
+  DRV_CHECK_HIP(hipStreamSynchronize(s));
+  runtime::procs_meet(start, stride, size);
   return 0;
 }
 
@@ -823,6 +942,8 @@ int rocshmem_amd_to_all(int dtype, int op, void *dest, const void *source, int n
   const int stride = 1 << logPE_stride;
   if (PE_start + static_cast<long>(stride) * (PE_size - 1) >= r.npes) return -1;
   if (nreduce < 0) return -1;
+  if (r.nprocs) return procs_reduce(dtype, op, dest, source, nreduce, PE_start, stride, PE_size,
+                                    as_stream(stream));
   const size_t bytes = static_cast<size_t>(nreduce) * dtype_size(dtype);
   if (!sym_ok_on(dest, bytes, PE_start) || !sym_ok_on(source, bytes, PE_start)) return -1;
   return grid_reduce_common(dtype, op, dest, source, static_cast<int64_t>(stride) * r.pe_stride,
@@ -834,6 +955,9 @@ int rocshmem_amd_reduce(int dtype, int op, rocshmem_amd_team_t team, void *dest,
   TeamView v;
   if (!view_team(team, &v) || nreduce < 0) return -1;
   auto &r = runtime::rt();
+  if (r.nprocs)
+    return procs_reduce(dtype, op, dest, source, nreduce, v.host->wrt_world.pe_start,
+                        v.host->wrt_world.stride, v.host->num_pes, as_stream(stream));
   const size_t bytes = static_cast<size_t>(nreduce) * dtype_size(dtype);
   if (!sym_ok_on(dest, bytes, r.me()) || !sym_ok_on(source, bytes, r.me())) return -1;
   const int64_t first = static_cast<int64_t>(v.host->wrt_world.pe_start) * r.pe_stride;
@@ -858,6 +982,9 @@ int rocshmem_amd_broadcast_active_set(void *dest, const void *source, size_t nby
   const int stride = 1 << logPE_stride;
   if (PE_start + static_cast<long>(stride) * (PE_size - 1) >= r.npes) return -1;
   if (pe_root < 0 || pe_root >= PE_size) return -1;
+  if (r.nprocs)
+    return procs_move<MOVE_BROADCAST>(dest, source, nbytes, pe_root, PE_start, stride, PE_size,
+                                      as_stream(stream));
   if (!sym_ok_on(dest, nbytes, PE_start) || !sym_ok_on(source, nbytes, PE_start)) return -1;
   launch_grid_move<MOVE_BROADCAST>(static_cast<char *>(dest), static_cast<const char *>(source),
                                    static_cast<int64_t>(stride) * r.pe_stride, PE_size, pe_root,

@@ -50,7 +50,8 @@ inline bool local_ok(const void *p, size_t bytes) {
   auto &r = runtime::rt();
   if (!p) return bytes == 0;
   const char *c = static_cast<const char *>(p);
-  if (r.live && c >= r.heap_base && c < r.heap_base + r.pe_stride * r.npes) return sym_ok(p, bytes);
+  (void)c;
+  if (r.live && r.pe_of(p) >= 0) return sym_ok(p, bytes);
   return true;
 }
 

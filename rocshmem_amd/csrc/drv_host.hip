@@ -18,7 +18,8 @@ namespace {
 bool device_accessible(const void *p) {
   auto &r = runtime::rt();
   const char *c = static_cast<const char *>(p);
-  if (r.live && c >= r.heap_base && c < r.heap_base + r.pe_stride * r.npes) return true;
+  (void)c;
+  if (r.live && r.pe_of(p) >= 0) return true;
   hipPointerAttribute_t attr;
   const hipError_t e = hipPointerGetAttributes(&attr, p);
   if (e != hipSuccess) {
@@ -121,8 +122,7 @@ int rocshmem_amd_host_putmem(void *dest, const void *source, size_t nbytes, int 
   if (!nbytes) return 0;
   if (!source || !sym_ok_on(dest, nbytes, my_pe)) return -1;
   auto &r = runtime::rt();
-  char *target = static_cast<char *>(dest) +
-                 static_cast<int64_t>(pe - my_pe) * static_cast<int64_t>(r.pe_stride);
+  char *target = static_cast<char *>(r.pe_ptr(dest, pe));
   g_host.ensure();
   if (device_accessible(source)) {
     if (!local_ok(source, nbytes)) return -1;
@@ -139,8 +139,7 @@ int rocshmem_amd_host_getmem(void *dest, const void *source, size_t nbytes, int 
   if (!nbytes) return 0;
   if (!dest || !sym_ok_on(source, nbytes, my_pe)) return -1;
   auto &r = runtime::rt();
-  const char *origin = static_cast<const char *>(source) +
-                       static_cast<int64_t>(pe - my_pe) * static_cast<int64_t>(r.pe_stride);
+  const char *origin = static_cast<const char *>(r.pe_ptr(source, pe));
   g_host.ensure();
   if (device_accessible(dest)) {
     if (!local_ok(dest, nbytes)) return -1;

@@ -6,6 +6,7 @@
 // MPI or HIP IPC: there is one heap allocation of P slices at a fixed stride,
 // so the table of peer base addresses collapses to (base, stride).
 #include "runtime.hpp"
+#include "proc_group.hpp"
 
 #include <hip/hip_runtime.h>
 
@@ -332,6 +333,8 @@ int Runtime::init(int want_npes, size_t want_heap) {
     fprintf(stderr, "rocshmem: no GPU available\n");
     abort();
   }
+  // Started as one PE of a job of processes?  Then the job says how many PEs.
+  if (procs().attach_from_env()) want_npes = procs().nprocs();
   npes = want_npes > 0 ? want_npes
                        : (g_requested_npes > 0
                               ? g_requested_npes
@@ -345,80 +348,159 @@ int Runtime::init(int want_npes, size_t want_heap) {
   if (max_ctxs > detail::CtxPool::kMaxWords * 64) max_ctxs = detail::CtxPool::kMaxWords * 64;
   max_teams = static_cast<int>(env_size("ROCSHMEM_MAX_NUM_TEAMS", 40));
   if (max_teams < 1) max_teams = 1;
-  // Slice placement.  Slices start on 2 MiB boundaries and sit `pe_stride`
-  // apart inside ONE device allocation.  By default the allocation holds the
-  // slices and nothing else: stride = heap size rounded up to 2 MiB.
-  //
-  // ROCSHMEM_EMU_SPREAD=1 trades device memory for bandwidth: the slices are
-  // spread over about half of the device memory on a 4 GiB grid (16 GiB apart
-  // for 8 PEs) and, when the GPU is otherwise empty, the block is placed by
-  // allocating half of the memory plus 1 GiB.  On MI355X a kernel that writes
-  // to all P slices at once (all-reduce, alltoall) then sustains about 10 %
-  // more HBM bandwidth (measured: 6.45 instead of 5.7-5.9 TB/s for the P = 8
-  // fp32 all-reduce) and is steadier from run to run.  That is a property of
-  // hosting P PEs inside one memory; it is off unless asked for.
-  // ROCSHMEM_EMU_PE_STRIDE=<bytes> sets the stride directly;
-  // ROCSHMEM_EMU_HEAP_ANCHOR=0 keeps the spread but not the placement.
-  const size_t two_mib = size_t{2} << 20;
-  const size_t min_stride = round_up(heap_size, two_mib);
-  const bool spread = env_size("ROCSHMEM_EMU_SPREAD", 0) != 0;
-  size_t want = env_size("ROCSHMEM_EMU_PE_STRIDE", 0);
-  size_t free_b = 0, total_b = 0;
-  RT_CHECK_HIP(hipMemGetInfo(&free_b, &total_b));
-  if (!want && spread) {
-    const size_t budget = total_b / 2;
-    const size_t grid = size_t{4} << 30;
-    want = npes <= 2 ? size_t{16} << 30 : budget / npes;
-    if (want >= grid) want = want / grid * grid;
-    if (want * npes > budget) want = budget / npes;
-  }
-  pe_stride = std::max(min_stride, want / two_mib * two_mib);
+  size_t alloc_bytes = 0;
+  bool anchored = false;
   acting_pe = 0;
   driver_ctx_options = 0;
-
-  // Three tries: the spread block placed in the upper half of the memory, the
-  // spread block, the packed slices.  Each first looks for an idle block from
-  // an earlier rocshmem_init of this process.
-  const size_t anchor = total_b / 2 + (size_t{1} << 30);
-  const bool want_anchor = spread && env_size("ROCSHMEM_EMU_HEAP_ANCHOR", 1) != 0 &&
-                           pe_stride * npes >= total_b / 4 && pe_stride * npes < anchor;
-  bool anchored = false;
   heap_base = nullptr;
-  size_t alloc_bytes = 0;
-  auto try_block = [&](size_t bytes) {
-    size_t had = 0;
-    if (!heap_cached_mode() && (heap_base = reuse_heap_block(bytes, &had))) {
-      alloc_bytes = had;
-      return true;
+  peer_base.clear();
+  nprocs = 0;
+  if (procs().active()) {
+    // One process per PE: this process allocates its own slice, publishes its
+    // IPC handle, and maps the slices of the others wherever HIP puts them
+    // (the reference does the same with MPI_Allgather of the handles,
+    // src/ipc_policy.cpp:34-118).  Allocations shared this way stay below
+    // 2 GiB: opening larger ones has not returned on this class of machines.
+    nprocs = procs().nprocs();
+    acting_pe = procs().rank();
+    const size_t two_mib = size_t{2} << 20;
+    pe_stride = round_up(heap_size, two_mib);
+    if (pe_stride >= (size_t{2} << 30)) {
+      fprintf(stderr,
+              "rocshmem: with one process per PE the heap of a PE must stay below 2 GiB "
+              "(ROCSHMEM_HEAP_SIZE=%zu asked for)\n", heap_size);
+      fflush(nullptr);
+      _Exit(EXIT_FAILURE);
     }
-    if (new_heap_block(&heap_base, bytes) == hipSuccess) {
-      alloc_bytes = bytes;
-      return true;
+    // The slice and the mappings of the other PEs' slices live until the
+    // process ends: a later rocshmem_init of the same job finds them again
+    // (same size, same handles), so nothing shared is ever unmapped or freed
+    // while another process may hold it, and no uncached block is given back.
+    struct Kept {
+      char *own = nullptr;
+      size_t bytes = 0;
+      bool cached = false;
+      std::vector<hipIpcMemHandle_t> handle;
+      std::vector<char *> mapped;
+    };
+    static Kept kept;
+    if (kept.own && (kept.bytes != pe_stride || kept.cached != heap_cached_mode())) {
+      fprintf(stderr, "rocshmem: a process that is one PE of a job keeps the heap size and kind of "
+                      "its first rocshmem_init (%zu bytes)\n", kept.bytes);
+      fflush(nullptr);
+      _Exit(EXIT_FAILURE);
     }
-    (void)hipGetLastError();
-    heap_base = nullptr;
-    return false;
-  };
-  if (want_anchor) {
-    size_t had = 0;
-    if (!heap_cached_mode() && (heap_base = reuse_heap_block(anchor, &had))) {
-      alloc_bytes = had;
-      anchored = true;
-    } else if (free_b > anchor + (size_t{16} << 30)) {
-      anchored = try_block(anchor);
+    if (!kept.own) {
+      const hipError_t e = heap_cached_mode()
+                               ? hipMalloc(reinterpret_cast<void **>(&kept.own), pe_stride)
+                               : hipExtMallocWithFlags(reinterpret_cast<void **>(&kept.own), pe_stride,
+                                                       hipDeviceMallocUncached);
+      if (e != hipSuccess || !kept.own) {
+        fprintf(stderr, "rocshmem: PE %d cannot allocate %zu bytes for its heap: %s\n", acting_pe,
+                pe_stride, hipGetErrorString(e));
+        fflush(nullptr);
+        _Exit(EXIT_FAILURE);
+      }
+      kept.bytes = pe_stride;
+      kept.cached = heap_cached_mode();
+      kept.handle.resize(npes);
+      kept.mapped.assign(npes, nullptr);
+      RT_CHECK_HIP(hipIpcGetMemHandle(&kept.handle[acting_pe], kept.own));
     }
-  }
-  if (!heap_base && !try_block(pe_stride * npes) && pe_stride != min_stride) {
-    fprintf(stderr,
-            "rocshmem: no room for %d slices %zu bytes apart; packing them (stride = heap size)\n",
-            npes, pe_stride);
-    pe_stride = min_stride;
-    try_block(pe_stride * npes);
-  }
-  if (!heap_base) {
-    fprintf(stderr, "rocshmem: cannot allocate %zu bytes of device memory for the symmetric heap\n",
-            pe_stride * npes);
-    exit(EXIT_FAILURE);
+    char *own = kept.own;
+    RT_CHECK_HIP(hipMemset(own, 0, pe_stride));
+    RT_CHECK_HIP(hipDeviceSynchronize());
+    static_assert(sizeof(hipIpcMemHandle_t) <= kBlobBytes, "IPC handle larger than a publish area");
+    procs().publish(&kept.handle[acting_pe], sizeof(hipIpcMemHandle_t));
+    if (procs().barrier_world() != 0) _Exit(EXIT_FAILURE);
+    peer_base.assign(npes, nullptr);
+    peer_base[acting_pe] = own;
+    for (int p = 0; p < npes; ++p) {
+      if (p == acting_pe) continue;
+      hipIpcMemHandle_t theirs;
+      procs().fetch(p, &theirs, sizeof(theirs));
+      if (!kept.mapped[p] || memcmp(&theirs, &kept.handle[p], sizeof(theirs)) != 0) {
+        RT_CHECK_HIP(hipIpcOpenMemHandle(reinterpret_cast<void **>(&kept.mapped[p]), theirs,
+                                         hipIpcMemLazyEnablePeerAccess));
+        kept.handle[p] = theirs;
+      }
+      peer_base[p] = kept.mapped[p];
+    }
+    // Everybody has read everybody's handle before anybody publishes again.
+    if (procs().barrier_world() != 0) _Exit(EXIT_FAILURE);
+    heap_base = own;
+    alloc_bytes = pe_stride;
+  } else {
+    // Slice placement.  Slices start on 2 MiB boundaries and sit `pe_stride`
+    // apart inside ONE device allocation.  By default the allocation holds the
+    // slices and nothing else: stride = heap size rounded up to 2 MiB.
+    //
+    // ROCSHMEM_EMU_SPREAD=1 trades device memory for bandwidth: the slices are
+    // spread over about half of the device memory on a 4 GiB grid (16 GiB apart
+    // for 8 PEs) and, when the GPU is otherwise empty, the block is placed by
+    // allocating half of the memory plus 1 GiB.  On MI355X a kernel that writes
+    // to all P slices at once (all-reduce, alltoall) then sustains about 10 %
+    // more HBM bandwidth (measured: 6.45 instead of 5.7-5.9 TB/s for the P = 8
+    // fp32 all-reduce) and is steadier from run to run.  That is a property of
+    // hosting P PEs inside one memory; it is off unless asked for.
+    // ROCSHMEM_EMU_PE_STRIDE=<bytes> sets the stride directly;
+    // ROCSHMEM_EMU_HEAP_ANCHOR=0 keeps the spread but not the placement.
+    const size_t two_mib = size_t{2} << 20;
+    const size_t min_stride = round_up(heap_size, two_mib);
+    const bool spread = env_size("ROCSHMEM_EMU_SPREAD", 0) != 0;
+    size_t want = env_size("ROCSHMEM_EMU_PE_STRIDE", 0);
+    size_t free_b = 0, total_b = 0;
+    RT_CHECK_HIP(hipMemGetInfo(&free_b, &total_b));
+    if (!want && spread) {
+      const size_t budget = total_b / 2;
+      const size_t grid = size_t{4} << 30;
+      want = npes <= 2 ? size_t{16} << 30 : budget / npes;
+      if (want >= grid) want = want / grid * grid;
+      if (want * npes > budget) want = budget / npes;
+    }
+    pe_stride = std::max(min_stride, want / two_mib * two_mib);
+
+    // Three tries: the spread block placed in the upper half of the memory, the
+    // spread block, the packed slices.  Each first looks for an idle block from
+    // an earlier rocshmem_init of this process.
+    const size_t anchor = total_b / 2 + (size_t{1} << 30);
+    const bool want_anchor = spread && env_size("ROCSHMEM_EMU_HEAP_ANCHOR", 1) != 0 &&
+                             pe_stride * npes >= total_b / 4 && pe_stride * npes < anchor;
+    auto try_block = [&](size_t bytes) {
+      size_t had = 0;
+      if (!heap_cached_mode() && (heap_base = reuse_heap_block(bytes, &had))) {
+        alloc_bytes = had;
+        return true;
+      }
+      if (new_heap_block(&heap_base, bytes) == hipSuccess) {
+        alloc_bytes = bytes;
+        return true;
+      }
+      (void)hipGetLastError();
+      heap_base = nullptr;
+      return false;
+    };
+    if (want_anchor) {
+      size_t had = 0;
+      if (!heap_cached_mode() && (heap_base = reuse_heap_block(anchor, &had))) {
+        alloc_bytes = had;
+        anchored = true;
+      } else if (free_b > anchor + (size_t{16} << 30)) {
+        anchored = try_block(anchor);
+      }
+    }
+    if (!heap_base && !try_block(pe_stride * npes) && pe_stride != min_stride) {
+      fprintf(stderr,
+              "rocshmem: no room for %d slices %zu bytes apart; packing them (stride = heap size)\n",
+              npes, pe_stride);
+      pe_stride = min_stride;
+      try_block(pe_stride * npes);
+    }
+    if (!heap_base) {
+      fprintf(stderr, "rocshmem: cannot allocate %zu bytes of device memory for the symmetric heap\n",
+              pe_stride * npes);
+      exit(EXIT_FAILURE);
+    }
   }
   heap_alloc_bytes = alloc_bytes;
   heap_uncached = !heap_cached_mode();
@@ -426,7 +508,9 @@ int Runtime::init(int want_npes, size_t want_heap) {
     fprintf(stderr, "rocshmem: %d PEs, heap %zu B per PE, slices %zu B apart, %zu B allocated%s%s\n",
             npes, heap_size, pe_stride, alloc_bytes, anchored ? " (placed)" : "",
             heap_cached_mode() ? " (cached)" : " (uncached)");
-  allocator.reset(reinterpret_cast<uint64_t>(heap_base), heap_size);
+  // With one process per PE every process runs the allocator for itself and
+  // all must arrive at the same offsets: the same model base everywhere.
+  allocator.reset(nprocs ? (uint64_t{1} << 40) : reinterpret_cast<uint64_t>(heap_base), heap_size);
 
   ws_stride = ws_bytes_per_pe();
   RT_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&d_ws), ws_stride * npes));
@@ -443,8 +527,18 @@ int Runtime::init(int want_npes, size_t want_heap) {
   const detail::TeamInfo world{0, 1, npes, 0};
   for (int pe = 0; pe < npes; ++pe) write_team(0, pe, world, world, pe);
 
+  // With one process per PE: where every PE's slice sits relative to this
+  // PE's, the table behind remote_addr (nullptr otherwise: equal strides).
+  d_peer_delta = nullptr;
+  if (nprocs) {
+    std::vector<int64_t> delta(npes);
+    for (int p = 0; p < npes; ++p) delta[p] = peer_base[p] - peer_base[acting_pe];
+    RT_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&d_peer_delta), sizeof(int64_t) * npes));
+    RT_CHECK_HIP(hipMemcpy(d_peer_delta, delta.data(), sizeof(int64_t) * npes, hipMemcpyHostToDevice));
+  }
   // Contexts: one default context and one pool per PE.
   auto fill_ctx = [&](detail::Context &c, int pe, int slot) {
+    c.peer_delta = d_peer_delta;
     c.heap_base = heap_base;
     c.pe_stride = pe_stride;
     c.ws_stride = ws_stride;
@@ -517,7 +611,7 @@ int Runtime::init(int want_npes, size_t want_heap) {
   // With a host thread per PE, kernels learn their PE from the queue their
   // launching thread bound (rocshmem_emu_bind_stream).
   state.pe_rule = pe_threads_count() > 0 ? detail::PE_RULE_QUEUE : detail::PE_RULE_FIXED;
-  state.fixed_pe = 0;
+  state.fixed_pe = acting_pe;
   state.max_teams = max_teams;
   state.default_ctx = d_default_ctx;
   state.world_team = d_teams;
@@ -532,12 +626,22 @@ int Runtime::init(int want_npes, size_t want_heap) {
   live = true;
   push_state();
   ROCSHMEM_TEAM_WORLD = team_handle(0, acting_pe);
+  if (nprocs && procs().barrier_world() != 0) _Exit(EXIT_FAILURE);
   return 0;
 }
 
 void Runtime::finalize() {
   if (!live) return;
   RT_CHECK_HIP(hipDeviceSynchronize());
+  if (nprocs) {
+    // Nobody leaves while another PE may still be writing to its slice.  The
+    // slice and the mappings stay (see rocshmem_init).
+    (void)procs().barrier_world();
+    RT_CHECK_HIP(hipFree(d_peer_delta));
+    d_peer_delta = nullptr;
+    heap_base = nullptr;
+    peer_base.clear();
+  }
   RT_CHECK_HIP(hipFree(d_queue_table));
   d_queue_table = nullptr;
   RT_CHECK_HIP(hipFree(d_gave_up));
@@ -549,8 +653,9 @@ void Runtime::finalize() {
   RT_CHECK_HIP(hipFree(d_default_ctx));
   RT_CHECK_HIP(hipFree(d_teams));
   RT_CHECK_HIP(hipFree(d_ws));
-  release_heap_block(heap_base);
+  if (heap_base) release_heap_block(heap_base);
   heap_base = nullptr;
+  nprocs = 0;
   d_ws = nullptr;
   d_teams = nullptr;
   h_teams.clear();
@@ -589,7 +694,7 @@ void *Runtime::sym_malloc(size_t size) {
   require_live("rocshmem_malloc");
   const uint64_t off = allocator.alloc(size);
   if (off == Pow2Allocator::kNoBlock) return nullptr;
-  return heap_base + static_cast<size_t>(me()) * pe_stride + off;
+  return slice_base(me()) + off;
 }
 
 void Runtime::sym_free(void *ptr) {
@@ -603,13 +708,19 @@ void Runtime::sym_free(void *ptr) {
 }
 
 uint64_t Runtime::offset_of(const void *ptr) const {
-  const char *p = static_cast<const char *>(ptr);
-  if (p < heap_base || p >= heap_base + pe_stride * npes) return Pow2Allocator::kNoBlock;
-  return static_cast<uint64_t>(p - heap_base) % pe_stride;
+  const int pe = pe_of(ptr);
+  if (pe < 0) return Pow2Allocator::kNoBlock;
+  return static_cast<uint64_t>(static_cast<const char *>(ptr) - slice_base(pe));
 }
 
 int Runtime::pe_of(const void *ptr) const {
   const char *p = static_cast<const char *>(ptr);
+  if (nprocs) {
+    // the slices are mapped wherever HIP put them: look the address up
+    for (int pe = 0; pe < npes; ++pe)
+      if (p >= peer_base[pe] && p < peer_base[pe] + pe_stride) return pe;
+    return -1;
+  }
   if (p < heap_base || p >= heap_base + pe_stride * npes) return -1;
   return static_cast<int>(static_cast<uint64_t>(p - heap_base) / pe_stride);
 }
@@ -617,7 +728,7 @@ int Runtime::pe_of(const void *ptr) const {
 void *Runtime::pe_ptr(const void *ptr, int pe) const {
   const uint64_t off = offset_of(ptr);
   if (off == Pow2Allocator::kNoBlock || pe < 0 || pe >= npes) return nullptr;
-  return heap_base + static_cast<size_t>(pe) * pe_stride + off;
+  return slice_base(pe) + off;
 }
 
 // src/rocshmem.cpp:221-303.  One call creates the team object of every member.
@@ -694,6 +805,11 @@ void Runtime::set_pe(int pe) {
     fprintf(stderr, "rocshmem: PE %d out of range\n", pe);
     abort();
   }
+  if (nprocs && pe != acting_pe) {
+    fprintf(stderr, "rocshmem: this process is PE %d of a job of processes and cannot act as PE %d\n",
+            acting_pe, pe);
+    abort();
+  }
   acting_pe = pe;
   ROCSHMEM_TEAM_WORLD = team_handle(0, pe);
   if (state.fixed_pe != pe) {
@@ -740,6 +856,21 @@ void Runtime::set_pe_rule(int rule) {
 
 }  // namespace runtime
 
+namespace runtime {
+// Meetings of the processes of a job (no-ops when all PEs live in this
+// process).  A meeting that fails — a process asked the job to end, or the
+// wait ran out — ends this process too.
+void procs_meet(int start, int stride, int size) {
+  if (!g_rt.live || !g_rt.nprocs) return;
+  if (procs().barrier(start, stride, size) != 0) {
+    const int asked = procs().abort_requested();
+    fflush(nullptr);
+    _Exit(asked >= 0 ? asked : EXIT_FAILURE);
+  }
+}
+void procs_meet_world() { procs_meet(0, 1, g_rt.npes); }
+}  // namespace runtime
+
 namespace detail {
 void register_state_uploader(StateUploader fn) {
   std::lock_guard<std::mutex> guard(runtime::g_uploader_lock);
@@ -783,7 +914,7 @@ __host__ void rocshmem_init(MPI_Comm) {
   }
   WorldMeeting w;
   if (w.mine) {
-    rt().init(runtime::pe_threads_count(), 0);
+    rt().init(runtime::pe_threads_count(), 0);  // one process per PE: meets the others inside
     w.done();
   }
   // A program built with -fgpu-default-stream=per-thread launches its
@@ -801,7 +932,7 @@ __host__ void rocshmem_query_thread(int *provided) { *provided = ROCSHMEM_THREAD
 __host__ void rocshmem_dump_stats() {}
 __host__ void rocshmem_reset_stats() {}
 __host__ void rocshmem_finalize() {
-  WorldMeeting w;
+  WorldMeeting w;  // (one process per PE: Runtime::finalize meets the others itself)
   if (w.mine) {
     rt().finalize();
     w.done();
@@ -815,10 +946,15 @@ __host__ void *rocshmem_malloc(size_t size) {
     void *mine = rt().sym_malloc(size);
     w.done(mine ? rt().offset_of(mine) + 1 : 0);
   }
+  // One process per PE: every process has run its own allocator to the same
+  // offset; the call is also a meeting, as in the reference
+  // (src/rocshmem.cpp: a barrier ends rocshmem_malloc).
+  runtime::procs_meet_world();
   if (!w.result) return nullptr;
-  return rt().heap_base + static_cast<size_t>(rt().me()) * rt().pe_stride + (w.result - 1);
+  return rt().slice_base(rt().me()) + (w.result - 1);
 }
 __host__ void rocshmem_free(void *ptr) {
+  runtime::procs_meet_world();  // nobody frees what another PE may still be using
   WorldMeeting w;
   if (w.mine) {
     rt().sym_free(ptr);
@@ -828,12 +964,14 @@ __host__ void rocshmem_free(void *ptr) {
 // Usable before rocshmem_init, as in the reference (src/rocshmem.cpp:113-121).
 __host__ int rocshmem_n_pes() {
   if (rt().live) return rt().npes;
+  if (runtime::procs().attach_from_env()) return runtime::procs().nprocs();
   if (runtime::pe_threads_count() > 0) return runtime::pe_threads_count();
   if (runtime::g_requested_npes > 0) return runtime::g_requested_npes;
   return static_cast<int>(runtime::env_size("ROCSHMEM_EMU_NPES", 1));
 }
 __host__ int rocshmem_my_pe() {
   if (runtime::tl_pe >= 0) return runtime::tl_pe;
+  if (!rt().live && runtime::procs().attach_from_env()) return runtime::procs().rank();
   return rt().live ? rt().acting_pe : 0;
 }
 __host__ int rocshmem_ctx_create(int64_t options, rocshmem_ctx_t *ctx) {
@@ -871,8 +1009,12 @@ __host__ int rocshmem_team_split_strided(rocshmem_team_t parent_team, int start,
                                          rocshmem_team_t *new_team) {
   parent_team = rt().my_view(parent_team);
   const detail::Team *pt = rt().host_team(parent_team);
-  if (!pt || runtime::tl_pe < 0)
-    return rt().team_split_strided(parent_team, start, stride, size, new_team);
+  if (!pt || runtime::tl_pe < 0) {
+    // (one process per PE: each member makes its own objects, then they meet)
+    const int rc = rt().team_split_strided(parent_team, start, stride, size, new_team);
+    if (pt) runtime::procs_meet(pt->wrt_world.pe_start, pt->wrt_world.stride, pt->wrt_world.size);
+    return rc;
+  }
   const detail::TeamInfo w = pt->wrt_world;
   uint64_t packed = 0;  // (return code + 1) << 32 | (slot + 1)
   if (runtime::pe_threads_enter(w.pe_start, w.stride, w.size, &packed)) {
@@ -928,6 +1070,7 @@ __host__ void rocshmem_barrier_all() {
     if (runtime::tl_pe < 0) RT_CHECK_HIP(hipDeviceSynchronize());
     w.done();
   }
+  runtime::procs_meet_world();
 }
 __host__ void rocshmem_sync_all() { rocshmem_barrier_all(); }
 // Ends the whole job at once, as the reference's MPI_Abort does
@@ -935,6 +1078,7 @@ __host__ void rocshmem_sync_all() { rocshmem_barrier_all(); }
 // no destructors run.
 __host__ void rocshmem_global_exit(int status) {
   fflush(nullptr);
+  runtime::procs().request_abort(status);  // the other processes of the job leave at their next meeting
   _Exit(status);
 }
 

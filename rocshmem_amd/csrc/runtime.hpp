@@ -33,6 +33,14 @@ struct Runtime {
   size_t heap_alloc_bytes = 0;  // size of the device allocation that holds the slices
   bool heap_uncached = true;    // false under ROCSHMEM_EMU_HEAP_CACHED=1
   char *heap_base = nullptr;
+  // One process per PE (proc_group.hpp): this process holds its own slice and
+  // has the others' mapped through HIP IPC wherever HIP put them.
+  int nprocs = 0;                   // 0: all PEs live in this process
+  std::vector<char *> peer_base;    // [npes] in process mode: where each PE's slice is mapped here
+  int64_t *d_peer_delta = nullptr;  // device, [npes]: peer_base[p] - peer_base[me]
+  char *slice_base(int pe) const {
+    return nprocs ? peer_base[pe] : heap_base + static_cast<size_t>(pe) * pe_stride;
+  }
   char *d_ws = nullptr;
   detail::Team *d_teams = nullptr;         // [max_teams][npes]
   detail::Context *d_default_ctx = nullptr;  // [2*npes]: default, then NOSTORE
@@ -111,6 +119,11 @@ struct Runtime {
 };
 
 Runtime &rt();
+
+// One process per PE: meet the other processes of the strided PE set / of the
+// world (nothing to do when all PEs live in this process).
+void procs_meet(int start, int stride, int size);
+void procs_meet_world();
 
 // Uncached heap blocks this process holds (they are kept until it ends): all
 // of them, and those no live runtime uses.

@@ -33,6 +33,13 @@ SIGNATURES = {
     "rocshmem_amd_set_pe_rule": (_i, [_i]),
     "rocshmem_amd_set_ctx_options": (C.c_int64, [C.c_int64]),
     "rocshmem_amd_set_coalesce_puts": (_i, [_i]),
+    "rocshmem_amd_procs_file_bytes": (_sz, []),
+    "rocshmem_amd_procs_attach": (_i, [C.c_char_p, _i, _i]),
+    "rocshmem_amd_procs_barrier": (_i, [_i, _i, _i]),
+    "rocshmem_amd_procs_publish": (_i, [_vp, _sz]),
+    "rocshmem_amd_procs_fetch": (_i, [_i, _vp, _sz]),
+    "rocshmem_amd_procs_request_abort": (_i, [_i]),
+    "rocshmem_amd_procs_abort_requested": (_i, []),
     "rocshmem_amd_set_spin_limit": (_i, [_u64]),
     "rocshmem_amd_waits_given_up": (C.c_int64, [_i]),
     "rocshmem_amd_malloc": (_vp, [_sz]),

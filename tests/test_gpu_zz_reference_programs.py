@@ -88,6 +88,43 @@ def test_reference_host_programs_run_with_a_thread_per_pe(rt, name, npes):
     assert r.returncode == 0, (name, npes, r.stdout[-800:], r.stderr[-800:])
 
 
+# One process per PE, as the reference runs them under mpirun: the launcher
+# starts P copies, rocshmem_init exchanges HIP IPC handles of the per-process
+# heaps through a rendezvous file, and every transfer between PEs crosses a
+# process boundary through a mapped peer heap.
+SOS_NOT_AS_PROCESSES = {
+    "bigput": "hands addresses of static variables to a reduction; only heap objects are symmetric",
+    "query_thread": "branches on a variable it never initialises",
+}
+SOS_TWO_PROCESSES_ONLY = {"put_ctx_mbw_mr"}  # says so itself
+
+
+def sos_process_cases():
+    cases = []
+    for name in sos_programs():
+        if name in SOS_NOT_AS_PROCESSES:
+            continue
+        cases.append((name, 2))
+        if name not in SOS_TWO_PROCESSES_ONLY:
+            cases.append((name, 8))
+    return cases
+
+
+@pytest.mark.skipif(not sos_programs(), reason="oracle/_ref/sos is built where the reference tree exists")
+@pytest.mark.parametrize("name,npes", sos_process_cases())
+def test_reference_host_programs_run_with_a_process_per_pe(rt, name, npes):
+    """The unchanged programs (the build that runs as one PE above) started as
+    2 and 8 processes by rocshmem_amd.launch.  This covers the programs that
+    cannot share one address space (file-scope symmetric pointers, threads of
+    their own, unsynchronised start-up) as well as the rest."""
+    from rocshmem_amd import launch
+    rt.down()
+    env = dict(os.environ, ROCSHMEM_HEAP_SIZE=str(1 << 30))
+    env.pop("ROCSHMEM_EMU_NPES", None)
+    status, outs = launch.run(npes, [os.path.join(SOS_DIR, name)], timeout=90, env=env, capture=True)
+    assert status == 0, (name, npes, [o[-600:] for o in outs])
+
+
 # ------------------------------------- the reference's device-API functional tests
 # The test matrix of scripts/functional_tests/driver.sh:142-320 (all of it runs
 # with 2 ranks): (test name, number of the TestType enum in
