@@ -1,9 +1,10 @@
 /* The few MPI names that programs written for the reference use around the
  * rocSHMEM calls (its launcher is mpirun: rocshmem_init takes an MPI_Comm,
  * tests call MPI_Barrier and MPI_Abort), for builds without an MPI
- * installation.  No message passing happens here: all PEs live in this
- * process, the "communicator" is the set of all PEs, and a barrier is the
- * library's own host barrier.  Put this directory on the include path to
+ * installation.  No message passing happens here: the "communicator" is the
+ * set of all PEs, whether they are threads of this process or the processes
+ * of a job started by rocshmem_amd.launch, and a barrier is the library's own
+ * host meeting.  Put this directory on the include path to
  * satisfy `#include <mpi.h>`; rocshmem.hpp pulls it in by itself when no real
  * mpi.h is found. */
 #ifndef ROCSHMEM_AMD_COMPAT_MPI_H_
@@ -47,15 +48,26 @@ static inline int MPI_Comm_size(MPI_Comm, int *size) {
   *size = rocshmem_amd_n_pes();
   return MPI_SUCCESS;
 }
-/* Every PE thread arrives; outside PE threads there is nobody to wait for. */
+/* Every PE thread, or every process of the job, arrives; otherwise there is
+ * nobody to wait for. */
 static inline int MPI_Barrier(MPI_Comm) {
   const int n = rocshmem_amd_n_pes();
+  if (rocshmem_amd_procs_count() > 0) {
+    if (rocshmem_amd_procs_barrier(0, 1, n) != 0) {
+      const int asked = rocshmem_amd_procs_abort_requested();
+      fflush(NULL);
+      _Exit(asked >= 0 ? asked : EXIT_FAILURE);
+    }
+    return MPI_SUCCESS;
+  }
   if (rocshmem_amd_pe_threads_enter(0, 1, n)) rocshmem_amd_pe_threads_leave(0, 1, n);
   return MPI_SUCCESS;
 }
-/* Programs written for the reference end a failed run with MPI_Abort. */
+/* Programs written for the reference end a failed run with MPI_Abort; the
+ * other processes of a job leave at their next meeting. */
 static inline int MPI_Abort(MPI_Comm, int errorcode) {
   fflush(NULL);
+  if (rocshmem_amd_procs_count() > 0) rocshmem_amd_procs_request_abort(errorcode);
   _Exit(errorcode);
   return MPI_SUCCESS;
 }

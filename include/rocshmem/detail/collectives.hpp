@@ -68,6 +68,33 @@ __device__ __forceinline__ bool reduce_accepted(int P, int nreduce) {
   return static_cast<size_t>(2 * P) <= ROCSHMEM_REDUCE_SYNC_SIZE;
 }
 
+// The fold when the members' slices do not sit a fixed distance apart (one
+// process per PE: every peer slice is mapped wherever HIP put it, and found
+// through the context's table).  Element by element, members combined in team
+// order like the strided fold; blocks of 1024 elements go round the members so
+// that the split does not depend on anybody's work-group size.
+template <typename E, ROCSHMEM_OP Op>
+__device__ __forceinline__ void fold_by_table(Context *c, Team *t,
+                                              typename ElemTraits<E>::storage *dest,
+                                              const typename ElemTraits<E>::storage *source,
+                                              size_t n, unsigned tid, unsigned bs) {
+  using Tr = ElemTraits<E>;
+  using S = typename Tr::storage;
+  using A = typename Tr::accum;
+  constexpr size_t kBlock = 1024;
+  const int P = t->num_pes, start = t->wrt_world.pe_start, stride = t->wrt_world.stride;
+  for (size_t b = static_cast<size_t>(t->my_pe) * kBlock; b < n; b += static_cast<size_t>(P) * kBlock) {
+    const size_t bend = b + kBlock < n ? b + kBlock : n;
+    for (size_t i = b + tid; i < bend; i += bs) {
+      A acc = Tr::widen(*remote_addr(c, source + i, start));
+      for (int p = 1; p < P; ++p)
+        acc = combine<A, Op>(acc, Tr::widen(*remote_addr(c, source + i, start + p * stride)));
+      const S out = Tr::narrow(acc);
+      for (int p = 0; p < P; ++p) store_value_through(remote_addr(c, dest + i, start + p * stride), out);
+    }
+  }
+}
+
 template <typename E, ROCSHMEM_OP Op>
 __device__ __forceinline__ int wg_reduce(Context *c, Team *t,
                                          typename ElemTraits<E>::storage *dest,
@@ -83,7 +110,8 @@ __device__ __forceinline__ int wg_reduce(Context *c, Team *t,
   // arrives: nobody draws before the entry barrier has seen every member, and
   // every draw of the call before has been answered by its exit barrier.
   // Small ones are split by rule, which costs no round trip to the counter.
-  const bool by_tickets = n * sizeof(S) >= kTicketBytesFrom && n * sizeof(S) <= kWindowBytes;
+  const bool by_table = ctx_view(c)->peer_delta != nullptr;
+  const bool by_tickets = !by_table && n * sizeof(S) >= kTicketBytesFrom && n * sizeof(S) <= kWindowBytes;
   SyncPad *const first_pad = remote_ws(c, &t->sync[SYNC_REDUCE], t->wrt_world.pe_start);
   unsigned long long *const tickets = &first_pad->tickets;
   if (by_tickets && t->my_pe == 0 && is_block_leader()) store_through(tickets, 0ull);
@@ -92,6 +120,11 @@ __device__ __forceinline__ int wg_reduce(Context *c, Team *t,
   // stores, is final.
   team_pad_sync(c, t, SYNC_REDUCE, publish_of(c));
 
+  if (by_table) {
+    fold_by_table<E, Op>(c, t, dest, source, n, flat_thread_id(), flat_block_size());
+    team_pad_sync(c, t, SYNC_REDUCE, PUBLISH_LIBRARY);
+    return ROCSHMEM_SUCCESS;
+  }
   const int64_t to_first = static_cast<int64_t>(t->wrt_world.pe_start - ctx_view(c)->my_pe) *
                            static_cast<int64_t>(ctx_view(c)->pe_stride);
   const int64_t hop = static_cast<int64_t>(t->wrt_world.stride) *

@@ -232,8 +232,11 @@ __device__ __forceinline__ T *remote_addr(const Context *c, T *local, int pe) {
 // Address of the same work/sync object on PE `pe`.
 template <typename T>
 __device__ __forceinline__ T *remote_ws(const Context *c, T *local, int pe) {
-  const int64_t hop = static_cast<int64_t>(pe - ctx_view(c)->my_pe) *
-                      static_cast<int64_t>(ctx_view(c)->ws_stride);
+  // (with one process per PE the area follows the slice in the mapped block)
+  const int64_t *table = ctx_view(c)->peer_delta;
+  const int64_t hop = table ? table[pe]
+                            : static_cast<int64_t>(pe - ctx_view(c)->my_pe) *
+                                  static_cast<int64_t>(ctx_view(c)->ws_stride);
   return reinterpret_cast<T *>(reinterpret_cast<char *>(local) + hop);
 }
 

@@ -153,8 +153,12 @@ int64_t rocshmem_amd_set_ctx_options(int64_t options);
  * seconds, default 120, or once a process has asked the job to end); publish
  * stores up to 192 bytes in this rank's area and fetch reads a rank's area
  * (meet in between); request_abort asks every process to leave at its next
- * meeting, abort_requested returns the status asked for or -1. */
+ * meeting, abort_requested returns the status asked for or -1; count is the
+ * number of processes of the job this process was started as one PE of (it
+ * attaches from the environment when that has not happened yet), 0 when it
+ * was not. */
 size_t rocshmem_amd_procs_file_bytes(void);
+int rocshmem_amd_procs_count(void);
 int rocshmem_amd_procs_attach(const char *path, int nprocs, int rank);
 int rocshmem_amd_procs_barrier(int PE_start, int PE_stride, int PE_size);
 int rocshmem_amd_procs_publish(const void *bytes, size_t n);
@@ -183,6 +187,10 @@ int rocshmem_amd_set_coalesce_puts(int on);
  * exhaustion; the object exists at the same offset on every PE. */
 void *rocshmem_amd_malloc(size_t size);
 int rocshmem_amd_free(void *ptr);
+/* Host rocshmem_barrier_all (rocshmem.hpp; src/rocshmem.cpp): waits for the
+ * device work of this process and, with one process per PE, for every other
+ * PE to arrive.  -1 before rocshmem_init. */
+int rocshmem_amd_barrier_all(void);
 /* Address of a symmetric object on another PE; NULL if ptr is not in the heap. */
 void *rocshmem_amd_pe_ptr(const void *ptr, int pe);
 /* Allocator accounting: SingleHeap::get_size/get_used/get_avail

@@ -33,6 +33,9 @@ int rocshmem_amd_set_pe_rule(int rule) {
   return 0;
 }
 size_t rocshmem_amd_procs_file_bytes(void) { return sizeof(rocshmem::runtime::ProcShared); }
+int rocshmem_amd_procs_count(void) {
+  return rocshmem::runtime::procs().attach_from_env() ? rocshmem::runtime::procs().nprocs() : 0;
+}
 int rocshmem_amd_procs_attach(const char *path, int nprocs, int rank) {
   return rocshmem::runtime::procs().attach(path, nprocs, rank);
 }
@@ -106,9 +109,23 @@ int rocshmem_amd_team_active_set(rocshmem_amd_team_t team, int *PE_start, int *P
   *PE_size = t->wrt_world.size;
   return 0;
 }
-void *rocshmem_amd_malloc(size_t size) { return rt().sym_malloc(size); }
+// (with one process per PE these are the collective calls: every PE makes
+// them and they meet, as rocshmem_malloc / rocshmem_free do)
+void *rocshmem_amd_malloc(size_t size) {
+  if (rt().nprocs) return rocshmem::rocshmem_malloc(size);
+  return rt().sym_malloc(size);
+}
 int rocshmem_amd_free(void *ptr) {
+  if (rt().nprocs) {
+    rocshmem::rocshmem_free(ptr);
+    return 0;
+  }
   rt().sym_free(ptr);
+  return 0;
+}
+int rocshmem_amd_barrier_all(void) {
+  if (!rt().live) return -1;
+  rocshmem::rocshmem_barrier_all();
   return 0;
 }
 void *rocshmem_amd_pe_ptr(const void *ptr, int pe) {

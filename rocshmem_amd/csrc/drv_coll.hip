@@ -696,6 +696,7 @@ extern "C" {
 int rocshmem_amd_wg_reduce(int dtype, int op, rocshmem_amd_team_t team, void *dest,
                            const void *source, int nreduce, int wg_size,
                            rocshmem_amd_stream_t stream) {
+  DRV_ONE_PROCESS_ONLY();
   TeamView v;
   if (!view_team(team, &v) || !valid_launch(1, wg_size) || nreduce < 0) return -1;
   {
@@ -789,6 +790,7 @@ static int enqueue_reduce_teams(int dtype, int op, const rocshmem_amd_team_t *te
 int rocshmem_amd_wg_reduce_teams(int dtype, int op, const rocshmem_amd_team_t *teams, int n_teams,
                                  void *dest, const void *source, int nreduce, int chunk_elems,
                                  int wg_size, int iters, rocshmem_amd_stream_t stream) {
+  DRV_ONE_PROCESS_ONLY();
   if (n_teams < 1 || n_teams > kMaxTeamsPerLaunch) return -1;
   hipStream_t s = as_stream(stream);
   int *d_status;
@@ -832,6 +834,7 @@ int rocshmem_amd_wg_reduce_teams_static(int dtype, int op, const rocshmem_amd_te
                                         int n_teams, void *dest, const void *source, int nreduce,
                                         int chunk_elems, int wg_size, int iters,
                                         rocshmem_amd_stream_t stream) {
+  DRV_ONE_PROCESS_ONLY();
   if (n_teams > kStaticStatusWords) {
     fprintf(stderr,
             "rocshmem: rocshmem_amd_wg_reduce_teams_static takes at most %d teams per call "
@@ -882,24 +885,28 @@ int rocshmem_amd_fold_shares(void *dest, const void *source, int nreduce,
 int rocshmem_amd_wg_alltoall(int elem_size, rocshmem_amd_team_t team, void *dest,
                              const void *source, int nelems, int wg_size,
                              rocshmem_amd_stream_t stream) {
+  DRV_ONE_PROCESS_ONLY();
   return wg_move_common<MOVE_ALLTOALL>(elem_size, team, dest, source, nelems, 0, wg_size,
                                        as_stream(stream));
 }
 int rocshmem_amd_wg_broadcast(int elem_size, rocshmem_amd_team_t team, void *dest,
                               const void *source, int nelems, int pe_root, int wg_size,
                               rocshmem_amd_stream_t stream) {
+  DRV_ONE_PROCESS_ONLY();
   return wg_move_common<MOVE_BROADCAST>(elem_size, team, dest, source, nelems, pe_root,
                                         wg_size, as_stream(stream));
 }
 int rocshmem_amd_wg_fcollect(int elem_size, rocshmem_amd_team_t team, void *dest,
                              const void *source, int nelems, int wg_size,
                              rocshmem_amd_stream_t stream) {
+  DRV_ONE_PROCESS_ONLY();
   return wg_move_common<MOVE_FCOLLECT>(elem_size, team, dest, source, nelems, 0, wg_size,
                                        as_stream(stream));
 }
 
 int rocshmem_amd_wg_sync(int sync_fn, rocshmem_amd_team_t team, uint64_t *scratch, int rounds,
                          int wg_size, rocshmem_amd_stream_t stream) {
+  DRV_ONE_PROCESS_ONLY();
   auto &r = runtime::rt();
   if (!r.live || rounds < 0 || !valid_launch(1, wg_size) || !sym_ok_on(scratch, 8, r.me())) return -1;
   if (sync_fn < ROCSHMEM_AMD_BARRIER_ALL || sync_fn > ROCSHMEM_AMD_TEAM_SYNC) return -1;

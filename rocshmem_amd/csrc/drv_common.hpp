@@ -30,6 +30,17 @@ inline bool valid_launch(int n_wgs, int wg_size) {
 inline bool valid_pe(int pe) {
   return runtime::rt().live && pe >= 0 && pe < runtime::rt().npes;
 }
+// The PE a driver is asked to act for: with one process per PE, only this
+// process's own.
+inline bool valid_actor(int pe) {
+  return valid_pe(pe) && (!runtime::rt().nprocs || pe == runtime::rt().acting_pe);
+}
+// Drivers that host several PEs in one launch belong to the one-process
+// harness; a process that is one PE of a job refuses them.
+#define DRV_ONE_PROCESS_ONLY()                 \
+  do {                                         \
+    if (::rocshmem::runtime::rt().nprocs) return -1; \
+  } while (0)
 inline hipStream_t as_stream(void *s) { return static_cast<hipStream_t>(s); }
 
 // [p, p+bytes) lies inside the usable part of one PE's slice.

@@ -118,7 +118,7 @@ int rocshmem_amd_ctx_pe(const void *ctx_opaque) {
 }
 
 int rocshmem_amd_host_putmem(void *dest, const void *source, size_t nbytes, int my_pe, int pe) {
-  if (!valid_pe(my_pe) || !valid_pe(pe)) return -1;
+  if (!valid_actor(my_pe) || !valid_pe(pe)) return -1;
   if (!nbytes) return 0;
   if (!source || !sym_ok_on(dest, nbytes, my_pe)) return -1;
   auto &r = runtime::rt();
@@ -135,7 +135,7 @@ int rocshmem_amd_host_putmem(void *dest, const void *source, size_t nbytes, int 
 }
 
 int rocshmem_amd_host_getmem(void *dest, const void *source, size_t nbytes, int my_pe, int pe) {
-  if (!valid_pe(my_pe) || !valid_pe(pe)) return -1;
+  if (!valid_actor(my_pe) || !valid_pe(pe)) return -1;
   if (!nbytes) return 0;
   if (!dest || !sym_ok_on(source, nbytes, my_pe)) return -1;
   auto &r = runtime::rt();
@@ -153,7 +153,7 @@ int rocshmem_amd_host_getmem(void *dest, const void *source, size_t nbytes, int 
 
 int rocshmem_amd_host_amo(int amo_op, int dtype, void *dest, const void *value, const void *cond,
                           int my_pe, int pe, void *fetched) {
-  if (!valid_pe(my_pe) || !valid_pe(pe) || !value) return -1;
+  if (!valid_actor(my_pe) || !valid_pe(pe) || !value) return -1;
   const size_t es = dtype_bytes(dtype);
   if (es != 4 && es != 8) return -1;
   if (amo_op == ROCSHMEM_AMD_AMO_COMPARE_SWAP && !cond) return -1;

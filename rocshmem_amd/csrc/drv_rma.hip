@@ -269,7 +269,7 @@ int rocshmem_amd_rma(int rma_op, int gran, void *dest, const void *source, size_
 int rocshmem_amd_rma_messages(int rma_op, int gran, void *dest, const void *source, size_t nbytes,
                               size_t tile_bytes, int scattered, int my_pe, int pe, int n_wgs,
                               int wg_size, int iters, rocshmem_amd_stream_t stream) {
-  if (!valid_pe(my_pe) || !valid_pe(pe) || !valid_launch(n_wgs, wg_size) || iters < 0)
+  if (!valid_actor(my_pe) || !valid_pe(pe) || !valid_launch(n_wgs, wg_size) || iters < 0)
     return -1;
   if (rma_op < ROCSHMEM_AMD_PUT || rma_op > ROCSHMEM_AMD_GET_NBI) return -1;
   if (gran < ROCSHMEM_AMD_THREAD || gran > ROCSHMEM_AMD_WG) return -1;
@@ -327,7 +327,7 @@ int rocshmem_amd_rma_messages(int rma_op, int gran, void *dest, const void *sour
 
 int rocshmem_amd_rma_staged(int gran, void *dest, const void *source, void *back, size_t nbytes,
                             int my_pe, int pe, int wg_size, rocshmem_amd_stream_t stream) {
-  if (!valid_pe(my_pe) || !valid_pe(pe) || !valid_launch(1, wg_size)) return -1;
+  if (!valid_actor(my_pe) || !valid_pe(pe) || !valid_launch(1, wg_size)) return -1;
   if (gran < ROCSHMEM_AMD_THREAD || gran > ROCSHMEM_AMD_WG) return -1;
   if (!nbytes || nbytes > ROCSHMEM_AMD_STAGED_MAX_BYTES) return -1;
   if (!sym_ok_on(dest, nbytes, my_pe) || !local_ok(source, nbytes) || !local_ok(back, nbytes))
@@ -383,6 +383,7 @@ int rocshmem_amd_compare(const void *x, const void *y, size_t nbytes, uint64_t *
 }
 
 int rocshmem_amd_fill_every_pe(void *sym, int byte, size_t nbytes, rocshmem_amd_stream_t stream) {
+  DRV_ONE_PROCESS_ONLY();
   auto &r = runtime::rt();
   if (!r.live || !sym_ok_on(sym, nbytes, 0)) return -1;
   if (!nbytes) return 0;
@@ -396,7 +397,7 @@ int rocshmem_amd_fill_every_pe(void *sym, int byte, size_t nbytes, rocshmem_amd_
 
 int rocshmem_amd_putmem(void *dest, const void *source, size_t nbytes, int my_pe, int pe,
                         rocshmem_amd_stream_t stream) {
-  if (!valid_pe(my_pe) || !valid_pe(pe)) return -1;
+  if (!valid_actor(my_pe) || !valid_pe(pe)) return -1;
   if (!sym_ok_on(dest, nbytes, my_pe) || !local_ok(source, nbytes)) return -1;
   char *target = static_cast<char *>(dest) +
                  static_cast<int64_t>(pe - my_pe) * static_cast<int64_t>(runtime::rt().pe_stride);
@@ -406,7 +407,7 @@ int rocshmem_amd_putmem(void *dest, const void *source, size_t nbytes, int my_pe
 
 int rocshmem_amd_getmem(void *dest, const void *source, size_t nbytes, int my_pe, int pe,
                         rocshmem_amd_stream_t stream) {
-  if (!valid_pe(my_pe) || !valid_pe(pe)) return -1;
+  if (!valid_actor(my_pe) || !valid_pe(pe)) return -1;
   if (!sym_ok_on(source, nbytes, my_pe) || !local_ok(dest, nbytes)) return -1;
   const char *origin = static_cast<const char *>(source) +
                        static_cast<int64_t>(pe - my_pe) * static_cast<int64_t>(runtime::rt().pe_stride);
@@ -417,7 +418,7 @@ int rocshmem_amd_getmem(void *dest, const void *source, size_t nbytes, int my_pe
 int rocshmem_amd_lane_puts(void *dest, const void *source, const int *pe, const uint64_t *src_off,
                            const uint64_t *dst_off, const uint64_t *size, uint64_t active_mask,
                            int my_pe, rocshmem_amd_stream_t stream) {
-  if (!valid_pe(my_pe) || !pe || !src_off || !dst_off || !size) return -1;
+  if (!valid_actor(my_pe) || !pe || !src_off || !dst_off || !size) return -1;
   for (int i = 0; i < 64; ++i) {
     if (!((active_mask >> i) & 1ull)) continue;
     if (!valid_pe(pe[i])) return -1;

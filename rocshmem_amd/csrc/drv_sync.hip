@@ -753,7 +753,7 @@ int rocshmem_amd_amo(int amo_op, int dtype, void *counters, uint32_t n_slots,
                      const uint32_t *ids, const void *values, const void *conds, void *fetched,
                      size_t n_ops, int my_pe, int n_wgs, int wg_size,
                      rocshmem_amd_stream_t stream) {
-  if (!valid_pe(my_pe) || !valid_launch(n_wgs, wg_size) || !n_slots || !ids) return -1;
+  if (!valid_actor(my_pe) || !valid_launch(n_wgs, wg_size) || !n_slots || !ids) return -1;
   if (amo_op == ROCSHMEM_AMD_AMO_COMPARE_SWAP && !conds) return -1;
   {
     const size_t es = (dtype == ROCSHMEM_AMD_INT || dtype == ROCSHMEM_AMD_UINT ||
@@ -780,7 +780,7 @@ int rocshmem_amd_amo(int amo_op, int dtype, void *counters, uint32_t n_slots,
 int rocshmem_amd_put_signal(int gran, void *dest, const void *source, size_t nbytes,
                             uint64_t *sig_addr, uint64_t signal, int sig_op, int my_pe, int pe,
                             int n_wgs, int wg_size, int calls, rocshmem_amd_stream_t stream) {
-  if (!valid_pe(my_pe) || !valid_pe(pe) || !valid_launch(n_wgs, wg_size) || calls < 0) return -1;
+  if (!valid_actor(my_pe) || !valid_pe(pe) || !valid_launch(n_wgs, wg_size) || calls < 0) return -1;
   if (gran < ROCSHMEM_AMD_THREAD || gran > ROCSHMEM_AMD_WG) return -1;
   if (!sym_ok_on(dest, nbytes, my_pe) || !local_ok(source, nbytes) ||
       !sym_ok_on(sig_addr, 8, my_pe))
@@ -809,7 +809,7 @@ int rocshmem_amd_put_signal(int gran, void *dest, const void *source, size_t nby
 }
 
 int rocshmem_amd_signal_fetch(int gran, const uint64_t *sig_addr, int my_pe, uint64_t *value_out) {
-  if (!valid_pe(my_pe) || !value_out || !sym_ok_on(sig_addr, 8, my_pe)) return -1;
+  if (!valid_actor(my_pe) || !value_out || !sym_ok_on(sig_addr, 8, my_pe)) return -1;
   uint64_t *d_out;
   DRV_CHECK_HIP(hipMalloc(&d_out, 2 * sizeof(uint64_t)));
   DRV_CHECK_HIP(hipMemset(d_out, 0, 2 * sizeof(uint64_t)));
@@ -829,6 +829,7 @@ int rocshmem_amd_signal_fetch(int gran, const uint64_t *sig_addr, int my_pe, uin
 int rocshmem_amd_pingpong(void *buf, uint64_t *sig, size_t nbytes, int iters, int pairs,
                           int pe_a, int pe_b, int wg_size, uint64_t *ticks_out,
                           double *tick_hz_out, rocshmem_amd_stream_t stream) {
+  DRV_ONE_PROCESS_ONLY();
   if (!valid_pe(pe_a) || !valid_pe(pe_b) || pe_a == pe_b || pairs < 1 || pairs > 128 ||
       !valid_launch(2 * pairs, wg_size) || iters < 0 || nbytes == 0)
     return -1;
@@ -874,6 +875,7 @@ int rocshmem_amd_pingpong(void *buf, uint64_t *sig, size_t nbytes, int iters, in
 int rocshmem_amd_poll_with_gets(uint64_t *words, uint64_t *ready, int pairs, int rounds, int pe_a,
                                 int pe_b, int kind, int wg_size, int *timed_out_out,
                                 rocshmem_amd_stream_t stream) {
+  DRV_ONE_PROCESS_ONLY();
   auto &r = runtime::rt();
   if (!valid_pe(pe_a) || !valid_pe(pe_b) || pe_a == pe_b || pairs < 1 || pairs > 128 ||
       !valid_launch(2 * pairs, wg_size) || wg_size < 64 || rounds < 0 || kind < 0 || kind > 2 ||
@@ -914,6 +916,7 @@ int rocshmem_amd_put_flag_check(void *data, uint64_t *flags, size_t nbytes, int 
                                 int pe_a, int pe_b, int wg_size, int with_signal,
                                 uint64_t *mismatches_out, int *timed_out_out,
                                 rocshmem_amd_stream_t stream) {
+  DRV_ONE_PROCESS_ONLY();
   auto &r = runtime::rt();
   if (!valid_pe(pe_a) || !valid_pe(pe_b) || pe_a == pe_b || pairs < 1 || pairs > 128 ||
       !valid_launch(2 * pairs, wg_size) || rounds < 0 || nbytes == 0 || (nbytes & 3) ||
@@ -989,6 +992,7 @@ int rocshmem_amd_dispatch_put_signal(void *recv, const void *send, uint64_t *sig
                                      const uint32_t *recv_row, size_t row_bytes,
                                      int rows_per_call, int wg_size, uint64_t *expect,
                                      rocshmem_amd_stream_t stream) {
+  DRV_ONE_PROCESS_ONLY();
   auto &r = runtime::rt();
   if (!r.live || rows_per_call < 1 || !valid_launch(1, wg_size) || !row_bytes) return -1;
   if (expect && !local_ok(expect, 8 * static_cast<size_t>(r.npes) * r.npes)) return -1;
@@ -1070,6 +1074,7 @@ int rocshmem_amd_wait_test_woken(int wait_fn, int dtype, void *ivars, size_t nel
                                  const int *status, int cmp, const void *value,
                                  size_t wake_index, const void *wake_value,
                                  uint64_t delay_ticks, size_t *ret_out, size_t *indices_out) {
+  DRV_ONE_PROCESS_ONLY();
   if (!runtime::rt().live || !ivars || !value || !wake_value) return -1;
   if (wait_fn < ROCSHMEM_AMD_WAIT_UNTIL || wait_fn > ROCSHMEM_AMD_WAIT_UNTIL_SOME) return -1;
   if (wake_index >= (nelems ? nelems : 1)) return -1;
@@ -1100,6 +1105,7 @@ int rocshmem_amd_poll_until(int dtype, void *ivar, int cmp, const void *value, u
 
 int rocshmem_amd_ctx_cycle(rocshmem_amd_team_t team, int n_wgs, int wg_size, int per_wg,
                            int *status_out, int *pe_out, int *npes_out) {
+  DRV_ONE_PROCESS_ONLY();
   if (!runtime::rt().live || !valid_launch(n_wgs, wg_size) || per_wg < 1 || per_wg > 64)
     return -1;
   if (!status_out || !pe_out || !npes_out) return -1;

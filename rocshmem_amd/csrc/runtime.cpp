@@ -188,11 +188,14 @@ size_t Runtime::ws_bytes_per_pe() const {
   return round_up(sizeof(detail::SyncPad) + per_team * max_teams, 4096);
 }
 
+char *Runtime::ws_of(int pe) const {
+  return nprocs ? peer_base[pe] + pe_stride : d_ws + static_cast<size_t>(pe) * ws_stride;
+}
+
 detail::SyncPad *Runtime::team_pads(int pool_index, int pe) const {
   const size_t per_team = sizeof(detail::SyncPad) * detail::SYNC_KINDS +
                           ROCSHMEM_REDUCE_MIN_WRKDATA_SIZE * sizeof(double);
-  char *p = d_ws + static_cast<size_t>(pe) * ws_stride + sizeof(detail::SyncPad) +
-            per_team * pool_index;
+  char *p = ws_of(pe) + sizeof(detail::SyncPad) + per_team * pool_index;
   return reinterpret_cast<detail::SyncPad *>(p);
 }
 
@@ -350,6 +353,7 @@ int Runtime::init(int want_npes, size_t want_heap) {
   if (max_teams < 1) max_teams = 1;
   size_t alloc_bytes = 0;
   bool anchored = false;
+  ws_stride = ws_bytes_per_pe();
   acting_pe = 0;
   driver_ctx_options = 0;
   heap_base = nullptr;
@@ -365,7 +369,10 @@ int Runtime::init(int want_npes, size_t want_heap) {
     acting_pe = procs().rank();
     const size_t two_mib = size_t{2} << 20;
     pe_stride = round_up(heap_size, two_mib);
-    if (pe_stride >= (size_t{2} << 30)) {
+    // The shared block: the slice, then this PE's work/sync area, so that the
+    // table that finds a peer's slice also finds its barrier and reduce pads.
+    const size_t block_bytes = pe_stride + ws_stride;
+    if (block_bytes >= (size_t{2} << 30)) {
       fprintf(stderr,
               "rocshmem: with one process per PE the heap of a PE must stay below 2 GiB "
               "(ROCSHMEM_HEAP_SIZE=%zu asked for)\n", heap_size);
@@ -384,7 +391,7 @@ int Runtime::init(int want_npes, size_t want_heap) {
       std::vector<char *> mapped;
     };
     static Kept kept;
-    if (kept.own && (kept.bytes != pe_stride || kept.cached != heap_cached_mode())) {
+    if (kept.own && (kept.bytes != block_bytes || kept.cached != heap_cached_mode())) {
       fprintf(stderr, "rocshmem: a process that is one PE of a job keeps the heap size and kind of "
                       "its first rocshmem_init (%zu bytes)\n", kept.bytes);
       fflush(nullptr);
@@ -392,23 +399,23 @@ int Runtime::init(int want_npes, size_t want_heap) {
     }
     if (!kept.own) {
       const hipError_t e = heap_cached_mode()
-                               ? hipMalloc(reinterpret_cast<void **>(&kept.own), pe_stride)
-                               : hipExtMallocWithFlags(reinterpret_cast<void **>(&kept.own), pe_stride,
+                               ? hipMalloc(reinterpret_cast<void **>(&kept.own), block_bytes)
+                               : hipExtMallocWithFlags(reinterpret_cast<void **>(&kept.own), block_bytes,
                                                        hipDeviceMallocUncached);
       if (e != hipSuccess || !kept.own) {
         fprintf(stderr, "rocshmem: PE %d cannot allocate %zu bytes for its heap: %s\n", acting_pe,
-                pe_stride, hipGetErrorString(e));
+                block_bytes, hipGetErrorString(e));
         fflush(nullptr);
         _Exit(EXIT_FAILURE);
       }
-      kept.bytes = pe_stride;
+      kept.bytes = block_bytes;
       kept.cached = heap_cached_mode();
       kept.handle.resize(npes);
       kept.mapped.assign(npes, nullptr);
       RT_CHECK_HIP(hipIpcGetMemHandle(&kept.handle[acting_pe], kept.own));
     }
     char *own = kept.own;
-    RT_CHECK_HIP(hipMemset(own, 0, pe_stride));
+    RT_CHECK_HIP(hipMemset(own, 0, block_bytes));
     RT_CHECK_HIP(hipDeviceSynchronize());
     static_assert(sizeof(hipIpcMemHandle_t) <= kBlobBytes, "IPC handle larger than a publish area");
     procs().publish(&kept.handle[acting_pe], sizeof(hipIpcMemHandle_t));
@@ -429,7 +436,7 @@ int Runtime::init(int want_npes, size_t want_heap) {
     // Everybody has read everybody's handle before anybody publishes again.
     if (procs().barrier_world() != 0) _Exit(EXIT_FAILURE);
     heap_base = own;
-    alloc_bytes = pe_stride;
+    alloc_bytes = block_bytes;
   } else {
     // Slice placement.  Slices start on 2 MiB boundaries and sit `pe_stride`
     // apart inside ONE device allocation.  By default the allocation holds the
@@ -512,9 +519,13 @@ int Runtime::init(int want_npes, size_t want_heap) {
   // all must arrive at the same offsets: the same model base everywhere.
   allocator.reset(nprocs ? (uint64_t{1} << 40) : reinterpret_cast<uint64_t>(heap_base), heap_size);
 
-  ws_stride = ws_bytes_per_pe();
-  RT_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&d_ws), ws_stride * npes));
-  RT_CHECK_HIP(hipMemset(d_ws, 0, ws_stride * npes));
+  // Work/sync areas: one block for all PEs, or (one process per PE) the tail
+  // of every PE's shared block, cleared with it above.
+  d_ws = nullptr;
+  if (!nprocs) {
+    RT_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&d_ws), ws_stride * npes));
+    RT_CHECK_HIP(hipMemset(d_ws, 0, ws_stride * npes));
+  }
 
   // Teams: slot 0 is the world team.
   h_teams.assign(static_cast<size_t>(max_teams) * npes, detail::Team{});
@@ -545,7 +556,7 @@ int Runtime::init(int want_npes, size_t want_heap) {
     c.my_pe = pe;
     c.num_pes = npes;
     c.tinfo = &d_teams[pe].wrt_world;
-    c.world_sync = reinterpret_cast<detail::SyncPad *>(d_ws + static_cast<size_t>(pe) * ws_stride);
+    c.world_sync = reinterpret_cast<detail::SyncPad *>(ws_of(pe));
     c.options = 0;
     c.pool_slot = slot;
   };
@@ -616,7 +627,7 @@ int Runtime::init(int want_npes, size_t want_heap) {
   state.default_ctx = d_default_ctx;
   state.world_team = d_teams;
   state.ctx_pool = d_pools;
-  state.ws_base = d_ws;
+  state.ws_base = ws_of(0);
   state.nt_bytes = env_size("ROCSHMEM_NT_THRESHOLD", detail::kNonTemporalBytes);
   state.coalesce_puts = env_size("ROCSHMEM_COALESCE_PUTS", 1) != 0 ? 1 : 0;
   state.spin_limit = env_size("ROCSHMEM_EMU_SPIN_LIMIT", 0);
@@ -652,7 +663,7 @@ void Runtime::finalize() {
   RT_CHECK_HIP(hipFree(d_ctx_slots));
   RT_CHECK_HIP(hipFree(d_default_ctx));
   RT_CHECK_HIP(hipFree(d_teams));
-  RT_CHECK_HIP(hipFree(d_ws));
+  if (d_ws) RT_CHECK_HIP(hipFree(d_ws));
   if (heap_base) release_heap_block(heap_base);
   heap_base = nullptr;
   nprocs = 0;
@@ -765,7 +776,9 @@ int Runtime::team_split_strided(rocshmem_team_t parent, int start, int stride, i
 
   // Fresh sync pads for the new team on every PE.
   const size_t pad_bytes = sizeof(detail::SyncPad) * detail::SYNC_KINDS;
-  for (int pe = 0; pe < npes; ++pe) RT_CHECK_HIP(hipMemset(team_pads(slot, pe), 0, pad_bytes));
+  // (one process per PE: each clears its own; the members meet before they use the team)
+  for (int pe = 0; pe < npes; ++pe)
+    if (!nprocs || pe == acting_pe) RT_CHECK_HIP(hipMemset(team_pads(slot, pe), 0, pad_bytes));
 
   const detail::TeamInfo world{start_world, stride_world, size, ilog2(stride_world)};
   const detail::TeamInfo wrt_parent{start, stride, size, ilog2(stride)};
@@ -1165,6 +1178,8 @@ hipError_t rocshmem_emu_device_synchronize() {
 }
 
 int rocshmem_emu_run_pes(int npes, int (*pe_main)(int, char **), int argc, char **argv) {
+  // Started as one PE of a job of processes: this process is that PE, no threads.
+  if (runtime::procs().attach_from_env()) return pe_main(argc, argv);
   if (npes <= 0) npes = rocshmem_n_pes();
   if (runtime::pe_threads_count() != 0 || rt().live) {
     fprintf(stderr, "rocshmem: rocshmem_emu_run_pes needs a runtime that is not yet up\n");

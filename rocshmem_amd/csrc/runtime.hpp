@@ -113,6 +113,7 @@ struct Runtime {
  private:
   const detail::Team *host_team_unlocked(rocshmem_team_t team) const;
   size_t ws_bytes_per_pe() const;
+  char *ws_of(int pe) const;  // work/sync area of a PE
   detail::SyncPad *team_pads(int pool_index, int pe) const;
   void write_team(int pool_index, int pe, const detail::TeamInfo &world,
                   const detail::TeamInfo &parent, int my_pe_in_team);

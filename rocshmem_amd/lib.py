@@ -34,6 +34,7 @@ SIGNATURES = {
     "rocshmem_amd_set_ctx_options": (C.c_int64, [C.c_int64]),
     "rocshmem_amd_set_coalesce_puts": (_i, [_i]),
     "rocshmem_amd_procs_file_bytes": (_sz, []),
+    "rocshmem_amd_procs_count": (_i, []),
     "rocshmem_amd_procs_attach": (_i, [C.c_char_p, _i, _i]),
     "rocshmem_amd_procs_barrier": (_i, [_i, _i, _i]),
     "rocshmem_amd_procs_publish": (_i, [_vp, _sz]),
@@ -44,6 +45,7 @@ SIGNATURES = {
     "rocshmem_amd_waits_given_up": (C.c_int64, [_i]),
     "rocshmem_amd_malloc": (_vp, [_sz]),
     "rocshmem_amd_free": (_i, [_vp]),
+    "rocshmem_amd_barrier_all": (_i, []),
     "rocshmem_amd_pe_ptr": (_vp, [_vp, _i]),
     "rocshmem_amd_heap_size": (_sz, []),
     "rocshmem_amd_heap_used": (_sz, []),

@@ -213,6 +213,35 @@ def test_reference_functional_driver(rt, name, number, wgs, threads, max_size):
     assert r.returncode == 0, (name, r.stdout[-600:], r.stderr[-600:])
 
 
+# Device waits between processes are bounded in these runs: a wait that would
+# never end (a lost signal, kernels of two processes that cannot run side by
+# side) gives up after this many polls and the tester's own check then fails,
+# instead of a kernel that never exits.
+PROCESS_RUN_SPIN_LIMIT = str(40_000_000)
+
+
+@pytest.mark.skipif(not functional_cases(),
+                    reason="oracle/_ref/functional is built where the reference tree exists")
+@pytest.mark.parametrize("name,number,wgs,threads,max_size", functional_cases(),
+                         ids=["%s-w%d-z%d-%s" % (c[0], c[2], c[3], c[4]) for c in functional_cases()])
+def test_reference_functional_driver_with_a_process_per_pe(rt, name, number, wgs, threads, max_size):
+    """The same driver and matrix with the 2 ranks as 2 processes, the way the
+    reference's script runs it (mpirun -np 2): every put, get, atomic and
+    signal issued inside a kernel lands in the other process's heap through
+    its HIP IPC mapping, and the device-side barriers and collectives of the
+    testers meet across the process boundary."""
+    from rocshmem_amd import launch
+    rt.down()
+    env = dict(os.environ, ROCSHMEM_EMU_SPIN_LIMIT=PROCESS_RUN_SPIN_LIMIT,
+               ROCSHMEM_MAX_NUM_CONTEXTS="1024" if name == "teamctxinfra" else str(wgs))
+    env.pop("ROCSHMEM_EMU_NPES", None)
+    cmd = [FUNCTIONAL_DRIVER, "-a", str(number), "-w", str(wgs), "-z", str(threads)]
+    if max_size is not None:
+        cmd += ["-s", str(max_size)]
+    status, outs = launch.run(2, cmd, timeout=90, env=env, capture=True)
+    assert status == 0, (name, [o[-600:] for o in outs])
+
+
 # ------------------------------------------------- the reference's example programs
 EXAMPLES_DIR = os.path.join(ROOT, "oracle", "_ref", "examples")
 
@@ -240,3 +269,20 @@ def test_reference_examples_run_with_a_thread_per_pe(rt, name, npes):
     assert r.returncode == 0, (name, npes, r.stdout[-600:], r.stderr[-600:])
     assert r.stdout.count("[FAIL]") == 0, r.stdout[-600:]
     assert r.stdout.count("[PASS]") >= npes - 1, r.stdout[-600:]
+
+
+@pytest.mark.skipif(not example_programs(), reason="oracle/_ref/examples is built where the reference tree exists")
+@pytest.mark.parametrize("npes", [2, 8])
+@pytest.mark.parametrize("name", example_programs())
+def test_reference_examples_run_with_a_process_per_pe(rt, name, npes):
+    """The examples as 2 and 8 processes (mpirun -np in the reference): their
+    kernels' collectives and signals cross process boundaries."""
+    from rocshmem_amd import launch
+    rt.down()
+    env = dict(os.environ, ROCSHMEM_EMU_SPIN_LIMIT=PROCESS_RUN_SPIN_LIMIT)
+    env.pop("ROCSHMEM_EMU_NPES", None)
+    status, outs = launch.run(npes, [os.path.join(EXAMPLES_DIR, name)], timeout=90, env=env, capture=True)
+    assert status == 0, (name, npes, [o[-600:] for o in outs])
+    text = "".join(outs)
+    assert text.count("[FAIL]") == 0, text[-600:]
+    assert text.count("[PASS]") >= npes - 1, text[-600:]
