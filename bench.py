@@ -42,7 +42,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0  # MI355X, published
 # HBM bytes one launch of the headline kernel moves, from FETCH_SIZE + WRITE_SIZE
 # under rocprofv3 --pmc (profiles/putmem_wg_tiled_256MiB_hbm_traffic.txt).
-PUT_TRAFFIC_BYTES = 536937497
+PUT_TRAFFIC_BYTES = 536952840
 P = 8
 MiB = 1 << 20
 
@@ -59,6 +59,11 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--quick", action="store_true", help="headline only, no CPU baseline")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--with-processes", action="store_true",
+                    help="also run the headline between two processes (one process per PE, HIP IPC); "
+                         "the record gains all_configs.process_per_pe_2_processes")
+    ap.add_argument("--process-leg", action="store_true",
+                    help="(internal) run as one PE of a two-process job started by rocshmem_amd.launch")
     ap.add_argument("--profile-kernels", action="store_true",
                     help="a short run for rocprofv3: a few launches each of the headline put, the "
                          "fp32 sum all-reduce, the alltoall and the dispatch, and three 256 MiB "
@@ -686,6 +691,99 @@ def profile_kernels():
                       "alltoall_gbs": a2a["gbs"], "dispatch": disp}))
 
 
+def process_leg(steps, warmup):
+    """One PE of a job of two processes (started by process_per_pe_config through
+    rocshmem_amd.launch): PE 0 runs the headline's tiled rocshmem_ctx_putmem_wg
+    and getmem_wg, and the host rocshmem_putmem, with PE 1 — another process,
+    its heap mapped here through HIP IPC — as the target.  Three buffer pairs
+    of 256 MiB in rotation (1.5 GiB, the heap of a process stays below 2 GiB)
+    keep the memory-side cache out of it.  PE 1 checks what arrived against PE
+    0's source, which it reads through its own mapping.  PE 0 prints the record."""
+    from rocshmem_amd import lib as L
+    b = Bench(L)
+    l = b.l
+    assert l.init(0, 1900 * MiB) == 0
+    me, n, pairs = l.my_pe(), 256 * MiB, 3
+    assert l.n_pes() == 2
+    bufs = [(l.malloc(n), l.malloc(n)) for _ in range(pairs)]
+    assert all(s and d for s, d in bufs)
+    for i, (s, d) in enumerate(bufs):
+        b.fill_random(s, n, me, 10 * me + i)
+        l.fill(d, 0, n)
+    l.barrier_all()
+    out = {}
+    if me == 0:
+        k = [0]
+
+        def rotating(fn):
+            def step():
+                s, d = bufs[k[0] % pairs]
+                k[0] += 1
+                assert fn(s, d) == 0
+            return step
+
+        wg, tile, _ = PUT_SHAPES["nostore_ctx"]
+        l.set_ctx_options(1)
+        put = rotating(lambda s, d: l.rma(L.PUT, L.WG, d, s, n, tile, 0, 1, n // tile, wg, 1, None))
+        for _ in range(2):
+            out["putmem_wg_nostore_gbs"] = round(2 * n / b.time_ms(put, steps, warmup) / 1e6, 1)
+        out["getmem_wg_nostore_gbs"] = round(2 * n / b.time_ms(
+            rotating(lambda s, d: l.rma(L.GET, L.WG, d, s, n, tile, 0, 1, n // tile, wg, 1, None)),
+            steps, warmup) / 1e6, 1)
+        l.set_ctx_options(0)
+        wg, tile, n_wgs = PUT_SHAPES["default_ctx"]
+        out["putmem_wg_default_ctx_gbs"] = round(2 * n / b.time_ms(
+            rotating(lambda s, d: l.rma(L.PUT, L.WG, d, s, n, tile, 0, 1, n_wgs, wg, 1, None)),
+            steps, warmup) / 1e6, 1)
+        out["host_putmem_gbs"] = round(2 * n / b.time_ms(
+            rotating(lambda s, d: l.putmem(d, s, n, 0, 1, None)), steps, warmup) / 1e6, 1)
+        # one more tiled put per pair into cleared destinations, for PE 1 to check
+        l.barrier_all()            # the timed loops are over
+        l.barrier_all()            # PE 1 has cleared its destinations
+        l.set_ctx_options(1)
+        for s, d in bufs:
+            assert l.rma(L.PUT, L.WG, d, s, n, 4096, 0, 1, n // 4096, 128, 1, None) == 0
+        l.set_ctx_options(0)
+        l.barrier_all()            # the puts have landed
+        print("PROCESS_LEG " + json.dumps(out), flush=True)
+    else:
+        l.barrier_all()            # PE 0 has finished its timed loops
+        for _, d in bufs:
+            l.fill(d, 0, n)
+        l.barrier_all()            # PE 0 may put
+        l.barrier_all()            # PE 0 has put
+        ok = True
+        for s, d in bufs:
+            bad = C.c_uint64(1)
+            assert l.compare(d, l.pe_ptr(s, 0), n, C.byref(bad), None) == 0
+            ok = ok and bad.value == 0
+        print("PROCESS_LEG_VERIFIED %d" % ok, flush=True)
+    l.finalize()
+
+
+def process_per_pe_config(steps, warmup):
+    """The headline between two processes (the reference's deployment: one
+    process per PE, peers mapped through HIP IPC).  Run while this process
+    holds no runtime, so that the two children have the GPU to themselves."""
+    from rocshmem_amd import launch
+    env = dict(os.environ)
+    for name in ("ROCSHMEM_EMU_SPREAD", "ROCSHMEM_EMU_HEAP_CACHED", "ROCSHMEM_EMU_NPES"):
+        env.pop(name, None)
+    status, outs = launch.run(2, [sys.executable, os.path.abspath(__file__), "--process-leg", "--steps",
+                                  str(steps), "--warmup", str(warmup)], timeout=120, env=env, capture=True)
+    rec = {"exit_status": status}
+    for o in outs:
+        for ln in o.splitlines():
+            if ln.startswith("PROCESS_LEG "):
+                rec.update(json.loads(ln[len("PROCESS_LEG "):]))
+            elif ln.startswith("PROCESS_LEG_VERIFIED "):
+                rec["verified"] = ln.split()[1] == "1"
+    rec.setdefault("verified", False)
+    if status != 0:
+        rec["output_tail"] = [o[-300:] for o in outs]
+    return rec
+
+
 def bring_up(L, heap_bytes, **env):
     """rocshmem_init with the given layout / heap switches in the environment
     (a value of None removes the variable)."""
@@ -704,6 +802,9 @@ def main():
     a = parse()
     if a.profile_kernels:
         profile_kernels()
+        return
+    if a.process_leg:
+        process_leg(a.steps, a.warmup)
         return
     if a.gpus != 1:
         print("bench.py measures one GPU: every PE is a slice of one symmetric heap on a single "
@@ -747,6 +848,8 @@ def main():
         allc["hbm_one_direction_256MiB"] = head["ceilings"]
         allc["putmem_wg_tiled_256MiB"] = head["tiled"]
     b.l.finalize()
+    if full and a.with_processes:
+        allc["process_per_pe_2_processes"] = process_per_pe_config(a.steps, a.warmup)
     if with_cpu:
         legs.update(cpu_copy_leg())
 
@@ -809,6 +912,8 @@ def main():
         dp, amo, pp = allc["dispatch_put_signal"], allc["atomic_fetch_add_16Mi"], allc["pingpong"]
         mr, ru = allc["message_rates"], allc["reuse_256MiB"]
         verified = verified and bool(packed["putmem_wg"]["verified"]) and bool(cached["putmem_wg"]["verified"])
+        if "process_per_pe_2_processes" in allc:
+            verified = verified and bool(allc["process_per_pe_2_processes"]["verified"])
         roof.update({
             # configs[1]: bulk putmem through the device API, both kinds of context
             "verified": verified,
@@ -867,6 +972,9 @@ def main():
             "pingpong_32pairs_msg_per_s": pp["8_x32pairs"]["nostore_ctx"]["msg_per_s"],
             "barrier_all_round_us": allc["barrier_P8"]["barrier_all_round_us"],
         })
+        if "process_per_pe_2_processes" in allc:
+            roof["putmem_wg_frac_nostore_between_processes"] = frac(
+                allc["process_per_pe_2_processes"].get("putmem_wg_nostore_gbs", 0.0))
     else:
         roof.update({"verified": verified, "putmem_wg_frac": frac(head["default_ctx_gbs"]),
                      "putmem_wg_frac_nostore": frac(head["gbs"]),

@@ -22,7 +22,7 @@ namespace detail {
 // ROCSHMEM_CTX_NOSTORE (include/rocshmem/rocshmem_common.hpp; the reference
 // switches its flush off for that option, src/fence_policy.hpp:45-63).
 __device__ __forceinline__ int publish_of(const Context *c) {
-  return (ctx_view(c)->options & static_cast<unsigned>(ROCSHMEM_CTX_NOSTORE)) ? PUBLISH_LIBRARY : PUBLISH_ALL;
+  return (ctx_options(c) & static_cast<unsigned>(ROCSHMEM_CTX_NOSTORE)) ? PUBLISH_LIBRARY : PUBLISH_ALL;
 }
 
 __device__ __forceinline__ void team_pad_sync(const Context *c, Team *t, int kind, int publish) {
@@ -110,7 +110,7 @@ __device__ __forceinline__ int wg_reduce(Context *c, Team *t,
   // arrives: nobody draws before the entry barrier has seen every member, and
   // every draw of the call before has been answered by its exit barrier.
   // Small ones are split by rule, which costs no round trip to the counter.
-  const bool by_table = ctx_view(c)->peer_delta != nullptr;
+  const bool by_table = peers_by_table(c);
   const bool by_tickets = !by_table && n * sizeof(S) >= kTicketBytesFrom && n * sizeof(S) <= kWindowBytes;
   SyncPad *const first_pad = remote_ws(c, &t->sync[SYNC_REDUCE], t->wrt_world.pe_start);
   unsigned long long *const tickets = &first_pad->tickets;

@@ -44,7 +44,7 @@ __device__ __forceinline__ int translate_pe(rocshmem_ctx_t ctx, int pe) {
 // on a NOSTORE context every wavefront also waits for its own share first, so
 // that a quiet by any one thread covers the whole work-group's put.
 __device__ __forceinline__ bool no_store_order(const Context *c) {
-  return (ctx_view(c)->options & static_cast<unsigned>(ROCSHMEM_CTX_NOSTORE)) != 0;
+  return (ctx_options(c) & static_cast<unsigned>(ROCSHMEM_CTX_NOSTORE)) != 0;
 }
 // A get reads what memory holds now: the L1 of the CU and the L2 of the XCD may
 // keep a line of the heap that another XCD has since written through to
@@ -86,7 +86,8 @@ __device__ __forceinline__ bool put_as_one_run(Context *c, void *dest, const voi
   const char *s = reinterpret_cast<const char *>(
       read_lane(reinterpret_cast<unsigned long long>(source), leader));
   const int to = read_lane(pe, leader);
-  copy_wave(remote_addr(c, d, to), s, total, g_state.nt_bytes);
+  const size_t nt = g_state.nt_bytes;  // (asked for before remote_addr's branch, see putmem_wg)
+  copy_wave(remote_addr(c, d, to), s, total, nt);
   drain_own_stores();
   return true;
 }
@@ -142,7 +143,8 @@ __device__ __forceinline__ void getmem_nbi(Context *c, void *dest, const void *s
 // ---- wavefront granularity (context_ipc_device.cpp:137-164) ---------------
 __device__ __forceinline__ void putmem_wave(Context *c, void *dest, const void *source,
                                             size_t n, int pe) {
-  copy_wave(remote_addr(c, static_cast<char *>(dest), pe), source, n, g_state.nt_bytes);
+  const size_t nt = g_state.nt_bytes;
+  copy_wave(remote_addr(c, static_cast<char *>(dest), pe), source, n, nt);
   drain_own_stores();
 }
 // A get's stores go to the caller's own buffer; the wait makes them complete
@@ -150,7 +152,8 @@ __device__ __forceinline__ void putmem_wave(Context *c, void *dest, const void *
 __device__ __forceinline__ void getmem_wave(Context *c, void *dest, const void *source,
                                             size_t n, int pe) {
   fresh_reads();
-  copy_wave(dest, remote_addr(c, static_cast<const char *>(source), pe), n, g_state.nt_bytes);
+  const size_t nt = g_state.nt_bytes;
+  copy_wave(dest, remote_addr(c, static_cast<const char *>(source), pe), n, nt);
   drain_own_stores();
 }
 
@@ -158,12 +161,14 @@ __device__ __forceinline__ void getmem_wave(Context *c, void *dest, const void *
 // either kind of context.
 __device__ __forceinline__ void putmem_nbi_wave(Context *c, void *dest, const void *source,
                                                 size_t n, int pe) {
-  copy_wave(remote_addr(c, static_cast<char *>(dest), pe), source, n, g_state.nt_bytes);
+  const size_t nt = g_state.nt_bytes;
+  copy_wave(remote_addr(c, static_cast<char *>(dest), pe), source, n, nt);
 }
 __device__ __forceinline__ void getmem_nbi_wave(Context *c, void *dest, const void *source,
                                                 size_t n, int pe) {
   fresh_reads();
-  copy_wave(dest, remote_addr(c, static_cast<const char *>(source), pe), n, g_state.nt_bytes);
+  const size_t nt = g_state.nt_bytes;
+  copy_wave(dest, remote_addr(c, static_cast<const char *>(source), pe), n, nt);
 }
 
 // ---- work-group granularity: copy, then __syncthreads (:109-125) ----------
@@ -174,8 +179,11 @@ __device__ __forceinline__ void getmem_nbi_wave(Context *c, void *dest, const vo
 __device__ __forceinline__ void putmem_wg(Context *c, void *dest, const void *source,
                                           size_t n, int pe) {
   const bool relaxed = no_store_order(c);
-  copy_lanes(remote_addr(c, static_cast<char *>(dest), pe), source, n,
-             flat_thread_id(), flat_block_size(), g_state.nt_bytes);
+  // (everything that comes from scalar loads is asked for before remote_addr,
+  // whose rare table path is a branch that later loads would queue behind)
+  const unsigned tid = flat_thread_id(), bs = flat_block_size();
+  const size_t nt = g_state.nt_bytes;
+  copy_lanes(remote_addr(c, static_cast<char *>(dest), pe), source, n, tid, bs, nt);
   // Each wavefront completes its own share, so that after the barrier a quiet
   // by any one thread covers the whole work-group's put.
   if (relaxed) drain_own_stores();
@@ -190,8 +198,9 @@ __device__ __forceinline__ void putmem_wg(Context *c, void *dest, const void *so
 // or wavefront-level get, or a wait.
 __device__ __forceinline__ void getmem_wg(Context *c, void *dest, const void *source,
                                           size_t n, int pe) {
-  copy_lanes(dest, remote_addr(c, static_cast<const char *>(source), pe), n,
-             flat_thread_id(), flat_block_size(), g_state.nt_bytes);
+  const unsigned tid = flat_thread_id(), bs = flat_block_size();
+  const size_t nt = g_state.nt_bytes;
+  copy_lanes(dest, remote_addr(c, static_cast<const char *>(source), pe), n, tid, bs, nt);
   __syncthreads();
 }
 

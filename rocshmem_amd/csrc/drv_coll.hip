@@ -861,6 +861,7 @@ int rocshmem_amd_wg_reduce_teams_static(int dtype, int op, const rocshmem_amd_te
 
 int rocshmem_amd_fold_shares(void *dest, const void *source, int nreduce,
                              const int *lanes_per_member, rocshmem_amd_stream_t stream) {
+  DRV_ONE_PROCESS_ONLY();
   auto &r = runtime::rt();
   if (!r.live || !lanes_per_member || nreduce < 0 || r.npes > detail::SyncPad::kMaxPes) return -1;
   const size_t bytes = static_cast<size_t>(nreduce) * sizeof(int);

@@ -399,8 +399,8 @@ int rocshmem_amd_putmem(void *dest, const void *source, size_t nbytes, int my_pe
                         rocshmem_amd_stream_t stream) {
   if (!valid_actor(my_pe) || !valid_pe(pe)) return -1;
   if (!sym_ok_on(dest, nbytes, my_pe) || !local_ok(source, nbytes)) return -1;
-  char *target = static_cast<char *>(dest) +
-                 static_cast<int64_t>(pe - my_pe) * static_cast<int64_t>(runtime::rt().pe_stride);
+  if (!nbytes) return 0;
+  char *target = static_cast<char *>(runtime::rt().pe_ptr(dest, pe));
   launch_bulk(target, static_cast<const char *>(source), nbytes, as_stream(stream));
   return 0;
 }
@@ -409,8 +409,8 @@ int rocshmem_amd_getmem(void *dest, const void *source, size_t nbytes, int my_pe
                         rocshmem_amd_stream_t stream) {
   if (!valid_actor(my_pe) || !valid_pe(pe)) return -1;
   if (!sym_ok_on(source, nbytes, my_pe) || !local_ok(dest, nbytes)) return -1;
-  const char *origin = static_cast<const char *>(source) +
-                       static_cast<int64_t>(pe - my_pe) * static_cast<int64_t>(runtime::rt().pe_stride);
+  if (!nbytes) return 0;
+  const char *origin = static_cast<const char *>(runtime::rt().pe_ptr(source, pe));
   launch_bulk(static_cast<char *>(dest), origin, nbytes, as_stream(stream));
   return 0;
 }

@@ -189,7 +189,7 @@ size_t Runtime::ws_bytes_per_pe() const {
 }
 
 char *Runtime::ws_of(int pe) const {
-  return nprocs ? peer_base[pe] + pe_stride : d_ws + static_cast<size_t>(pe) * ws_stride;
+  return nprocs ? peer_base[pe] + slice_bytes : d_ws + static_cast<size_t>(pe) * ws_stride;
 }
 
 detail::SyncPad *Runtime::team_pads(int pool_index, int pe) const {
@@ -368,10 +368,11 @@ int Runtime::init(int want_npes, size_t want_heap) {
     nprocs = procs().nprocs();
     acting_pe = procs().rank();
     const size_t two_mib = size_t{2} << 20;
-    pe_stride = round_up(heap_size, two_mib);
+    pe_stride = 0;
+    slice_bytes = round_up(heap_size, two_mib);
     // The shared block: the slice, then this PE's work/sync area, so that the
     // table that finds a peer's slice also finds its barrier and reduce pads.
-    const size_t block_bytes = pe_stride + ws_stride;
+    const size_t block_bytes = slice_bytes + ws_stride;
     if (block_bytes >= (size_t{2} << 30)) {
       fprintf(stderr,
               "rocshmem: with one process per PE the heap of a PE must stay below 2 GiB "
@@ -509,6 +510,7 @@ int Runtime::init(int want_npes, size_t want_heap) {
       exit(EXIT_FAILURE);
     }
   }
+  if (!nprocs) slice_bytes = pe_stride;
   heap_alloc_bytes = alloc_bytes;
   heap_uncached = !heap_cached_mode();
   if (verbose())
@@ -538,20 +540,31 @@ int Runtime::init(int want_npes, size_t want_heap) {
   const detail::TeamInfo world{0, 1, npes, 0};
   for (int pe = 0; pe < npes; ++pe) write_team(0, pe, world, world, pe);
 
-  // With one process per PE: where every PE's slice sits relative to this
-  // PE's, the table behind remote_addr (nullptr otherwise: equal strides).
-  d_peer_delta = nullptr;
-  if (nprocs) {
-    std::vector<int64_t> delta(npes);
-    for (int p = 0; p < npes; ++p) delta[p] = peer_base[p] - peer_base[acting_pe];
-    RT_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&d_peer_delta), sizeof(int64_t) * npes));
-    RT_CHECK_HIP(hipMemcpy(d_peer_delta, delta.data(), sizeof(int64_t) * npes, hipMemcpyHostToDevice));
+  // Where every PE's slice sits relative to PE q's, for every q: row q is the
+  // table of q's contexts.  With all slices in one allocation device code
+  // takes the product and never reads it (the rows hold the same products, so
+  // that the pointer is never a dangling one); with one process per PE only
+  // this PE's row means anything (the others stay zero: the own slice).
+  {
+    std::vector<int64_t> delta(static_cast<size_t>(npes) * npes, 0);
+    for (int q = 0; q < npes; ++q)
+      for (int p = 0; p < npes; ++p) {
+        if (nprocs) {
+          if (q == acting_pe) delta[static_cast<size_t>(q) * npes + p] = peer_base[p] - peer_base[q];
+        } else {
+          delta[static_cast<size_t>(q) * npes + p] =
+              static_cast<int64_t>(p - q) * static_cast<int64_t>(pe_stride);
+        }
+      }
+    RT_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&d_peer_delta), sizeof(int64_t) * delta.size()));
+    RT_CHECK_HIP(hipMemcpy(d_peer_delta, delta.data(), sizeof(int64_t) * delta.size(),
+                           hipMemcpyHostToDevice));
   }
   // Contexts: one default context and one pool per PE.
   auto fill_ctx = [&](detail::Context &c, int pe, int slot) {
-    c.peer_delta = d_peer_delta;
+    c.peer_delta = d_peer_delta + static_cast<size_t>(pe) * npes;
     c.heap_base = heap_base;
-    c.pe_stride = pe_stride;
+    c.pe_stride = pe_stride;  // 0 with one process per PE: device code takes the table
     c.ws_stride = ws_stride;
     c.my_pe = pe;
     c.num_pes = npes;
@@ -648,11 +661,11 @@ void Runtime::finalize() {
     // Nobody leaves while another PE may still be writing to its slice.  The
     // slice and the mappings stay (see rocshmem_init).
     (void)procs().barrier_world();
-    RT_CHECK_HIP(hipFree(d_peer_delta));
-    d_peer_delta = nullptr;
     heap_base = nullptr;
     peer_base.clear();
   }
+  RT_CHECK_HIP(hipFree(d_peer_delta));
+  d_peer_delta = nullptr;
   RT_CHECK_HIP(hipFree(d_queue_table));
   d_queue_table = nullptr;
   RT_CHECK_HIP(hipFree(d_gave_up));
@@ -729,7 +742,7 @@ int Runtime::pe_of(const void *ptr) const {
   if (nprocs) {
     // the slices are mapped wherever HIP put them: look the address up
     for (int pe = 0; pe < npes; ++pe)
-      if (p >= peer_base[pe] && p < peer_base[pe] + pe_stride) return pe;
+      if (p >= peer_base[pe] && p < peer_base[pe] + slice_bytes) return pe;
     return -1;
   }
   if (p < heap_base || p >= heap_base + pe_stride * npes) return -1;

@@ -28,7 +28,12 @@ struct Runtime {
   int max_teams = 0;
   int num_user_teams = 0;
   size_t heap_size = 0;
+  // Bytes between the slices of consecutive PEs.  With one process per PE the
+  // slices are separate mappings and no such distance exists: the stride is 0
+  // there (host or device arithmetic that still used it would stay inside the
+  // caller's own slice) and slice_bytes is what a slice spans.
   size_t pe_stride = 0;
+  size_t slice_bytes = 0;
   size_t ws_stride = 0;
   size_t heap_alloc_bytes = 0;  // size of the device allocation that holds the slices
   bool heap_uncached = true;    // false under ROCSHMEM_EMU_HEAP_CACHED=1
@@ -37,7 +42,7 @@ struct Runtime {
   // has the others' mapped through HIP IPC wherever HIP put them.
   int nprocs = 0;                   // 0: all PEs live in this process
   std::vector<char *> peer_base;    // [npes] in process mode: where each PE's slice is mapped here
-  int64_t *d_peer_delta = nullptr;  // device, [npes]: peer_base[p] - peer_base[me]
+  int64_t *d_peer_delta = nullptr;  // device, [npes][npes]: (slice of p) - (slice of q) at [q][p]
   char *slice_base(int pe) const {
     return nprocs ? peer_base[pe] : heap_base + static_cast<size_t>(pe) * pe_stride;
   }

@@ -43,7 +43,8 @@ def main():
     src, dst = l.malloc(n + 64), l.malloc(n + 64)
     assert src and dst
     for case, (off_s, off_d, size) in enumerate([(0, 0, n), (1, 3, 4099), (5, 2, 1), (16, 7, 65536), (3, 3, 0)]):
-        for how in ("host_put", "host_get", "put_wg", "put_wave", "put_thread", "get_wg", "put_nbi_wg"):
+        for how in ("host_put", "host_get", "bulk_put", "bulk_get", "put_wg", "put_wave", "put_thread",
+                    "get_wg", "put_nbi_wg"):
             mine = orc.fill_u8(n + 64, 100 + case, me)
             put_bytes(l, src, mine)
             assert l.fill(dst, 0xA5, n + 64) == 0
@@ -52,6 +53,10 @@ def main():
                 assert l.host_putmem(dst + off_d, src + off_s, size, me, nxt) == 0
             elif how == "host_get":
                 assert l.host_getmem(dst + off_d, src + off_s, size, me, prv) == 0
+            elif how == "bulk_put":  # the whole-GPU kernels behind the host's rocshmem_putmem / getmem
+                assert l.putmem(dst + off_d, src + off_s, size, me, nxt, None) == 0
+            elif how == "bulk_get":
+                assert l.getmem(dst + off_d, src + off_s, size, me, prv, None) == 0
             elif how.startswith("put"):
                 gran = {"wg": L.WG, "wave": L.WAVE, "thread": L.THREAD}[how.split("_")[-1]]
                 op = L.PUT_NBI if "nbi" in how else L.PUT
