@@ -80,6 +80,11 @@ def run(nprocs, argv, timeout=300.0, env=None, capture=False):
                 out.close()
         return status, texts
     finally:
+        # whatever ended the wait (an exception included), no PE outlives its launcher
+        for proc in procs:
+            if proc.poll() is None:
+                proc.kill()
+                proc.wait()
         try:
             os.unlink(path)
         except OSError:
