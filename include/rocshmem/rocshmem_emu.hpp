@@ -67,7 +67,8 @@ void *rocshmem_emu_pe_ptr(const void *ptr, int pe);
 // Handle of the same team as seen by PE `pe` (ROCSHMEM_TEAM_INVALID when that
 // PE is not a member).
 rocshmem_team_t rocshmem_emu_team_on(rocshmem_team_t team, int pe);
-// Bytes between the slices of consecutive PEs.
+// Bytes between the slices of consecutive PEs; 0 in a process that is one PE of
+// a job of processes (the slices are separate mappings: use rocshmem_emu_pe_ptr).
 size_t rocshmem_emu_pe_stride();
 
 }  // namespace rocshmem

@@ -198,6 +198,8 @@ void *rocshmem_amd_pe_ptr(const void *ptr, int pe);
 size_t rocshmem_amd_heap_size(void);
 size_t rocshmem_amd_heap_used(void);
 size_t rocshmem_amd_heap_avail(void);
+/* Bytes between the slices of consecutive PEs (0 with one process per PE,
+ * where the slices are separate mappings: use rocshmem_amd_pe_ptr). */
 size_t rocshmem_amd_pe_stride(void);
 /* Bytes of the one device allocation that holds the P slices (no reference
  * counterpart: there every PE allocates its own heap, src/memory/heap_memory.hpp).
