@@ -329,6 +329,10 @@ void heap_held(size_t *total, size_t *idle) {
   held_unlocked(total, idle);
 }
 
+// Default bound on the polls of one device wait in a process that is one PE of
+// a job (a poll of a word in the heap takes 0.5-1 us on MI355X).
+constexpr uint64_t kProcessSpinLimit = 400000000ull;
+
 int Runtime::init(int want_npes, size_t want_heap) {
   if (live) return 0;
   int ndev = 0;
@@ -418,19 +422,49 @@ int Runtime::init(int want_npes, size_t want_heap) {
     char *own = kept.own;
     RT_CHECK_HIP(hipMemset(own, 0, block_bytes));
     RT_CHECK_HIP(hipDeviceSynchronize());
-    static_assert(sizeof(hipIpcMemHandle_t) <= kBlobBytes, "IPC handle larger than a publish area");
-    procs().publish(&kept.handle[acting_pe], sizeof(hipIpcMemHandle_t));
+    // What every PE tells the others: the handle of its block and how the
+    // block is laid out.  The layouts must agree — a peer's sync pads are
+    // found at the same offset as one's own — so a job whose processes were
+    // given different heap sizes or team counts ends here, with a message,
+    // and not in a kernel that writes past a smaller peer block.
+    struct Announce {
+      hipIpcMemHandle_t handle;
+      uint64_t slice_bytes, ws_bytes;
+      uint32_t npes, cached;
+    };
+    static_assert(sizeof(Announce) <= kBlobBytes, "announcement larger than a publish area");
+    Announce mine{};
+    mine.handle = kept.handle[acting_pe];
+    mine.slice_bytes = slice_bytes;
+    mine.ws_bytes = ws_stride;
+    mine.npes = static_cast<uint32_t>(npes);
+    mine.cached = heap_cached_mode() ? 1u : 0u;
+    procs().publish(&mine, sizeof(mine));
     if (procs().barrier_world() != 0) _Exit(EXIT_FAILURE);
     peer_base.assign(npes, nullptr);
     peer_base[acting_pe] = own;
     for (int p = 0; p < npes; ++p) {
       if (p == acting_pe) continue;
-      hipIpcMemHandle_t theirs;
+      Announce theirs{};
       procs().fetch(p, &theirs, sizeof(theirs));
-      if (!kept.mapped[p] || memcmp(&theirs, &kept.handle[p], sizeof(theirs)) != 0) {
-        RT_CHECK_HIP(hipIpcOpenMemHandle(reinterpret_cast<void **>(&kept.mapped[p]), theirs,
+      if (theirs.slice_bytes != mine.slice_bytes || theirs.ws_bytes != mine.ws_bytes ||
+          theirs.npes != mine.npes) {
+        fprintf(stderr,
+                "rocshmem: PE %d and PE %d disagree about the job: %u PEs, %llu + %llu bytes per PE here, "
+                "%u PEs, %llu + %llu there (every process needs the same ROCSHMEM_HEAP_SIZE and "
+                "ROCSHMEM_MAX_NUM_TEAMS)\n",
+                acting_pe, p, mine.npes, static_cast<unsigned long long>(mine.slice_bytes),
+                static_cast<unsigned long long>(mine.ws_bytes), theirs.npes,
+                static_cast<unsigned long long>(theirs.slice_bytes),
+                static_cast<unsigned long long>(theirs.ws_bytes));
+        fflush(nullptr);
+        procs().request_abort(EXIT_FAILURE);
+        _Exit(EXIT_FAILURE);
+      }
+      if (!kept.mapped[p] || memcmp(&theirs.handle, &kept.handle[p], sizeof(theirs.handle)) != 0) {
+        RT_CHECK_HIP(hipIpcOpenMemHandle(reinterpret_cast<void **>(&kept.mapped[p]), theirs.handle,
                                          hipIpcMemLazyEnablePeerAccess));
-        kept.handle[p] = theirs;
+        kept.handle[p] = theirs.handle;
       }
       peer_base[p] = kept.mapped[p];
     }
@@ -643,7 +677,11 @@ int Runtime::init(int want_npes, size_t want_heap) {
   state.ws_base = ws_of(0);
   state.nt_bytes = env_size("ROCSHMEM_NT_THRESHOLD", detail::kNonTemporalBytes);
   state.coalesce_puts = env_size("ROCSHMEM_COALESCE_PUTS", 1) != 0 ? 1 : 0;
-  state.spin_limit = env_size("ROCSHMEM_EMU_SPIN_LIMIT", 0);
+  // Device waits spin for ever by default, as the reference's do.  Between
+  // processes the peer that would end a wait may have died: there the default
+  // is a limit generous enough for any live job (minutes of polling), after
+  // which the wait gives up and is counted (rocshmem_amd_waits_given_up).
+  state.spin_limit = env_size("ROCSHMEM_EMU_SPIN_LIMIT", nprocs ? kProcessSpinLimit : 0);
   RT_CHECK_HIP(hipMalloc(reinterpret_cast<void **>(&d_gave_up), sizeof(unsigned long long)));
   RT_CHECK_HIP(hipMemset(d_gave_up, 0, sizeof(unsigned long long)));
   state.gave_up = d_gave_up;

@@ -34,6 +34,11 @@ def main():
     P = int(os.environ["ROCSHMEM_EMU_PROCS"])
     me = int(os.environ["ROCSHMEM_EMU_RANK"])
     l = L.load()
+    if sys.argv[1:] == ["unequal-heaps"]:
+        # every PE asks for another heap size: rocshmem_init ends the job with a message
+        l.init(0, (64 << 20) * (me + 1))
+        print("init returned", me)
+        return
     assert l.init(0, HEAP) == 0
     assert (l.n_pes(), l.my_pe()) == (P, me)
     nxt, prv = (me + 1) % P, (me - 1) % P

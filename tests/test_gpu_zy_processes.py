@@ -22,3 +22,18 @@ def test_every_operation_between_processes_matches_the_oracle(rt, nprocs):
     assert status == 0, [o[-1500:] for o in outs]
     for pe, o in enumerate(outs):
         assert "ok %d" % pe in o, o[-1500:]
+
+
+def test_processes_that_disagree_about_the_heap_are_stopped_at_init(rt):
+    """A peer's barrier pads are found at the same offset as one's own, so a
+    job whose processes bring different heap sizes must not get as far as a
+    kernel: rocshmem_init compares the announced layouts and ends the job."""
+    from rocshmem_amd import launch
+    rt.down()
+    env = dict(os.environ)
+    env.pop("ROCSHMEM_EMU_NPES", None)
+    status, outs = launch.run(2, WORKER + ["unequal-heaps"], timeout=60, env=env, capture=True)
+    assert status != 0, outs
+    text = "".join(outs)
+    assert "disagree about the job" in text, text[-800:]
+    assert "init returned" not in text
