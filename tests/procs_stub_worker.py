@@ -1,0 +1,213 @@
+"""Host logic of the runtime on a machine without a GPU: a child process of
+tests/test_host_logic_without_gpu.py, run with tests/hip_stub's stand-in for
+the HIP runtime in front of the real one.  Kernels do not run under it (only
+the whole-GPU copy kernel is carried out, with bounds checks), so everything
+here is about bring-up, bookkeeping, address resolution and host-initiated
+copies.  One process (argv[1] == "one") or one PE of a job of processes."""
+import ctypes as C
+import os
+import struct
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, ROOT)
+from oracle import pyoracle as orc  # noqa: E402  (the checker)
+from rocshmem_amd import lib as L  # noqa: E402
+
+HEAP = 8 << 20
+TWO_MIB = 2 << 20
+NOSTORE = 1
+
+
+class CtxHandle(C.Structure):  # rocshmem_ctx_t (include/rocshmem/rocshmem_common.hpp)
+    _fields_ = [("ctx_opaque", C.c_void_p), ("team_opaque", C.c_void_p)]
+
+
+def get_bytes(l, dev, n, dtype=np.uint8):
+    out = np.empty(n // np.dtype(dtype).itemsize, dtype)
+    assert l.copy_out(out.ctypes.data, dev, n) == 0
+    return out
+
+
+def put_bytes(l, dev, a):
+    a = np.ascontiguousarray(a)
+    assert l.copy_in(dev, a.ctypes.data, a.nbytes) == 0
+
+
+def context_fields(l, options):
+    """The device-side context object that rocshmem_ctx_create hands out, field
+    by field (detail/state.hpp: struct Context, 64 bytes)."""
+    create = l.cdll._ZN8rocshmem19rocshmem_ctx_createElPNS_14rocshmem_ctx_tE
+    create.restype, create.argtypes = C.c_int, [C.c_long, C.POINTER(CtxHandle)]
+    destroy = l.cdll._ZN8rocshmem20rocshmem_ctx_destroyENS_14rocshmem_ctx_tE
+    destroy.restype, destroy.argtypes = None, [CtxHandle]
+    h = CtxHandle()
+    assert create(options, C.byref(h)) == 0 and h.ctx_opaque
+    raw = get_bytes(l, h.ctx_opaque, 64).tobytes()
+    names = ("pe_stride", "my_pe", "options", "peer_delta", "heap_base", "ws_stride", "num_pes", "pool_slot",
+             "tinfo", "world_sync")
+    f = dict(zip(names, struct.unpack("<QiIQQQiiQQ", raw)))
+    assert l.ctx_pe(h.ctx_opaque) == f["my_pe"]
+    destroy(h)
+    return f
+
+
+def check_contexts(l, P, me, probe):
+    """What device code would compute from a context of this PE: the address
+    of `probe` on every PE, compared with the host's own resolution."""
+    for options in (0, NOSTORE):
+        f = context_fields(l, options)
+        assert (f["my_pe"], f["num_pes"], f["options"] & NOSTORE) == (me, P, options)
+        assert f["pe_stride"] == l.pe_stride()
+        table = get_bytes(l, f["peer_delta"], 8 * P, np.int64)
+        for p in range(P):
+            by_table = probe + int(table[p])
+            by_stride = probe + (p - me) * f["pe_stride"]
+            assert by_table == l.pe_ptr(probe, p), (me, p, "table")
+            if f["pe_stride"]:
+                assert by_stride == l.pe_ptr(probe, p), (me, p, "stride")
+        # the PE's own work/sync area starts where its slice ends
+        slice_bytes = (l.heap_size() + TWO_MIB - 1) // TWO_MIB * TWO_MIB
+        if f["pe_stride"] == 0:
+            assert f["world_sync"] - f["heap_base"] == slice_bytes
+            for p in range(P):  # and a peer's is readable through the same table entry
+                get_bytes(l, f["world_sync"] + int(table[p]), 64)
+    return True
+
+
+def ring_copies(l, P, me, seed):
+    """Host-called and whole-GPU-kernel copies to the next PE and from the
+    previous one, ragged sizes and offsets; every PE checks its own slice."""
+    nxt, prv = (me + 1) % P, (me - 1) % P
+    n = 70001
+    src, dst = l.malloc(n + 64), l.malloc(n + 64)
+    assert src and dst
+    for case, (off_s, off_d, size) in enumerate([(0, 0, n), (1, 3, 4099), (5, 2, 1), (16, 7, 65536), (3, 3, 0)]):
+        for how in ("host_put", "host_get", "bulk_put", "bulk_get"):
+            put_bytes(l, src, orc.fill_u8(n + 64, seed + case, me))
+            assert l.fill(dst, 0xA5, n + 64) == 0
+            assert l.barrier_all() == 0
+            if how == "host_put":
+                assert l.host_putmem(dst + off_d, src + off_s, size, me, nxt) == 0
+            elif how == "host_get":
+                assert l.host_getmem(dst + off_d, src + off_s, size, me, prv) == 0
+            elif how == "bulk_put":
+                assert l.putmem(dst + off_d, src + off_s, size, me, nxt, None) == 0
+            else:
+                assert l.getmem(dst + off_d, src + off_s, size, me, prv, None) == 0
+            assert l.barrier_all() == 0
+            want = np.full(n + 64, 0xA5, np.uint8)
+            want[off_d:off_d + size] = orc.fill_u8(n + 64, seed + case, prv)[off_s:off_s + size]
+            got = get_bytes(l, dst, n + 64)
+            assert np.array_equal(got, want), (how, case, me)
+    l.free(src)
+    l.free(dst)
+
+
+def one_process():
+    l = L.load()
+    for P in (8, 3):
+        assert l.init(P, HEAP) == 0
+        assert l.n_pes() == P and l.pe_stride() >= HEAP
+        probe = l.malloc(4096)
+        for me in range(P):
+            l.set_pe(me)
+            mine = l.pe_ptr(probe, me)
+            check_contexts(l, P, me, mine)
+            for p in range(P):
+                assert l.pe_ptr(mine, p) - mine == (p - me) * l.pe_stride()
+        l.set_pe(0)
+        # copies between every pair of PEs through the whole-GPU kernel's driver
+        n = 10007
+        a, b = l.malloc(n), l.malloc(n)
+        for me in range(P):
+            put_bytes(l, l.pe_ptr(a, me), orc.fill_u8(n, 5, me))
+        for me in range(P):
+            for pe in range(P):
+                assert l.putmem(l.pe_ptr(b, me), l.pe_ptr(a, me), n, me, pe, None) == 0
+                assert np.array_equal(get_bytes(l, l.pe_ptr(b, pe), n), orc.fill_u8(n, 5, me))
+                assert l.getmem(l.pe_ptr(b, me) + 1, l.pe_ptr(a, me) + 2, 333, me, pe, None) == 0
+                assert np.array_equal(get_bytes(l, l.pe_ptr(b, me) + 1, 333), orc.fill_u8(n, 5, pe)[2:335])
+        assert l.finalize() == 0
+    print("one process ok")
+
+
+def one_pe_of_a_job():
+    P = int(os.environ["ROCSHMEM_EMU_PROCS"])
+    me = int(os.environ["ROCSHMEM_EMU_RANK"])
+    l = L.load()
+    if sys.argv[1] == "unequal-heaps":
+        l.init(0, (4 << 20) * (me + 1))
+        print("init returned", me)
+        return
+    for bring_up in range(2):  # the second rocshmem_init finds the block and the mappings of the first
+        assert l.init(0, HEAP) == 0
+        assert (l.n_pes(), l.my_pe(), l.pe_stride()) == (P, me, 0)
+        probe = l.malloc(4096)
+        assert l.pe_ptr(probe, me) == probe
+        assert len({l.pe_ptr(probe, p) for p in range(P)}) == P
+        check_contexts(l, P, me, probe)
+        # every PE sees every PE's bytes at the address the table gives
+        put_bytes(l, probe, orc.fill_u8(4096, 40 + bring_up, me))
+        assert l.barrier_all() == 0
+        for p in range(P):
+            assert np.array_equal(get_bytes(l, l.pe_ptr(probe, p), 4096), orc.fill_u8(4096, 40 + bring_up, p))
+        assert l.barrier_all() == 0
+        ring_copies(l, P, me, 100 * bring_up)
+
+        # block moves between the processes (they pull with the copy kernel)
+        nb = 5003
+        s, d = l.malloc(P * nb), l.malloc(P * nb)
+        srcs = [orc.fill_u8(P * nb, 77, p) for p in range(P)]
+        put_bytes(l, s, srcs[me])
+        world = l.team_world()
+        assert l.barrier_all() == 0
+        assert l.alltoallmem(world, d, s, nb, None) == 0
+        assert np.array_equal(get_bytes(l, d, P * nb), orc.alltoall(srcs, nb)[me])
+        assert l.barrier_all() == 0
+        assert l.fcollectmem(world, d, s, nb, None) == 0
+        assert np.array_equal(get_bytes(l, d, P * nb), orc.fcollect([x[:nb] for x in srcs], nb)[me])
+        assert l.barrier_all() == 0
+        assert l.fill(d, 0x11, P * nb) == 0
+        assert l.barrier_all() == 0
+        assert l.broadcastmem(world, d, s, nb, P - 1, None) == 0
+        want = [np.full(nb, 0x11, np.uint8) for _ in range(P)]
+        orc.broadcast([x[:nb] for x in srcs], want, nb, P - 1)
+        assert np.array_equal(get_bytes(l, d, nb), want[me])
+        assert l.barrier_all() == 0
+
+        # a team of the even PEs: made by its members, met by the whole parent team
+        team = C.c_void_p()
+        assert l.team_split_strided(world, 0, 2, (P + 1) // 2, C.byref(team)) == 0
+        if me % 2 == 0:
+            assert team.value and (l.team_n_pes(team), l.team_my_pe(team)) == ((P + 1) // 2, me // 2)
+            assert l.broadcastmem(team, d, s, nb, 0, None) == 0
+            if me:
+                assert np.array_equal(get_bytes(l, d, nb), srcs[0][:nb])
+        else:
+            assert not team.value
+        assert l.barrier_all() == 0
+
+        # what belongs to the one-process harness is refused before anything is launched
+        assert l.wg_reduce(L.INT, L.SUM, world, d, s, 4, 64, None) == -1
+        assert l.rma(L.PUT, L.WG, d, s, 16, 0, (me + 1) % P, me, 1, 64, 1, None) == -1
+        assert l.fill_every_pe(d, 0, 16, None) == -1
+        for p in (s, d, probe):
+            l.free(p)
+        assert l.finalize() == 0
+    print("ok", me)
+
+
+if __name__ == "__main__":
+    if sys.argv[1] == "one":
+        one_process()
+    elif sys.argv[1] == "memset-outside":
+        l = L.load()
+        assert l.init(2, HEAP) == 0
+        a = l.malloc(64)
+        l.fill(a + (1 << 40), 0, 64)  # the stand-in ends the process: on a GPU this is a fault
+        print("survived")
+    else:
+        one_pe_of_a_job()

@@ -1,0 +1,71 @@
+"""The runtime's host logic without a GPU: rocshmem_init in one process and
+between the processes of a job (handle exchange, layout check, peer table,
+contexts), address resolution, the allocator's symmetry, team bookkeeping and
+host-initiated copies, with tests/hip_stub's stand-in for the HIP runtime in
+front of the real one for the child processes that load the product library.
+Kernels do not run there — launches are counted and dropped, except the
+whole-GPU copy kernel, which the stand-in carries out after checking both
+ranges against the memory the process has allocated or mapped — so nothing
+here is a parity result of device code; those are the -m gpu tests.
+
+What these tests pin is what a kernel would be GIVEN: the context fields and
+the table from which device code forms a peer's address
+(detail/state.hpp::remote_addr; the reference's ipc_bases[pe] + offset,
+src/ipc/context_ipc_device.cpp:62-69) must give the address the host resolves,
+in one process and across processes, and a host-computed address that leaves
+the mapped memory ends the test instead of faulting a GPU."""
+import os
+import subprocess
+import sys
+
+import pytest
+
+from rocshmem_amd import launch
+from rocshmem_amd import lib as L
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+STUB_DIR = os.path.join(HERE, "hip_stub")
+STUB = os.path.join(STUB_DIR, "_build", "libamdhip64.so.7")
+WORKER = [sys.executable, os.path.join(HERE, "procs_stub_worker.py")]
+
+
+@pytest.fixture(scope="module")
+def stub_env():
+    if not os.path.exists(L.LIB_PATH):
+        pytest.skip("library not built")
+    r = subprocess.run(["make", "-C", STUB_DIR], capture_output=True, text=True)
+    if r.returncode != 0 or not os.path.exists(STUB):
+        pytest.skip("the HIP stand-in does not build here: " + r.stderr[-300:])
+    env = dict(os.environ)
+    env["LD_LIBRARY_PATH"] = os.path.dirname(STUB) + os.pathsep + env.get("LD_LIBRARY_PATH", "")
+    for name in ("ROCSHMEM_EMU_NPES", "ROCSHMEM_EMU_SPREAD", "ROCSHMEM_EMU_HEAP_CACHED", "ROCSHMEM_HEAP_SIZE"):
+        env.pop(name, None)
+    return env
+
+
+def test_one_process_contexts_and_copies(stub_env):
+    r = subprocess.run(WORKER + ["one"], env=stub_env, capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, (r.stdout[-800:], r.stderr[-1500:])
+    assert "one process ok" in r.stdout
+
+
+@pytest.mark.parametrize("nprocs", [2, 5])
+def test_a_job_of_processes_brings_up_and_moves_data(stub_env, nprocs):
+    status, outs = launch.run(nprocs, WORKER + ["job"], timeout=120, env=stub_env, capture=True)
+    assert status == 0, [o[-1500:] for o in outs]
+    for pe, o in enumerate(outs):
+        assert "ok %d" % pe in o, o[-1500:]
+
+
+def test_processes_that_disagree_about_the_heap_are_stopped_at_init(stub_env):
+    status, outs = launch.run(2, WORKER + ["unequal-heaps"], timeout=60, env=stub_env, capture=True)
+    text = "".join(outs)
+    assert status != 0 and "disagree about the job" in text, text[-800:]
+    assert "init returned" not in text
+
+
+def test_the_stand_in_ends_a_process_that_leaves_its_memory(stub_env):
+    r = subprocess.run(WORKER + ["memset-outside"], env=stub_env, capture_output=True, text=True, timeout=60)
+    assert r.returncode == 97, (r.returncode, r.stderr[-500:])
+    assert "not inside memory this process has allocated or mapped" in r.stderr
+    assert "survived" not in r.stdout
