@@ -69,3 +69,48 @@ def test_the_stand_in_ends_a_process_that_leaves_its_memory(stub_env):
     assert r.returncode == 97, (r.returncode, r.stderr[-500:])
     assert "not inside memory this process has allocated or mapped" in r.stderr
     assert "survived" not in r.stdout
+
+
+# The reference's host programs (tests/sos_tests, built unchanged by
+# oracle/Makefile) that get by without any kernel of the library — puts, gets,
+# barriers, broadcasts, allocation, teams, global_exit — and that do not race
+# by construction: as 2 and 4 processes under the stand-in they exercise the
+# host API between processes end to end, each program checking its own data.
+SOS_DIR = os.path.join(os.path.dirname(HERE), "oracle", "_ref", "sos")
+SOS_WITHOUT_KERNELS = ["hello", "barrier", "put1", "get1", "bigget", "circular_shift", "shmalloc",
+                       "asym_alloc", "bcast", "bcast_flood", "broadcast_active_set", "global_exit",
+                       "get_nbi", "shmem_team_translate", "shmem_team_reuse_teams", "cxx_test_shmem_p",
+                       "cxx_test_shmem_g"]
+
+
+@pytest.mark.skipif(not os.path.isdir(SOS_DIR), reason="oracle/_ref/sos is built where the reference tree exists")
+@pytest.mark.parametrize("nprocs", [2, 4])
+@pytest.mark.parametrize("name", SOS_WITHOUT_KERNELS)
+def test_reference_host_programs_as_processes(stub_env, name, nprocs):
+    prog = os.path.join(SOS_DIR, name)
+    if not os.access(prog, os.X_OK):
+        pytest.skip("not built")
+    env = dict(stub_env, ROCSHMEM_HEAP_SIZE=str(64 << 20))
+    status, outs = launch.run(nprocs, [prog], timeout=60, env=env, capture=True)
+    assert status == 0, (name, nprocs, [o[-600:] for o in outs])
+
+
+# The same with a host thread per PE (the builds with their main() run once per
+# PE): there the host broadcast is a kernel of its own, which the stand-in
+# drops, so the broadcast programs are left to the GPU tests.
+SOS_THREADS_DIR = os.path.join(os.path.dirname(HERE), "oracle", "_ref", "sos_threads")
+SOS_THREADS_WITHOUT_KERNELS = [n for n in SOS_WITHOUT_KERNELS
+                               if n not in ("bcast", "bcast_flood", "broadcast_active_set")]
+
+
+@pytest.mark.skipif(not os.path.isdir(SOS_THREADS_DIR),
+                    reason="oracle/_ref/sos_threads is built where the reference tree exists")
+@pytest.mark.parametrize("npes", [2, 8])
+@pytest.mark.parametrize("name", SOS_THREADS_WITHOUT_KERNELS)
+def test_reference_host_programs_with_a_thread_per_pe(stub_env, name, npes):
+    prog = os.path.join(SOS_THREADS_DIR, name)
+    if not os.access(prog, os.X_OK):
+        pytest.skip("not built")
+    env = dict(stub_env, ROCSHMEM_EMU_NPES=str(npes), ROCSHMEM_HEAP_SIZE=str(64 << 20))
+    r = subprocess.run([prog], env=env, capture_output=True, text=True, timeout=60)
+    assert r.returncode == 0, (name, npes, r.stdout[-600:], r.stderr[-600:])
