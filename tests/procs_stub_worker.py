@@ -200,9 +200,92 @@ def one_pe_of_a_job():
     print("ok", me)
 
 
+def refusals():
+    """Calls that must be refused on the host: each returns -1 and the stand-in
+    sees no launch (what rocshmem_amd.h promises: pointers and sizes are
+    checked against the heap before anything is enqueued)."""
+    l = L.load()
+    P, heap = 4, HEAP
+    assert l.init(P, heap) == 0
+    stub = C.CDLL("libamdhip64.so.7")
+    stub.hip_stub_counts.argtypes = [C.POINTER(C.c_ulonglong), C.POINTER(C.c_ulonglong)]
+
+    def launches():
+        n = C.c_ulonglong()
+        stub.hip_stub_counts(C.byref(n), None)
+        return n.value
+
+    a, b = l.malloc(4096), l.malloc(4096)
+    last = l.malloc(heap // 4)        # some block; its PE-0 slice ends at base + heap
+    base = a - (a - l.pe_ptr(a, 0))   # a is PE 0's
+    end = base + l.heap_size()        # first byte past PE 0's usable slice
+    local = l.dev_alloc(4096)
+    world = l.team_world()
+    outside = np.zeros(64, np.uint8).ctypes.data  # host memory, not in the heap
+    calls = [
+        # a PE that does not exist, either side
+        lambda: l.rma(L.PUT, L.WG, a, b, 64, 0, 0, P, 1, 64, 1, None),
+        lambda: l.rma(L.PUT, L.WG, a, b, 64, 0, -1, 1, 1, 64, 1, None),
+        # launch shapes
+        lambda: l.rma(L.PUT, L.WG, a, b, 64, 0, 0, 1, 0, 64, 1, None),
+        lambda: l.rma(L.PUT, L.WG, a, b, 64, 0, 0, 1, 1, 2048, 1, None),
+        lambda: l.rma(9, L.WG, a, b, 64, 0, 0, 1, 1, 64, 1, None),
+        lambda: l.rma(L.PUT, 7, a, b, 64, 0, 0, 1, 1, 64, 1, None),
+        # the symmetric side straddles the end of the slice, or is not symmetric at all
+        lambda: l.rma(L.PUT, L.WG, end - 8, b, 16, 0, 0, 1, 1, 64, 1, None),
+        lambda: l.rma(L.GET, L.WG, local, end - 8, 16, 0, 0, 1, 1, 64, 1, None),
+        lambda: l.rma(L.PUT, L.WG, local, b, 16, 0, 0, 1, 1, 64, 1, None),
+        lambda: l.rma(L.PUT, L.WG, l.pe_ptr(a, 1), b, 16, 0, 0, 1, 1, 64, 1, None),  # another PE's address
+        lambda: l.putmem(end - 8, b, 16, 0, 1, None),
+        lambda: l.getmem(local, end - 8, 16, 0, 1, None),
+        lambda: l.putmem(a, b, 16, 0, P, None),
+        lambda: l.host_putmem(end - 8, outside, 16, 0, 1),
+        lambda: l.host_getmem(outside, end - 8, 16, 0, 1),
+        lambda: l.host_putmem(a, outside, 16, P, 1),
+        lambda: l.rma_staged(L.WG, a, local, local, 1 << 20, 0, 1, 64, None),
+        lambda: l.rma_staged(L.WG, end - 8, local, local, 64, 0, 1, 64, None),
+        lambda: l.put_signal(L.WG, end - 8, local, 64, b, 1, L.SIGNAL_SET, 0, 1, 1, 64, 1, None),
+        lambda: l.put_signal(L.WG, a, local, 64, end - 4, 1, L.SIGNAL_SET, 0, 1, 1, 64, 1, None),
+        lambda: l.amo(L.AMO_FETCH_ADD, L.LONG, end - 8, 4, local, None, None, None, 4, 0, 1, 64, None),
+        lambda: l.amo(L.AMO_FETCH_ADD, L.LONG, a, 0, local, None, None, None, 4, 0, 1, 64, None),
+        lambda: l.amo(L.AMO_FETCH_ADD, L.LONG, a, 4, None, None, None, None, 4, 0, 1, 64, None),
+        # collectives: sets that leave the world, buffers that leave the slice, teams that are none
+        lambda: l.to_all(L.INT, L.SUM, a, b, 4, 0, 0, P + 1, None),
+        lambda: l.to_all(L.INT, L.SUM, a, b, 4, 2, 1, 2, None),
+        lambda: l.to_all(L.INT, L.SUM, a, b, -1, 0, 0, P, None),
+        lambda: l.to_all(L.INT, L.SUM, end - 8, b, 4, 0, 0, P, None),
+        lambda: l.to_all(99, L.SUM, a, b, 4, 0, 0, P, None),
+        lambda: l.reduce(L.INT, L.SUM, None, a, b, 4, None),
+        lambda: l.alltoallmem(world, a, b, heap // 2, None),     # P blocks of that size leave the slice
+        lambda: l.fcollectmem(world, a, b, heap // 2, None),
+        lambda: l.broadcastmem(world, a, b, 64, P, None),
+        lambda: l.broadcastmem(world, end - 8, b, 64, 0, None),
+        lambda: l.broadcast_active_set(a, b, 64, 5, 0, 0, P, None),
+        lambda: l.wg_reduce(L.INT, L.SUM, world, a, b, 4, 0, None),
+        lambda: l.wg_reduce(L.INT, L.SUM, None, a, b, 4, 64, None),
+        lambda: l.wg_alltoall(4, world, a, b, heap // 8, 64, None),
+        lambda: l.wg_sync(L.BARRIER_ALL, world, end - 4, 1, 64, None),
+        lambda: l.pingpong(a, b, 64, 1, 1, 0, 0, 64, None, None, None),
+        lambda: l.pingpong(a, b, 64, 1, 500, 0, 1, 64, None, None, None),
+    ]
+    for i, call in enumerate(calls):
+        before = launches()
+        assert call() == -1, i
+        assert launches() == before, (i, "launched something")
+    # and a call that is accepted does launch
+    before = launches()
+    assert l.rma(L.PUT, L.WG, a, b, 64, 0, 0, 1, 1, 64, 1, None) == 0
+    assert launches() == before + 1
+    assert last
+    l.finalize()
+    print("refusals ok", len(calls))
+
+
 if __name__ == "__main__":
     if sys.argv[1] == "one":
         one_process()
+    elif sys.argv[1] == "refusals":
+        refusals()
     elif sys.argv[1] == "memset-outside":
         l = L.load()
         assert l.init(2, HEAP) == 0

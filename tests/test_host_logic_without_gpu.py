@@ -49,6 +49,15 @@ def test_one_process_contexts_and_copies(stub_env):
     assert "one process ok" in r.stdout
 
 
+def test_refused_calls_launch_nothing(stub_env):
+    """include/rocshmem_amd.h: every driver validates pointers and sizes against
+    the heap on the host before launching.  Forty calls that must be refused,
+    with the stand-in counting the launches in between."""
+    r = subprocess.run(WORKER + ["refusals"], env=stub_env, capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, (r.stdout[-800:], r.stderr[-1500:])
+    assert "refusals ok" in r.stdout
+
+
 @pytest.mark.parametrize("nprocs", [2, 5])
 def test_a_job_of_processes_brings_up_and_moves_data(stub_env, nprocs):
     status, outs = launch.run(nprocs, WORKER + ["job"], timeout=120, env=stub_env, capture=True)
