@@ -42,7 +42,7 @@ struct Block {
 std::mutex g_lock;
 std::map<uintptr_t, Block> g_blocks;           // by base address
 std::map<const void *, std::string> g_kernels;  // host stub address -> device name
-unsigned long long g_launches = 0, g_copies_run = 0;
+unsigned long long g_launches = 0, g_copies_run = 0, g_alloc_calls = 0;
 thread_local hipError_t g_last = hipSuccess;
 
 constexpr size_t kShareFrom = size_t{1} << 20;
@@ -67,6 +67,10 @@ const Block *holder(const void *p, size_t n, uintptr_t *base_out = nullptr) {
 }
 
 hipError_t allocate(void **ptr, size_t bytes) {
+  {
+    std::lock_guard<std::mutex> guard(g_lock);
+    ++g_alloc_calls;
+  }
   if (!ptr) return hipErrorInvalidValue;
   if (!bytes) {
     *ptr = nullptr;
@@ -168,6 +172,12 @@ void hip_stub_counts(unsigned long long *launches, unsigned long long *copies_ru
   if (copies_run) *copies_run = g_copies_run;
 }
 
+// Calls of hipMalloc / hipExtMallocWithFlags / hipHostMalloc / hipFree / hipHostFree so far.
+unsigned long long hip_stub_alloc_calls(void) {
+  std::lock_guard<std::mutex> guard(g_lock);
+  return g_alloc_calls;
+}
+
 // ---- device, errors ----------------------------------------------------------
 hipError_t hipGetDeviceCount(int *n) {
   *n = 1;
@@ -206,16 +216,25 @@ hipError_t hipMemGetInfo(size_t *free_bytes, size_t *total_bytes) {
 hipError_t hipMalloc(void **ptr, size_t bytes) { return allocate(ptr, bytes); }
 hipError_t hipExtMallocWithFlags(void **ptr, size_t bytes, unsigned int) { return allocate(ptr, bytes); }
 hipError_t hipHostMalloc(void **ptr, size_t bytes, unsigned int) {
+  {
+    std::lock_guard<std::mutex> guard(g_lock);
+    ++g_alloc_calls;
+  }
   *ptr = calloc(1, bytes ? bytes : 1);
   return *ptr ? hipSuccess : hipErrorOutOfMemory;
 }
 hipError_t hipHostFree(void *ptr) {
+  {
+    std::lock_guard<std::mutex> guard(g_lock);
+    ++g_alloc_calls;
+  }
   free(ptr);
   return hipSuccess;
 }
 hipError_t hipFree(void *ptr) {
-  if (!ptr) return hipSuccess;
   std::lock_guard<std::mutex> guard(g_lock);
+  ++g_alloc_calls;
+  if (!ptr) return hipSuccess;
   auto it = g_blocks.find(reinterpret_cast<uintptr_t>(ptr));
   if (it == g_blocks.end()) return hipErrorInvalidValue;
   if (it->second.fd >= 0 || it->second.mapped) {

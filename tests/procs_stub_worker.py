@@ -281,9 +281,40 @@ def refusals():
     print("refusals ok", len(calls))
 
 
+def no_alloc():
+    """rocshmem_amd_wg_reduce_teams_static must not allocate or free anything
+    (it is the entry point for callers that cannot); its sibling does.  The
+    stand-in counts every allocating and freeing call of the HIP runtime."""
+    l = L.load()
+    P = 8
+    assert l.init(P, HEAP) == 0
+    stub = C.CDLL("libamdhip64.so.7")
+    stub.hip_stub_alloc_calls.restype = C.c_ulonglong
+    n_teams = 5
+    teams = (C.c_void_p * n_teams)()
+    for t in range(n_teams):
+        h = C.c_void_p()
+        assert l.team_split_strided(l.team_world(), 0, 1, P, C.byref(h)) == 0 and h.value
+        teams[t] = h.value
+    n = 4099
+    src, dst = l.malloc(n * 4), l.malloc(n * 4)
+    l.wg_reduce_teams_static(L.INT, L.SUM, teams, n_teams, dst, src, n, 0, 64, 1, None)  # first call: set-up
+    before = stub.hip_stub_alloc_calls()
+    for _ in range(3):
+        assert l.wg_reduce_teams_static(L.INT, L.SUM, teams, n_teams, dst, src, n, 0, 64, 1, None) == 0
+        assert l.wg_reduce_teams_static(L.INT, L.SUM, teams, 300, dst, src, n, 0, 64, 1, None) == -1
+    assert stub.hip_stub_alloc_calls() == before, "the static entry point allocated or freed"
+    assert l.wg_reduce_teams(L.INT, L.SUM, teams, n_teams, dst, src, n, 0, 64, 1, None) == 0
+    assert stub.hip_stub_alloc_calls() > before, "the counter does not see the allocating entry point"
+    l.finalize()
+    print("no alloc ok")
+
+
 if __name__ == "__main__":
     if sys.argv[1] == "one":
         one_process()
+    elif sys.argv[1] == "no-alloc":
+        no_alloc()
     elif sys.argv[1] == "refusals":
         refusals()
     elif sys.argv[1] == "memset-outside":

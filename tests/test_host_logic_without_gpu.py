@@ -58,6 +58,12 @@ def test_refused_calls_launch_nothing(stub_env):
     assert "refusals ok" in r.stdout
 
 
+def test_the_entry_point_for_callers_that_cannot_allocate_allocates_nothing(stub_env):
+    r = subprocess.run(WORKER + ["no-alloc"], env=stub_env, capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, (r.stdout[-800:], r.stderr[-1500:])
+    assert "no alloc ok" in r.stdout
+
+
 @pytest.mark.parametrize("nprocs", [2, 5])
 def test_a_job_of_processes_brings_up_and_moves_data(stub_env, nprocs):
     status, outs = launch.run(nprocs, WORKER + ["job"], timeout=120, env=stub_env, capture=True)
