@@ -142,6 +142,20 @@ def one_pe_of_a_job():
         l.init(0, (4 << 20) * (me + 1))
         print("init returned", me)
         return
+    if sys.argv[1] == "one-dies":
+        assert l.init(0, HEAP) == 0
+        if me == 1:
+            os._exit(3)          # without finalize, without a word to the others
+        l.barrier_all()          # never completes: the wait runs out and ends this process too
+        print("barrier returned", me)
+        return
+    if sys.argv[1] == "global-exit":
+        assert l.init(0, HEAP) == 0
+        if me == P - 1:
+            l.cdll._ZN8rocshmem20rocshmem_global_exitEi(7)
+        l.barrier_all()          # the others leave here, with the status asked for
+        print("barrier returned", me)
+        return
     for bring_up in range(2):  # the second rocshmem_init finds the block and the mappings of the first
         assert l.init(0, HEAP) == 0
         assert (l.n_pes(), l.my_pe(), l.pe_stride()) == (P, me, 0)

@@ -79,6 +79,27 @@ def test_processes_that_disagree_about_the_heap_are_stopped_at_init(stub_env):
     assert "init returned" not in text
 
 
+def test_a_process_that_dies_does_not_leave_the_others_waiting_for_ever(stub_env):
+    """Failure handling between processes, on the CPU: the survivors' meeting
+    runs out (ROCSHMEM_EMU_RDV_TIMEOUT_S) and they end; the launcher reports
+    the first failure."""
+    import time
+    env = dict(stub_env, ROCSHMEM_EMU_RDV_TIMEOUT_S="2")
+    t0 = time.monotonic()
+    status, outs = launch.run(3, WORKER + ["one-dies"], timeout=60, env=env, capture=True)
+    assert status == 3, outs
+    assert time.monotonic() - t0 < 30
+    assert "barrier returned" not in "".join(outs)
+
+
+def test_global_exit_ends_every_process_with_its_status(stub_env):
+    """rocshmem_global_exit(status) (the reference: MPI_Abort): the caller ends
+    at once and the others at their next meeting, all with that status."""
+    status, outs = launch.run(3, WORKER + ["global-exit"], timeout=60, env=stub_env, capture=True)
+    assert status == 7, outs
+    assert "barrier returned" not in "".join(outs)
+
+
 def test_the_stand_in_ends_a_process_that_leaves_its_memory(stub_env):
     r = subprocess.run(WORKER + ["memset-outside"], env=stub_env, capture_output=True, text=True, timeout=60)
     assert r.returncode == 97, (r.returncode, r.stderr[-500:])
