@@ -11,7 +11,10 @@
  *     would, with the PE each work-group acts for given by the caller.
  *
  * Conventions
- *   - All P processing elements live in this process on one GPU.  A symmetric
+ *   - All P processing elements live in this process on one GPU, unless the
+ *     process was started as one PE of a job of processes (see "One process
+ *     per PE" below): then it acts for that PE only (`my_pe` must be it) and
+ *     the drivers that host several PEs in one launch return -1.  A symmetric
  *     address is always passed as the address on PE `my_pe` (what
  *     rocshmem_amd_malloc returned while that PE was acting, or
  *     rocshmem_amd_pe_ptr of it).
