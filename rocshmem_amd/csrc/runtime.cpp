@@ -126,7 +126,10 @@ void pe_threads_start(int npes) { g_threads.npes = npes; }
 
 // ROCSHMEM_EMU_TRACE=1: one line on stderr per arrival at a meeting point.
 bool tracing() {
-  static const bool on = getenv("ROCSHMEM_EMU_TRACE") && atoi(getenv("ROCSHMEM_EMU_TRACE")) != 0;
+  static const bool on = [] {
+    const char *v = getenv("ROCSHMEM_EMU_TRACE");
+    return v && atoi(v) != 0;
+  }();
   return on;
 }
 
