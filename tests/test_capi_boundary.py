@@ -133,3 +133,39 @@ def test_every_function_name_of_the_reference_headers_is_declared(tmp_path):
     assert r.returncode == 0, r.stderr[-3000:]
     have = function_names(out.read_text(errors="ignore"))
     assert not sorted(wanted - have), sorted(wanted - have)[:40]
+
+
+def test_the_header_is_plain_c_and_the_library_links_from_c(L, tmp_path):
+    """The boundary is a C ABI: include/rocshmem_amd.h must compile as C99
+    (pedantic) and a C program must link with the library and call it.  The
+    calls made here need no GPU: the allocator model (SingleHeap / Pow2Bins,
+    src/memory/single_heap.cpp:29-64: 128-byte minimum block, power-of-two
+    rounding, alloc(0) -> "nullptr") and the size of the rendezvous file."""
+    src = tmp_path / "c_abi.c"
+    src.write_text(r'''
+#include <stdio.h>
+#include "rocshmem_amd.h"
+#include "rocshmem_amd_probes.h"
+int main(void) {
+  void *m = rocshmem_amd_heap_model_create(0x1000000, 1u << 20);
+  uint64_t a = rocshmem_amd_heap_model_alloc(m, 1), b = rocshmem_amd_heap_model_alloc(m, 129);
+  uint64_t none = rocshmem_amd_heap_model_alloc(m, 0);
+  uint64_t used = rocshmem_amd_heap_model_used(m);
+  int freed = rocshmem_amd_heap_model_free(m, a);
+  rocshmem_amd_heap_model_destroy(m);
+  printf("%llu %llu %d %llu %d %d\n", (unsigned long long)a, (unsigned long long)b,
+         none == UINT64_MAX, (unsigned long long)used, freed, rocshmem_amd_procs_file_bytes() > 0);
+  return rocshmem_amd_n_pes() < 0;
+}
+''')
+    exe = tmp_path / "c_abi"
+    libdir = os.path.dirname(L.LIB_PATH)
+    r = subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", os.path.join(ROOT, "include"),
+                        str(src), "-o", str(exe), "-L", libdir, "-lrocshmem_amd", "-Wl,-rpath," + libdir],
+                       capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr[-1500:]
+    r = subprocess.run([str(exe)], capture_output=True, text=True, timeout=60)
+    assert r.returncode == 0, (r.stdout, r.stderr[-500:])
+    a, b, none, used, freed, has_rdv = r.stdout.split()
+    assert (int(a), int(b), none, int(used), has_rdv) == (0, 256, "1", 128 + 256, "1"), r.stdout
+    assert int(freed) in (0, 1)
