@@ -150,3 +150,30 @@ def test_reference_host_programs_with_a_thread_per_pe(stub_env, name, npes):
     env = dict(stub_env, ROCSHMEM_EMU_NPES=str(npes), ROCSHMEM_HEAP_SIZE=str(64 << 20))
     r = subprocess.run([prog], env=env, capture_output=True, text=True, timeout=60)
     assert r.returncode == 0, (name, npes, r.stdout[-600:], r.stderr[-600:])
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU; asked for more it says so and exits."""
+    r = subprocess.run([sys.executable, os.path.join(os.path.dirname(HERE), "bench.py"), "--gpus", "2"],
+                       capture_output=True, text=True, timeout=60)
+    assert r.returncode != 0 and "one GPU" in r.stderr
+
+
+def test_bench_two_process_leg_runs_to_completion(stub_env):
+    """The plumbing of bench.py's optional leg between two processes (bring-up
+    with a 1.9 GiB heap per process, three rotating 256 MiB buffer pairs, the
+    order of the meetings between the timing PE and the checking PE, the
+    record it prints).  Under the stand-in no kernel runs, so the figures mean
+    nothing and the check passes vacuously; what is tested is that both
+    processes get through and that the record parses."""
+    import json
+    bench = os.path.join(os.path.dirname(HERE), "bench.py")
+    status, outs = launch.run(2, [sys.executable, bench, "--process-leg", "--steps", "2", "--warmup", "1"],
+                              timeout=240, env=stub_env, capture=True)
+    assert status == 0, [o[-800:] for o in outs]
+    text = "\n".join(outs)
+    rec = [ln for ln in text.splitlines() if ln.startswith("PROCESS_LEG ")]
+    assert len(rec) == 1 and "PROCESS_LEG_VERIFIED 1" in text
+    fields = json.loads(rec[0][len("PROCESS_LEG "):])
+    assert set(fields) == {"putmem_wg_nostore_gbs", "getmem_wg_nostore_gbs", "putmem_wg_default_ctx_gbs",
+                           "host_putmem_gbs"}
