@@ -99,13 +99,23 @@ SOS_NOT_AS_PROCESSES = {
 SOS_TWO_PROCESSES_ONLY = {"put_ctx_mbw_mr"}  # says so itself
 
 
+# Every program runs as 2 processes; as 8 processes, the ones that cannot run
+# as PE threads (this mode is their only run with more than one PE) and the
+# collective ones.  ROCSHMEM_TEST_FULL_PROCESS_MATRIX=1 runs everything at both
+# sizes and the whole functional matrix as processes (about 100 s more).
+FULL_PROCESS_MATRIX = os.environ.get("ROCSHMEM_TEST_FULL_PROCESS_MATRIX", "0") not in ("", "0")
+SOS_EIGHT_PROCESSES = set(SOS_NOT_AS_PE_THREADS) | {
+    "barrier", "bcast", "broadcast_active_set", "big_reduction", "max_reduction", "reduce_active_set",
+    "reduce_in_place", "shmem_team_reduce", "shmem_team_b2b_collectives", "circular_shift", "atomic_inc"}
+
+
 def sos_process_cases():
     cases = []
     for name in sos_programs():
         if name in SOS_NOT_AS_PROCESSES:
             continue
         cases.append((name, 2))
-        if name not in SOS_TWO_PROCESSES_ONLY:
+        if name not in SOS_TWO_PROCESSES_ONLY and (FULL_PROCESS_MATRIX or name in SOS_EIGHT_PROCESSES):
             cases.append((name, 8))
     return cases
 
@@ -220,16 +230,34 @@ def test_reference_functional_driver(rt, name, number, wgs, threads, max_size):
 PROCESS_RUN_SPIN_LIMIT = str(40_000_000)
 
 
+def functional_process_cases():
+    """One row of the matrix per tester (the cheapest one: a bounded message
+    size where the script has one), all pingpong rows; the whole matrix with
+    ROCSHMEM_TEST_FULL_PROCESS_MATRIX=1.  The whole matrix always runs with
+    the ranks as PE threads, above."""
+    if FULL_PROCESS_MATRIX:
+        return functional_cases()
+    best = {}
+    for c in functional_cases():
+        cost = (c[4] if c[4] is not None else 0, c[2] * c[3])
+        if c[0] == "pingpong":
+            best[(c[0], c[2])] = (cost, c)
+        elif c[0] not in best or cost < best[c[0]][0]:
+            best[c[0]] = (cost, c)
+    keep = {id(v[1]) for v in best.values()}
+    return [c for c in functional_cases() if id(c) in keep]
+
+
 @pytest.mark.skipif(not functional_cases(),
                     reason="oracle/_ref/functional is built where the reference tree exists")
-@pytest.mark.parametrize("name,number,wgs,threads,max_size", functional_cases(),
-                         ids=["%s-w%d-z%d-%s" % (c[0], c[2], c[3], c[4]) for c in functional_cases()])
+@pytest.mark.parametrize("name,number,wgs,threads,max_size", functional_process_cases(),
+                         ids=["%s-w%d-z%d-%s" % (c[0], c[2], c[3], c[4]) for c in functional_process_cases()])
 def test_reference_functional_driver_with_a_process_per_pe(rt, name, number, wgs, threads, max_size):
-    """The same driver and matrix with the 2 ranks as 2 processes, the way the
-    reference's script runs it (mpirun -np 2): every put, get, atomic and
-    signal issued inside a kernel lands in the other process's heap through
-    its HIP IPC mapping, and the device-side barriers and collectives of the
-    testers meet across the process boundary."""
+    """The same driver with the 2 ranks as 2 processes, the way the reference's
+    script runs it (mpirun -np 2): every put, get, atomic and signal issued
+    inside a kernel lands in the other process's heap through its HIP IPC
+    mapping, and the device-side barriers and collectives of the testers meet
+    across the process boundary."""
     from rocshmem_amd import launch
     rt.down()
     env = dict(os.environ, ROCSHMEM_EMU_SPIN_LIMIT=PROCESS_RUN_SPIN_LIMIT,
